@@ -1,0 +1,241 @@
+"""Lattice multi-head attention module on the HIP operator path.
+
+Drop-in for ``CrystalformerMultiheadAttentionCUDA``
+(models/indexed_lattice_multi_head_attention_cuda.py:790-1016): same
+constructor, parameter names/shapes (``gauss_scale``, ``atten_scale``,
+``q/k/v_proj_weight``, ``in_proj_bias``, ``out_proj``, ``lattice_pos_weights``,
+``pe_dist_proj``), initialisation order and ``forward`` signature.  Only the
+real-space domain (and ``"no"``) is served; the dense projections stay on
+torch / rocBLAS.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor
+from torch.nn import Module, Parameter
+from torch.nn.init import constant_, normal_, xavier_uniform_
+
+from . import global_config as config
+from .hip_funcs import (FusedDotProductAttentionCUDA, RealPeriodicEncodingFuncCUDA,
+                        RealPeriodicEncodingWithProjFuncCUDA)
+from .params import LatticeformerParams
+
+ATOM_NUM = 98
+
+
+def make_positive_func(spec: str):
+    """rho(x, lower_bound) for the Gaussian widths
+    (models/indexed_lattice_multi_head_attention_cuda.py:675-692)."""
+    beta = float(spec.split("=")[1]) if "=" in spec else 1.0
+    if spec == "abs":
+        return lambda x, lb: (1 - lb) * x.abs() + lb
+    if spec.startswith("softplus"):
+        return lambda x, lb: F.softplus(x + 1 / beta * math.log(math.exp(beta * (1 - lb)) - 1), beta=beta) + lb
+    if spec.startswith("exp"):
+        return lambda x, lb: (1.0 - lb) * torch.exp(x * (beta / (1.0 - lb))) + lb
+    if spec.startswith("elu"):
+        return lambda x, lb: (1.0 - lb) * F.elu(x * (beta / (1.0 - lb))) + 1.0
+    if spec.startswith("sigmoid"):
+        return lambda x, lb: (1 / lb - lb) * torch.sigmoid(x * (beta * (1 + lb) / (1.0 - lb)) + math.log(lb)) + lb
+    raise NotImplementedError(f"Unknown positive_func: {spec}")
+
+
+def gaussian_exponents(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, gauss_scale: Tensor,
+                       params: LatticeformerParams, training: bool) -> Tensor:
+    """a[i,h] = -rho(normalised alpha) / (2 r0^2), alpha from the un-scaled
+    per-head query (models/indexed_lattice_multi_head_attention_cuda.py:636-722)."""
+    n, h, d = q.shape
+    if params.gauss_state.startswith("q"):
+        alpha = q.reshape(n, h, 1, d) @ lattice_pos_weights.reshape(h, d, 1)
+    elif params.gauss_state == "1":
+        alpha = torch.ones_like(q).reshape(n, h, 1, d) @ lattice_pos_weights.reshape(h, d, 1)
+    else:
+        alpha = F.linear(query, lattice_pos_weights)
+    alpha = alpha.view(n, h)
+    if params.normalize_gauss:
+        stored = bool(gauss_scale[0] > 0)
+        if stored:
+            scale, shift = gauss_scale[0], gauss_scale[1]
+        else:
+            scale = torch.reciprocal(alpha.detach().std())
+            shift = -alpha.detach().mean()
+        alpha = (alpha + shift) * scale
+        if training and not stored:   # stored once, in the first training step
+            with torch.no_grad():
+                gauss_scale[0] = scale
+                gauss_scale[1] = shift
+    rho = make_positive_func(params.positive_func)(alpha, params.gauss_lb_real)
+    return rho * (-0.5 * params.scale_real ** -2)
+
+
+def conditional_projection(proj: Tensor, onehot: Tensor, edges: Tensor, mode: str) -> Tensor:
+    """Species-conditioned projection, one matrix per edge
+    (models/indexed_lattice_multi_head_attention_cuda.py:612-626)."""
+    W = onehot @ proj.reshape(proj.shape[0], -1)
+    if mode in ("i", "I"):
+        W = W[edges[0]]
+    elif mode in ("j", "J"):
+        W = W[edges[1]]
+    elif mode in ("ij", "IJ"):
+        W = (W[edges[0]] + W[edges[1]]) * 0.5
+    else:
+        raise NotImplementedError(mode)
+    return W.reshape(-1, proj.shape[1], proj.shape[2], proj.shape[3])
+
+
+def loop_attention(q: Tensor, k: Tensor, v: Tensor, batch: Tensor, edges: Tensor,
+                   bias: Optional[Tensor], values: Optional[Tensor]) -> Tensor:
+    """Per-crystal softmax/aggregate with stock torch ops: what the reference
+    runs when its numerics switch is below 2
+    (models/indexed_lattice_multi_head_attention_cuda.py:231-306, mode 0)."""
+    logits = (q[edges[0]] * k[edges[1]]).sum(dim=-1)
+    if bias is not None:
+        logits = logits + bias
+    sizes = torch.zeros(int(batch.max().item()) + 1, dtype=torch.long, device=q.device)
+    sizes.scatter_add_(0, batch, torch.ones_like(batch))
+    sizes = sizes.tolist()
+    esz = [s * s for s in sizes]
+    prob = torch.cat([F.softmax(a.view(s, s, -1), dim=1).view(s * s, -1)
+                      for a, s in zip(torch.split_with_sizes(logits, esz), sizes)])
+    msg = v[edges[1]] if values is None else v[edges[1]] + values
+    msg = prob[..., None] * msg
+    return torch.cat([m.view((s, s) + m.shape[1:]).sum(dim=1)
+                      for m, s in zip(torch.split_with_sizes(msg, esz), sizes)])
+
+
+class CrystalformerMultiheadAttentionCUDA(Module):
+    def __init__(self, embed_dim, num_heads, dropout=0., bias=True, kdim=None, vdim=None,
+                 params: LatticeformerParams = LatticeformerParams(), device=None, dtype=None) -> None:
+        kw = {"device": device, "dtype": dtype}
+        super().__init__()
+        if params.domain not in ("real", "no"):
+            raise NotImplementedError(
+                f"domain={params.domain!r}: only the real-space encoding has HIP kernels")
+        self.embed_dim = embed_dim
+        self.kdim = kdim * num_heads if kdim is not None and kdim > 0 else embed_dim
+        self.vdim = vdim * num_heads if vdim is not None and vdim > 0 else embed_dim
+        self.params = params
+        self.gauss_scale = Parameter(torch.zeros(2, **kw), requires_grad=False)
+        self.atten_scale = Parameter(torch.zeros(1, **kw), requires_grad=False)
+        self.num_heads = num_heads
+        self.dropout = dropout
+        self.head_dim = embed_dim // num_heads
+        assert self.head_dim * num_heads == embed_dim, "embed_dim must be divisible by num_heads"
+
+        self.q_proj_weight = Parameter(torch.empty((self.kdim, embed_dim), **kw))
+        self.k_proj_weight = Parameter(torch.empty((self.kdim, embed_dim), **kw))
+        self.v_proj_weight = Parameter(torch.empty((self.vdim, embed_dim), **kw))
+        if bias:
+            self.in_proj_bias = Parameter(torch.empty(self.kdim * 2 + self.vdim, **kw))
+        else:
+            self.register_parameter("in_proj_bias", None)
+        self.out_proj = torch.nn.Linear(self.vdim, embed_dim, bias=bias, **kw)
+
+        if params.domain == "no":
+            self.lattice_pos_weights = None
+        elif params.gauss_state.startswith("q") or params.gauss_state == "1":
+            self.lattice_pos_weights = Parameter(torch.empty((self.kdim), **kw))
+        elif params.gauss_state.startswith("x") and params.gauss_state != "x-xn":
+            self.lattice_pos_weights = Parameter(torch.empty((num_heads, embed_dim), **kw))
+        else:
+            raise NotImplementedError(f"gauss_state={params.gauss_state!r}")
+
+        heads = num_heads if params.value_pe_headed else 1
+        cond = 1 if params.value_pe_condproj == "no" else ATOM_NUM
+        self.pe_dist_proj = None
+        self.pe_wave_proj = None
+        if params.domain == "real" and params.value_pe_dist_real > 0:
+            self.pe_dist_proj = Parameter(torch.empty(cond, heads, self.head_dim, params.value_pe_dist_real, **kw))
+        if params.domain == "real" and params.value_pe_wave_real > 0:
+            raise NotImplementedError("value_pe_wave_real > 0 has no HIP kernel")
+        self._reset_parameters()
+
+    def _reset_parameters(self):
+        xavier_uniform_(self.q_proj_weight)
+        xavier_uniform_(self.k_proj_weight)
+        xavier_uniform_(self.v_proj_weight)
+        xavier_uniform_(self.out_proj.weight)
+        if self.in_proj_bias is not None:
+            constant_(self.in_proj_bias, 0.)
+            constant_(self.out_proj.bias, 0.)
+        if self.lattice_pos_weights is not None:
+            gs = self.params.gauss_state
+            if gs in ("q", "q-headdim", "1"):
+                normal_(self.lattice_pos_weights, 0., (self.kdim // self.num_heads) ** -0.5)
+            elif gs == "q-kdim":
+                normal_(self.lattice_pos_weights, 0., self.kdim ** -0.5)
+            elif gs in ("x", "x-norm"):
+                normal_(self.lattice_pos_weights, 0., self.embed_dim ** -0.5)
+            elif gs == "x-xavier":
+                xavier_uniform_(self.lattice_pos_weights)
+            else:
+                raise NotImplementedError(gs)
+        if self.pe_dist_proj is not None:
+            with torch.no_grad():
+                for idx, W in enumerate(self.pe_dist_proj):
+                    if idx != 0 and self.params.value_pe_condproj in ("I", "J", "IJ"):
+                        W.set_(self.pe_dist_proj[0])
+                    else:
+                        flat = W.view(-1, W.shape[-1])
+                        xavier_uniform_(flat, flat.shape[1] ** -0.5)
+
+    def forward(self, query: Tensor, key: Tensor, value: Tensor, batch_q: Tensor, batch_kv: Tensor,
+                edges: Tensor, points: Tensor, dist2_min: Optional[Tensor], tvecs: Tensor,
+                kr_base: Optional[Tensor] = None, rvecs: Optional[Tensor] = None,
+                vcell: Optional[Tensor] = None, onehot: Optional[Tensor] = None,
+                need_weights: bool = True) -> Tuple[Tensor, Optional[Tensor]]:
+        P = self.params
+        H = self.num_heads
+        n = query.shape[0]
+        kd, vd = self.kdim, self.vdim
+        b_q = b_k = b_v = None
+        if self.in_proj_bias is not None:
+            b_q, b_k, b_v = self.in_proj_bias.split([kd, kd, vd])
+        q = F.linear(query, self.q_proj_weight, b_q).contiguous().view(n, H, kd // H)
+        k = F.linear(key, self.k_proj_weight, b_k).contiguous().view(key.shape[0], H, kd // H)
+        v = F.linear(value, self.v_proj_weight, b_v).contiguous().view(value.shape[0], H, vd // H)
+
+        bias = values = None
+        if P.domain == "real":
+            proj = self.pe_dist_proj
+            if proj is not None and P.value_pe_condproj != "no":
+                proj = conditional_projection(proj, onehot, edges, P.value_pe_condproj)
+            a = gaussian_exponents(q, query, self.lattice_pos_weights, self.gauss_scale, P, self.training)
+            dist_max = P.value_pe_dist_max
+            if dist_max < 0:
+                dist_max = (-dist_max) * P.scale_real
+            adaptive = ()
+            if P.adaptive_cutoff_sigma < 0:
+                adaptive = (torch.norm(rvecs, 2, dim=-1), P.adaptive_cutoff_sigma)
+            elif P.adaptive_cutoff_sigma > 0:
+                adaptive = (torch.norm(rvecs, 2, dim=-1),
+                            P.scale_real * P.gauss_lb_real ** (-0.5) * P.adaptive_cutoff_sigma)
+            if proj is not None and not P.value_pe_headed:
+                proj = proj.expand(proj.shape[0], H, proj.shape[2], proj.shape[3])
+            enc = RealPeriodicEncodingWithProjFuncCUDA if P.use_low_memory else RealPeriodicEncodingFuncCUDA
+            out = enc.apply(a, points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real, dist_max,
+                            P.value_pe_width_scale, proj, *adaptive)
+            bias = out[0]
+            values = out[1] if len(out) >= 2 else None
+
+        if P.norm_func_mode != 0:
+            raise NotImplementedError("norm_func_mode != 0 is not served by the HIP path")
+        if self.training and self.dropout > 0.0:
+            raise NotImplementedError("attention dropout is not served by the HIP path")
+        qs = q / math.sqrt(q.shape[-1])
+        if config.REPRODUCIBLITY_STATE >= 2 and batch_q is batch_kv:
+            attn = FusedDotProductAttentionCUDA.apply(qs, k, v, bias, values, batch_q, edges)
+        else:
+            attn = loop_attention(qs, k, v, batch_q, edges, bias, values)
+        attn = attn.contiguous().view(n, vd)
+        attn = F.linear(attn, self.out_proj.weight, self.out_proj.bias)
+        if need_weights:
+            raise NotImplementedError("need_weights=True: attention weights are not returned by the fused path")
+        return attn, values
+
+
+CrystalformerMultiheadAttentionHIP = CrystalformerMultiheadAttentionCUDA

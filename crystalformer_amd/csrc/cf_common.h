@@ -1,0 +1,115 @@
+// Shared helpers for the gfx950 kernels: error reporting for the C ABI,
+// wave64 reductions and the hardware transcendental wrappers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/crystalformer_hip.h"
+
+namespace cf {
+
+constexpr int WAVE = 64;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+// The reference kernels divide by 2.0 * CUDART_PI_F (the float constant widened
+// to double); the translation half-widths are only bit-exact with that value.
+constexpr float PI_F = 3.141592654f;
+constexpr int MAX_RANGE = 64;
+
+// ---- error reporting -------------------------------------------------------
+void set_error(const char *fmt, ...);
+int hip_failed(hipError_t err, const char *what);
+int device_cu_count();
+
+#define CF_REQUIRE(cond, code, ...)            \
+    do {                                       \
+        if (!(cond)) {                         \
+            cf::set_error(__VA_ARGS__);        \
+            return (code);                     \
+        }                                      \
+    } while (0)
+
+#define CF_CHECK_LAUNCH(what)                                        \
+    do {                                                             \
+        hipError_t _e = hipGetLastError();                           \
+        if (_e != hipSuccess) return cf::hip_failed(_e, (what));     \
+    } while (0)
+
+// ---- device helpers --------------------------------------------------------
+#if defined(__HIPCC__)
+
+__device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float log2_hw(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float sqrt_hw(float x) { return __builtin_amdgcn_sqrtf(x); }
+
+__device__ __forceinline__ float readlane_f(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float wave_min(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, WAVE));
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
+    return v;
+}
+
+__device__ __forceinline__ int wave_max_i(int v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, WAVE));
+    return v;
+}
+
+// Orders this wave's earlier LDS/global writes before its later reads.
+__device__ __forceinline__ void wave_mem_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// Translation half-width along one axis: ceil((cutoff+0.01f)*rvl / (2*pi)),
+// float product, double quotient.
+__device__ __forceinline__ int range_axis(float cutoff, float rvl, int minimum_range)
+{
+    float num = (cutoff + 0.01f) * rvl;
+    double q = ceil((double)num / (2.0 * (double)PI_F));
+    int r = (q >= 0.0 && q <= (double)MAX_RANGE) ? (int)q : (q > (double)MAX_RANGE ? MAX_RANGE : 0);
+    if (q != q) r = MAX_RANGE;  // NaN exponent: bounded loop, result is NaN anyway
+    return max(r, minimum_range);
+}
+
+// Half-widths for one (atom, head).  cutoff == 0 selects the fixed cube.
+__device__ __forceinline__ void range_rule(float a, float cutoff, const float *rvl,
+                                           int lattice_range, int minimum_range,
+                                           int &R1, int &R2, int &R3)
+{
+    R1 = R2 = R3 = lattice_range;
+    if (cutoff != 0.0f) {
+        if (cutoff < 0.0f) cutoff = sqrtf(-0.5f / a) * (-cutoff);
+        R1 = range_axis(cutoff, rvl[0], minimum_range);
+        R2 = range_axis(cutoff, rvl[1], minimum_range);
+        R3 = range_axis(cutoff, rvl[2], minimum_range);
+    }
+}
+
+#endif  // __HIPCC__
+
+}  // namespace cf

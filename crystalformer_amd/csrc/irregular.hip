@@ -1,0 +1,109 @@
+// Irregular (per-crystal) helpers for gfx950: mean pooling over the atoms of
+// each crystal, its backward, and the dense intra-crystal edge list.
+#include "cf_common.h"
+
+namespace {
+
+using namespace cf;
+
+// One thread per (crystal, channel); atoms are summed in blocks of 8 combined
+// by a fixed tree, blocks accumulated in order: deterministic and close to
+// pairwise accuracy for crystals of any size.
+__global__ void irregular_mean_fwd_kernel(const float *src, const int64_t *start_n, int64_t B, int64_t D,
+                                          float *dst)
+{
+    int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid >= B * D) return;
+    const int64_t n = tid / D, k = tid - n * D;
+    const int64_t r0 = start_n[n], r1 = start_n[n + 1];
+    const float *col = src + k;
+    float total = 0.f;
+    int64_t r = r0;
+    for (; r + 8 <= r1; r += 8) {
+        float t0 = col[r * D] + col[(r + 1) * D];
+        float t1 = col[(r + 2) * D] + col[(r + 3) * D];
+        float t2 = col[(r + 4) * D] + col[(r + 5) * D];
+        float t3 = col[(r + 6) * D] + col[(r + 7) * D];
+        total += (t0 + t1) + (t2 + t3);
+    }
+    float tail = 0.f;
+    for (; r < r1; r++) tail += col[r * D];
+    total += tail;
+    dst[tid] = total / (float)(r1 - r0);
+}
+
+__global__ void irregular_mean_bwd_kernel(const float *go, const int64_t *batch_i, const int64_t *start_n,
+                                          int64_t N, int64_t D, float *gx)
+{
+    int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid >= N * D) return;
+    const int64_t i = tid / D, k = tid - i * D;
+    const int64_t n = batch_i[i];
+    gx[tid] = go[n * D + k] / (float)(start_n[n + 1] - start_n[n]);
+}
+
+// One thread per edge: locate the crystal by bisection over edge_start_n, then
+// (i,j) = divmod(local edge, atoms in crystal).
+__global__ void edge_index_kernel(const int64_t *atom_start, const int64_t *edge_start, int64_t B, int64_t E,
+                                  const float *pos, int64_t *edges, float *rpos)
+{
+    int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= E) return;
+    int64_t lo = 0, hi = B;   // invariant: edge_start[lo] <= e < edge_start[hi]
+    while (hi - lo > 1) {
+        int64_t mid = (lo + hi) >> 1;
+        if (edge_start[mid] <= e) lo = mid; else hi = mid;
+    }
+    const int64_t a0 = atom_start[lo];
+    const int64_t n = atom_start[lo + 1] - a0;
+    const int64_t local = e - edge_start[lo];
+    const int64_t il = local / n;
+    const int64_t i = a0 + il, j = a0 + (local - il * n);
+    edges[e] = i;
+    edges[E + e] = j;
+    if (pos && rpos) {
+        rpos[e * 3 + 0] = pos[j * 3 + 0] - pos[i * 3 + 0];
+        rpos[e * 3 + 1] = pos[j * 3 + 1] - pos[i * 3 + 1];
+        rpos[e * 3 + 2] = pos[j * 3 + 2] - pos[i * 3 + 2];
+    }
+}
+
+}  // namespace
+
+extern "C" int cf_irregular_mean_fwd(const float *src, const int64_t *start_n, int64_t B, int64_t D,
+                                     float *dst, void *stream)
+{
+    CF_REQUIRE(B >= 0 && D >= 0, CF_ERR_INVALID_ARGUMENT, "cf_irregular_mean_fwd: negative size");
+    if (B * D == 0) return CF_OK;
+    CF_REQUIRE(src && start_n && dst, CF_ERR_INVALID_ARGUMENT, "cf_irregular_mean_fwd: null pointer");
+    int64_t total = B * D;
+    irregular_mean_fwd_kernel<<<(int)((total + 127) / 128), 128, 0, (hipStream_t)stream>>>(src, start_n, B, D, dst);
+    CF_CHECK_LAUNCH("cf_irregular_mean_fwd");
+    return CF_OK;
+}
+
+extern "C" int cf_irregular_mean_bwd(const float *go, const int64_t *batch_i, const int64_t *start_n,
+                                     int64_t N, int64_t D, float *gx, void *stream)
+{
+    CF_REQUIRE(N >= 0 && D >= 0, CF_ERR_INVALID_ARGUMENT, "cf_irregular_mean_bwd: negative size");
+    if (N * D == 0) return CF_OK;
+    CF_REQUIRE(go && batch_i && start_n && gx, CF_ERR_INVALID_ARGUMENT, "cf_irregular_mean_bwd: null pointer");
+    int64_t total = N * D;
+    irregular_mean_bwd_kernel<<<(int)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(go, batch_i, start_n,
+                                                                                          N, D, gx);
+    CF_CHECK_LAUNCH("cf_irregular_mean_bwd");
+    return CF_OK;
+}
+
+extern "C" int cf_edge_index(const int64_t *atom_start_n, const int64_t *edge_start_n, int64_t B, int64_t E,
+                             const float *pos, int64_t *edge_ij_e, float *rpos_ij_e, void *stream)
+{
+    CF_REQUIRE(B >= 0 && E >= 0, CF_ERR_INVALID_ARGUMENT, "cf_edge_index: negative size");
+    if (E == 0) return CF_OK;
+    CF_REQUIRE(B > 0 && atom_start_n && edge_start_n && edge_ij_e, CF_ERR_INVALID_ARGUMENT,
+               "cf_edge_index: null pointer or no crystals");
+    edge_index_kernel<<<(int)((E + 255) / 256), 256, 0, (hipStream_t)stream>>>(atom_start_n, edge_start_n, B, E,
+                                                                              pos, edge_ij_e, rpos_ij_e);
+    CF_CHECK_LAUNCH("cf_edge_index");
+    return CF_OK;
+}

@@ -1,0 +1,171 @@
+"""Encoder stack on the HIP operator path.
+
+Drop-in for ``CrystalformerEncoderCUDA`` / ``CrystalformerEncoderLayerCUDA``
+(models/indexed_latticeformer_encoder.py:620-890): same constructor arguments,
+sub-module names (``layers.N.self_attn``, ``linear1``, ``linear2``), t-fixup
+scaling and ``forward(src, pos, batch, trans, sizes, onehot=None)``.
+The geometry prologue (edge list, p_j - p_i, reciprocal vectors) runs on the
+device.
+"""
+from __future__ import annotations
+
+import math
+from typing import Callable, Optional, Union
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor
+from torch.nn import Dropout, Identity, LayerNorm, Linear, Module, ModuleList
+from torch.nn.init import constant_, xavier_uniform_
+
+from . import ops
+from .attention import CrystalformerMultiheadAttentionCUDA
+from .hip_funcs import compile_kernels
+from .params import LatticeformerParams
+
+
+def det_3x3(m: Tensor) -> Tensor:
+    """Cofactor expansion, term order of models/indexed_latticeformer_encoder.py:34-44."""
+    return (m[:, 0, 0] * m[:, 1, 1] * m[:, 2, 2] + m[:, 0, 1] * m[:, 1, 2] * m[:, 2, 0]
+            + m[:, 0, 2] * m[:, 1, 0] * m[:, 2, 1] - m[:, 0, 2] * m[:, 1, 1] * m[:, 2, 0]
+            - m[:, 0, 0] * m[:, 1, 2] * m[:, 2, 1] - m[:, 0, 1] * m[:, 1, 0] * m[:, 2, 2])
+
+
+def compute_lattice_distances_for_cuda(pos: Tensor, batch: Tensor, trans_vec: Tensor, sizes, lattice_range,
+                                       cutoff_radius=0, output_real=False, output_reci=False):
+    """Geometry prologue of the kernel path
+    (models/indexed_latticeformer_encoder.py:183-253): relative positions per
+    edge, reciprocal vectors, cell volume and the dense edge list.  Returns
+    ``(pos_ij, dist2_min, kr_base, recip_vec, vcell, edges)``; ``dist2_min`` and
+    ``kr_base`` are None (the kernels find the minimum themselves; there is no
+    reciprocal-space kernel here)."""
+    if output_reci:
+        raise NotImplementedError("reciprocal-space outputs are not served by the HIP path")
+    if sizes is None:
+        sizes = torch.zeros(trans_vec.shape[0], dtype=torch.long, device=pos.device)
+        sizes.scatter_add_(0, batch, torch.ones_like(batch))
+    if not torch.is_tensor(sizes):
+        sizes = torch.tensor(sizes, dtype=torch.long, device=pos.device)
+    sizes = sizes.to(device=pos.device, dtype=torch.long)
+    vcell = det_3x3(trans_vec).contiguous()
+    recip_vec = (torch.stack([
+        torch.cross(trans_vec[:, 1], trans_vec[:, 2], dim=1),
+        torch.cross(trans_vec[:, 2], trans_vec[:, 0], dim=1),
+        torch.cross(trans_vec[:, 0], trans_vec[:, 1], dim=1),
+    ], dim=1) * (2.0 * math.pi / vcell[:, None, None])).contiguous()
+    edges, pos_ij = ops.edge_index(sizes, pos.contiguous())
+    return pos_ij, None, None, recip_vec, vcell, edges
+
+
+def _activation(name):
+    if callable(name):
+        return name
+    if name == "relu":
+        return F.relu
+    if name == "gelu":
+        return F.gelu
+    raise RuntimeError(f"activation should be relu/gelu, not {name}")
+
+
+class CrystalformerEncoderLayerCUDA(Module):
+    def __init__(self, d_model: int, nhead: int, dim_feedforward: int = 2048, dropout: float = 0.1,
+                 activation: Union[str, Callable[[Tensor], Tensor]] = F.relu, layer_norm_eps: float = 1e-5,
+                 norm_first: bool = False, no_layer_norm=False, params=LatticeformerParams(),
+                 k_dim=0, v_dim=0, device=None, dtype=None) -> None:
+        super().__init__()
+        assert params.domain in ("real",), "only the real-space domain is served"
+        self.domain = params.domain
+        self.self_attn = CrystalformerMultiheadAttentionCUDA(d_model, nhead, dropout=dropout, kdim=k_dim,
+                                                             vdim=v_dim, params=params)
+        self.linear1 = Linear(d_model, dim_feedforward)
+        self.dropout = Dropout(dropout) if dropout > 0 else Identity()
+        self.linear2 = Linear(dim_feedforward, d_model)
+        self.norm_first = norm_first
+        self.norm1 = LayerNorm(d_model, eps=layer_norm_eps) if not no_layer_norm else Identity()
+        self.norm2 = LayerNorm(d_model, eps=layer_norm_eps) if not no_layer_norm else Identity()
+        self.dropout1 = Dropout(dropout) if dropout > 0 else Identity()
+        self.dropout2 = Dropout(dropout) if dropout > 0 else Identity()
+        self.activation = _activation(activation)
+        self._reset_parameters()
+
+    def _reset_parameters(self):
+        xavier_uniform_(self.linear1.weight)
+        xavier_uniform_(self.linear2.weight)
+        constant_(self.linear1.bias, 0)
+        constant_(self.linear2.bias, 0)
+
+    def fixup_initialization(self, num_layers: int) -> None:
+        """t-fixup: scale the value path by 0.67 L^-1/4
+        (models/indexed_latticeformer_encoder.py:832-850)."""
+        factor = 0.67 * num_layers ** (-1.0 / 4.0)
+        scaled = ("linear1.weight", "linear2.weight", "self_attn.out_proj.weight", "self_attn.v_proj_weight")
+        with torch.no_grad():
+            for name, param in self.named_parameters():
+                if name in scaled:
+                    param.copy_(factor * param)
+
+    def forward(self, src: Tensor, batch: Tensor, edges: Tensor, pos_ij: Tensor = None,
+                dist2_min: Tensor = None, trans: Tensor = None, kr_base: Tensor = None,
+                rvecs: Tensor = None, vcell: Tensor = None, onehot: Tensor = None) -> Tensor:
+        assert pos_ij is not None and trans is not None
+        x = src
+        if self.norm_first:
+            x = x + self._sa_block(self.norm1(x), batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot)
+            x = x + self._ff_block(self.norm2(x))
+        else:
+            x = self.norm1(x + self._sa_block(x, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot))
+            x = self.norm2(x + self._ff_block(x))
+        return x
+
+    def _sa_block(self, x, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot):
+        x = self.self_attn(x, x, x, batch, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell,
+                           onehot, need_weights=False)[0]
+        return self.dropout1(x)
+
+    def _ff_block(self, x: Tensor) -> Tensor:
+        return self.dropout2(self.linear2(self.dropout(self.activation(self.linear1(x)))))
+
+
+class CrystalformerEncoderCUDA(Module):
+    def __init__(self, d_model: int = 512, nhead: int = 8, num_encoder_layers: int = 6,
+                 dim_feedforward: int = 2048, dropout: float = 0.1,
+                 activation: Union[str, Callable[[Tensor], Tensor]] = F.relu, layer_norm_eps: float = 1e-5,
+                 norm_first: bool = False, t_fixup_init=False, no_layer_norm=False,
+                 lattice_params: LatticeformerParams = LatticeformerParams(), k_dim=0, v_dim=0,
+                 device=None, dtype=None) -> None:
+        super().__init__()
+        self.lattice_params = lattice_params
+        self.layers = ModuleList([
+            CrystalformerEncoderLayerCUDA(d_model, nhead, dim_feedforward, dropout, activation, layer_norm_eps,
+                                          norm_first, no_layer_norm,
+                                          params=lattice_params.getLayerParameters(i), k_dim=k_dim, v_dim=v_dim)
+            for i in range(num_encoder_layers)])
+        if t_fixup_init:
+            for layer in self.layers:
+                layer.fixup_initialization(num_encoder_layers)
+        self.num_layers = num_encoder_layers
+        self.norm = LayerNorm(d_model, eps=layer_norm_eps) if not no_layer_norm else None
+        self.d_model = d_model
+        self.nhead = nhead
+        compile_kernels(lattice_params.lattice_range, nhead, k_dim if k_dim > 0 else d_model // nhead,
+                        lattice_params.value_pe_dist_real, v_dim if v_dim > 0 else d_model // nhead,
+                        lattice_params.minimum_range)
+
+    def forward(self, src: Tensor, pos: Tensor, batch: Tensor, trans: Tensor, sizes: Tensor,
+                onehot: Optional[Tensor] = None) -> Tensor:
+        if src.size(-1) != self.d_model:
+            raise RuntimeError("the feature number of src and tgt must be equal to d_model")
+        batch = batch - batch[0]
+        P = self.lattice_params
+        pos_ij, dist2_min, kr_base, rvecs, vcell, edges = compute_lattice_distances_for_cuda(
+            pos, batch, trans, sizes, P.lattice_range, -1, output_real=True, output_reci=False)
+        output = src
+        for layer in self.layers:
+            output = layer(output, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot)
+        if self.norm is not None:
+            output = self.norm(output)
+        return output
+
+
+CrystalformerEncoderHIP = CrystalformerEncoderCUDA
+CrystalformerEncoderLayerHIP = CrystalformerEncoderLayerCUDA

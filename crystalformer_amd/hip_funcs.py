@@ -1,0 +1,238 @@
+"""Operator boundary: the ``torch.autograd.Function`` classes and the compile hook
+that Crystalformer's attention module imports from its ``cuda_funcs`` package
+(models/cuda_funcs/__init__.py:12-27), served by the gfx950 kernels.
+
+Same class names, positional arguments, outputs and gradients as the
+reference, so ``from crystalformer_amd.hip_funcs import *`` can stand in for
+``from .cuda_funcs import *``:
+
+* ``RealPeriodicEncodingFuncCUDA``          models/cuda_funcs/real_space_enc.py:17-247
+* ``RealPeriodicEncodingWithProjFuncCUDA``  models/cuda_funcs/real_space_enc_proj.py:18-178
+* ``FusedDotProductAttentionCUDA``          models/cuda_funcs/fused_dpa.py:17-208
+* ``IrregularMeanCUDA``                     models/cuda_funcs/irregular_mean.py:19-69
+* ``compile_kernels`` / ``KernelManager``   models/cuda_funcs/kernel_manager.py:24-134
+
+Differences by design: kernels are built ahead of time, so ``compile_kernels``
+only records the constants the reference substitutes into its sources
+(lattice range, minimum range) and checks that the library supports the shapes;
+there is no limit on atoms per crystal; ``gW`` comes back already reduced to the
+shape of ``W``.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from . import lib as _lib
+from . import ops
+
+__all__ = [
+    "KernelManager", "compile_kernels", "CUPY_AVAILABLE", "HIP_AVAILABLE",
+    "RealPeriodicEncodingFuncCUDA", "RealPeriodicEncodingWithProjFuncCUDA",
+    "FusedDotProductAttentionCUDA", "IrregularMeanCUDA", "compute_minimum_distance",
+]
+
+
+def _hip_available() -> bool:
+    return _lib.is_built() and torch.cuda.is_available()
+
+
+HIP_AVAILABLE = _hip_available()
+# The reference gates its kernel path on this flag (models/latticeformer.py:139-143).
+CUPY_AVAILABLE = HIP_AVAILABLE
+
+
+class KernelManager:
+    """Constants shared by all launches, set by ``compile_kernels``."""
+    LATTICE_RANGE: int = 2
+    MINIMUM_RANGE: int = 0
+    HEAD_NUM: int = 8
+    K_HEAD_DIM: int = 16
+    V_HEAD_DIM: int = 16
+    VPE_DIM: int = 64
+    # kept for code that reads them; the kernels have no per-crystal size limit
+    MAX_SYSTEM_SIZE: int = 1 << 30
+    MAX_SYSTEM_SIZE_POW2: int = 1 << 30
+    RUNNING_SUM_LEN: int = 8
+    compiled: bool = False
+
+
+def compile_kernels(lattice_range: int, head_num: int, key_head_dim: int, value_pe_dim: int,
+                    value_head_dim: int, set_minimum_range: bool) -> None:
+    """Record the launch constants (models/cuda_funcs/kernel_manager.py:109-134)
+    and verify that the prebuilt library covers the requested shapes."""
+    if head_num not in (1, 2, 4, 8, 16):
+        raise _lib.CrystalformerHipError(f"head_num={head_num} not supported (1,2,4,8,16)")
+    if not 0 <= value_pe_dim <= 128:
+        raise _lib.CrystalformerHipError(f"value_pe_dim={value_pe_dim} outside 0..128")
+    if value_pe_dim > 0 and not 1 <= value_head_dim <= 64:
+        raise _lib.CrystalformerHipError(f"value_head_dim={value_head_dim} outside 1..64")
+    KernelManager.LATTICE_RANGE = int(lattice_range)
+    KernelManager.MINIMUM_RANGE = int(lattice_range) if set_minimum_range else 0
+    KernelManager.HEAD_NUM = int(head_num)
+    KernelManager.K_HEAD_DIM = int(key_head_dim)
+    KernelManager.V_HEAD_DIM = int(value_head_dim)
+    KernelManager.VPE_DIM = int(value_pe_dim)
+    _lib.load()
+    KernelManager.compiled = True
+
+
+def _w_leading(W_k: Optional[Tensor]) -> int:
+    if W_k is None:
+        return 0
+    assert W_k.dim() in (3, 4)
+    return 1 if W_k.dim() == 3 else W_k.shape[0]
+
+
+def _enc_backward_tail(ga_ik, gW_k, has_adaptive_args: bool):
+    base = (ga_ik, None, None, None, None, None, None, None, None, gW_k)
+    return base + (None, None) if has_adaptive_args else base
+
+
+class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
+    """z[e,h] = log sum_n exp(a[i,h] |r_ij + n.L|^2) and the Gaussian value
+    encoding with the per-head projection fused into the kernel.
+
+    Returns ``(z_ek,)`` when ``K <= 0`` else ``(z_ek, v_ekd)`` with v of shape
+    (E,H,D) when ``W_k`` is given and (E,H,K) otherwise.
+    """
+
+    @staticmethod
+    def forward(ctx, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale,
+                W_k, rvlen_n=None, cutoff_radius=None):
+        a_ik = a_ik.contiguous().detach()
+        rpos_ij_e = rpos_ij_e.contiguous()
+        tvecs_n = tvecs_n.contiguous()
+        batch_i = batch_i.contiguous()
+        edge_ij_e = edge_ij_e.contiguous()
+        W_k = W_k.detach().contiguous() if W_k is not None else None
+        z_ek, v_ekd = ops.real_enc_fwd(
+            a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, W_k, rvlen_n,
+            cutoff_radius, KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
+        ctx.save_for_backward(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, W_k, z_ek)
+        ctx.K, ctx.dist_max, ctx.wscale, ctx.cutoff_radius = K, dist_max, wscale, cutoff_radius
+        ctx.ranges = (KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
+        ctx.adaptive_args = rvlen_n is not None
+        if K <= 0:
+            return (z_ek,)
+        return z_ek, v_ekd
+
+    @staticmethod
+    def backward(ctx, gz_ek, gv_ekd=None):
+        a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, W_k, z_ek = ctx.saved_tensors
+        e_start_i = ops.edge_row_offsets(edge_ij_e, a_ik.shape[0])
+        gz = gz_ek.detach().contiguous() if gz_ek is not None else None
+        gv = gv_ekd.detach().contiguous() if gv_ekd is not None else None
+        ga_ik, gW_k = ops.real_enc_bwd(
+            a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz, gv, ctx.K, ctx.dist_max,
+            ctx.wscale, W_k, rvlen_n, ctx.cutoff_radius, ctx.ranges[0], ctx.ranges[1],
+            want_gW=W_k is not None and ctx.needs_input_grad[9])
+        return _enc_backward_tail(ga_ik, gW_k, ctx.adaptive_args)
+
+
+class RealPeriodicEncodingFuncCUDA(torch.autograd.Function):
+    """Same encoding with the projection left to a batched matmul: the kernel
+    produces the (E,H,K) Gaussian averages and ``W_k`` is applied outside, as in
+    the reference's unfused path (``W_k`` leading size 1 or E)."""
+
+    @staticmethod
+    def forward(ctx, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale,
+                W_k, rvlen_n=None, cutoff_radius=None):
+        a_ik = a_ik.contiguous().detach()
+        rpos_ij_e = rpos_ij_e.contiguous()
+        tvecs_n = tvecs_n.contiguous()
+        batch_i = batch_i.contiguous()
+        edge_ij_e = edge_ij_e.contiguous()
+        E = edge_ij_e.shape[1]
+        z_ek, s_ekk = ops.real_enc_fwd(
+            a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, None, rvlen_n,
+            cutoff_radius, KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
+        v_out = s_ekk
+        if W_k is not None and K > 0:
+            W_k = W_k.detach().contiguous()
+            assert _w_leading(W_k) in (E, 1)
+            v_out = (W_k @ s_ekk[..., None]).reshape(E, a_ik.shape[1], -1)
+        else:
+            W_k = None
+        ctx.save_for_backward(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, W_k, z_ek,
+                              s_ekk if W_k is not None else None)
+        ctx.K, ctx.dist_max, ctx.wscale, ctx.cutoff_radius = K, dist_max, wscale, cutoff_radius
+        ctx.ranges = (KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
+        ctx.adaptive_args = rvlen_n is not None
+        if K <= 0:
+            return (z_ek,)
+        return z_ek, v_out
+
+    @staticmethod
+    def backward(ctx, gz_ek, gv_ekd=None):
+        a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, W_k, z_ek, s_ekk = ctx.saved_tensors
+        e_start_i = ops.edge_row_offsets(edge_ij_e, a_ik.shape[0])
+        gW_k = None
+        gv = gv_ekd.detach().contiguous() if gv_ekd is not None else None
+        if W_k is not None and gv is not None:
+            # dv/dW: outer product per edge; autograd sums it down to W's shape
+            gW_k = gv[..., :, None] * s_ekk[..., None, :]
+            gv = (W_k.transpose(-1, -2) @ gv[..., None]).squeeze(-1).contiguous()
+        gz = gz_ek.detach().contiguous() if gz_ek is not None else None
+        ga_ik, _ = ops.real_enc_bwd(
+            a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz, gv, ctx.K, ctx.dist_max,
+            ctx.wscale, None, rvlen_n, ctx.cutoff_radius, ctx.ranges[0], ctx.ranges[1], want_gW=False)
+        return _enc_backward_tail(ga_ik, gW_k, ctx.adaptive_args)
+
+
+class FusedDotProductAttentionCUDA(torch.autograd.Function):
+    """out[i,h,:] = sum_j softmax_j(q_i.k_j + a_ij) (v_j + b_ij) over each atom's
+    edge row.  ``que_ihk`` is expected pre-divided by sqrt(head dim)."""
+
+    @staticmethod
+    def forward(ctx, que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e):
+        que_ihk = que_ihk.contiguous().detach()
+        key_ihk = key_ihk.contiguous().detach()
+        val_ihk = val_ihk.contiguous().detach()
+        aij_eh = aij_eh.contiguous().detach() if aij_eh is not None else None
+        bij_ehk = bij_ehk.contiguous().detach() if bij_ehk is not None else None
+        batch_i = batch_i.contiguous()
+        edge_ij_e = edge_ij_e.contiguous()
+        e_start_i = ops.edge_row_offsets(edge_ij_e, que_ihk.shape[0])
+        output, prob_eh = ops.fused_dpa_fwd(que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, edge_ij_e, e_start_i)
+        ctx.save_for_backward(que_ihk, key_ihk, val_ihk, bij_ehk, batch_i, edge_ij_e, e_start_i, prob_eh,
+                              output)
+        ctx.has_aij = aij_eh is not None
+        return output
+
+    @staticmethod
+    def backward(ctx, go_ihk):
+        que_ihk, key_ihk, val_ihk, bij_ehk, batch_i, edge_ij_e, e_start_i, prob_eh, output = ctx.saved_tensors
+        gque, gkey, gval, gaij, gbij = ops.fused_dpa_bwd(
+            que_ihk, key_ihk, val_ihk, bij_ehk, batch_i, edge_ij_e, e_start_i, prob_eh, output,
+            go_ihk.contiguous().detach())
+        return gque, gkey, gval, (gaij if ctx.has_aij else None), gbij, None, None
+
+
+class IrregularMeanCUDA(torch.autograd.Function):
+    """Per-crystal mean over atoms with a fixed summation order."""
+
+    @staticmethod
+    def forward(ctx, x_ik: Tensor, batch_i: Tensor, sizes: Optional[Tensor]):
+        if sizes is None:
+            B = int(batch_i.max().item()) + 1
+            sizes = torch.zeros(B, dtype=torch.long, device=x_ik.device)
+            sizes.scatter_add_(0, batch_i, torch.ones_like(batch_i))
+        start_n = torch.constant_pad_nd(torch.cumsum(sizes, 0), (1, 0)).contiguous()
+        o_nk = ops.irregular_mean_fwd(x_ik.contiguous().detach(), start_n)
+        ctx.save_for_backward(batch_i.contiguous(), start_n)
+        return o_nk
+
+    @staticmethod
+    def backward(ctx, go_nk):
+        batch_i, start_n = ctx.saved_tensors
+        return ops.irregular_mean_bwd(go_nk.contiguous(), batch_i, start_n), None, None
+
+
+def compute_minimum_distance(rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, cutoff_radius):
+    """Per-edge minimum squared distance (models/cuda_funcs/minimum_distance.py:18-41)."""
+    assert cutoff_radius >= 0
+    return ops.minimum_distance(rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, cutoff_radius,
+                                KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)

@@ -1,0 +1,271 @@
+"""Thin functional wrappers over the C ABI: validate, allocate outputs with
+torch, pass raw device pointers and torch's current stream.  No autograd here
+(see ``hip_funcs.py``) and no CPU fallback.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor
+
+from . import lib as _lib
+from .lib import check, ptr, require_device, stream_handle
+
+
+def _f32(t: Optional[Tensor], name: str) -> Optional[Tensor]:
+    if t is None:
+        return None
+    if t.dtype != torch.float32:
+        raise _lib.CrystalformerHipError(f"{name} must be float32, got {t.dtype}")
+    return t.contiguous()
+
+
+def _i64(t: Optional[Tensor], name: str) -> Optional[Tensor]:
+    if t is None:
+        return None
+    if t.dtype != torch.int64:
+        raise _lib.CrystalformerHipError(f"{name} must be int64, got {t.dtype}")
+    return t.contiguous()
+
+
+def _w_shape(W_k: Optional[Tensor], H: int, K: int) -> Tuple[int, int]:
+    if W_k is None:
+        return 0, 0
+    if W_k.dim() not in (3, 4):
+        raise _lib.CrystalformerHipError("W_k must be (H,D,K) or (W_num,H,D,K)")
+    if W_k.shape[-3] != H or W_k.shape[-1] != K:
+        raise _lib.CrystalformerHipError(
+            f"W_k shape {tuple(W_k.shape)} does not match H={H}, K={K}")
+    return (1 if W_k.dim() == 3 else W_k.shape[0]), W_k.shape[-2]
+
+
+def edge_row_offsets(edge_ij_e: Tensor, num_atoms: int) -> Tensor:
+    """CSR offsets of each source atom's edges, (N+1) int64, computed on the
+    device without a host sync (models/cuda_funcs/fused_dpa.py:24-26)."""
+    start = torch.zeros(num_atoms + 1, dtype=torch.int64, device=edge_ij_e.device)
+    start.scatter_add_(0, edge_ij_e[0] + 1, torch.ones_like(edge_ij_e[0]))
+    return start.cumsum(0)
+
+
+def crystal_offsets(batch_i: Tensor, num_slots: Optional[int] = None) -> Tuple[Tensor, Tensor]:
+    """(atom_start, edge_start): leading-zero cumulative sums of the crystal
+    sizes and of their squares.  ``num_slots`` defaults to the atom count, an
+    upper bound on the number of crystals that needs no host sync."""
+    slots = batch_i.numel() if num_slots is None else num_slots
+    sizes = torch.zeros(slots, dtype=torch.int64, device=batch_i.device)
+    sizes.scatter_add_(0, batch_i, torch.ones_like(batch_i))
+    atom_start = F.pad(sizes.cumsum(0), (1, 0))
+    edge_start = F.pad((sizes * sizes).cumsum(0), (1, 0))
+    return atom_start, edge_start
+
+
+def real_enc_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor,
+                 K: int, dist_max: float, wscale: float, W_k: Optional[Tensor] = None,
+                 rvlen_n: Optional[Tensor] = None, cutoff_radius: Optional[float] = None,
+                 lattice_range: int = 2, minimum_range: int = 0) -> Tuple[Tensor, Optional[Tensor]]:
+    dev = require_device(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, W_k, rvlen_n)
+    a_ik, rpos_ij_e, tvecs_n = _f32(a_ik, "a_ik"), _f32(rpos_ij_e, "rpos_ij_e"), _f32(tvecs_n, "tvecs_n")
+    batch_i, edge_ij_e = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e")
+    W_k, rvlen_n = _f32(W_k, "W_k"), _f32(rvlen_n, "rvlen_n")
+    N, H = a_ik.shape
+    E = edge_ij_e.shape[1]
+    B = tvecs_n.shape[0]
+    if rpos_ij_e.shape != (E, 3) or batch_i.shape != (N,) or tvecs_n.shape[1:] != (3, 3):
+        raise _lib.CrystalformerHipError("real_enc_fwd: inconsistent input shapes")
+    if rvlen_n is not None and rvlen_n.shape != (B, 3):
+        raise _lib.CrystalformerHipError("real_enc_fwd: rvlen_n must be (B,3)")
+    K = int(K)
+    W_num, D = _w_shape(W_k, H, K) if K > 0 else (0, 0)
+    cutoff = 0.0 if (cutoff_radius is None or rvlen_n is None) else float(cutoff_radius)
+    z = torch.empty((E, H), dtype=torch.float32, device=dev)
+    v = None
+    if K > 0:
+        v = torch.empty((E, H, D if W_k is not None else K), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_real_enc_fwd(
+            ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), N, H, E, B, K, D,
+            float(dist_max), float(wscale), ptr(W_k if K > 0 else None), W_num,
+            ptr(rvlen_n), cutoff, int(lattice_range), int(minimum_range), ptr(z), ptr(v),
+            stream_handle(dev))
+    check(rc, "cf_real_enc_fwd")
+    return z, v
+
+
+def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor,
+                 e_start_i: Tensor, z_ek: Tensor, gz_ek: Optional[Tensor], gv_ekd: Optional[Tensor],
+                 K: int, dist_max: float, wscale: float, W_k: Optional[Tensor] = None,
+                 rvlen_n: Optional[Tensor] = None, cutoff_radius: Optional[float] = None,
+                 lattice_range: int = 2, minimum_range: int = 0,
+                 want_gW: bool = True) -> Tuple[Tensor, Optional[Tensor]]:
+    dev = require_device(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd,
+                         W_k, rvlen_n)
+    a_ik, rpos_ij_e, tvecs_n = _f32(a_ik, "a_ik"), _f32(rpos_ij_e, "rpos_ij_e"), _f32(tvecs_n, "tvecs_n")
+    batch_i, edge_ij_e, e_start_i = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e"), \
+        _i64(e_start_i, "e_start_i")
+    z_ek, gz_ek, gv_ekd = _f32(z_ek, "z_ek"), _f32(gz_ek, "gz_ek"), _f32(gv_ekd, "gv_ekd")
+    W_k, rvlen_n = _f32(W_k, "W_k"), _f32(rvlen_n, "rvlen_n")
+    N, H = a_ik.shape
+    E = edge_ij_e.shape[1]
+    B = tvecs_n.shape[0]
+    K = int(K)
+    W_num, D = _w_shape(W_k, H, K) if K > 0 else (0, 0)
+    if e_start_i.shape != (N + 1,) or z_ek.shape != (E, H):
+        raise _lib.CrystalformerHipError("real_enc_bwd: inconsistent input shapes")
+    if gz_ek is not None and gz_ek.shape != (E, H):
+        raise _lib.CrystalformerHipError("real_enc_bwd: gz_ek must be (E,H)")
+    if gv_ekd is not None and K > 0:
+        last = D if W_k is not None else K
+        if gv_ekd.shape != (E, H, last):
+            raise _lib.CrystalformerHipError(f"real_enc_bwd: gv_ekd must be (E,H,{last})")
+    cutoff = 0.0 if (cutoff_radius is None or rvlen_n is None) else float(cutoff_radius)
+    want_gW = bool(want_gW and W_k is not None and K > 0)
+    ga = torch.empty_like(a_ik)
+    gW = torch.empty_like(W_k) if want_gW else None
+    L = _lib.load()
+    ws_bytes = int(L.cf_real_enc_bwd_workspace(N, H, E, K, D, W_num, 1 if want_gW else 0))
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = L.cf_real_enc_bwd(
+            ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i),
+            ptr(z_ek), ptr(gz_ek), ptr(gv_ekd if K > 0 else None), N, H, E, B, K, D, float(dist_max),
+            float(wscale), ptr(W_k if K > 0 else None), W_num, ptr(rvlen_n), cutoff, int(lattice_range),
+            int(minimum_range), ptr(ws), ws_bytes, ptr(ga), ptr(gW), stream_handle(dev))
+    check(rc, "cf_real_enc_bwd")
+    return ga, gW
+
+
+def translation_ranges(a_ik: Tensor, rvlen_n: Optional[Tensor], batch_i: Tensor,
+                       cutoff_radius: float, lattice_range: int, minimum_range: int) -> Tensor:
+    dev = require_device(a_ik, rvlen_n, batch_i)
+    a_ik, rvlen_n, batch_i = _f32(a_ik, "a_ik"), _f32(rvlen_n, "rvlen_n"), _i64(batch_i, "batch_i")
+    N, H = a_ik.shape
+    out = torch.empty((N, H, 3), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_translation_ranges(ptr(a_ik), ptr(rvlen_n), ptr(batch_i), N, H,
+                                               float(cutoff_radius), int(lattice_range),
+                                               int(minimum_range), ptr(out), stream_handle(dev))
+    check(rc, "cf_translation_ranges")
+    return out
+
+
+def fused_dpa_fwd(que: Tensor, key: Tensor, val: Tensor, aij_eh: Optional[Tensor],
+                  bij_ehd: Optional[Tensor], edge_ij_e: Tensor,
+                  e_start_i: Tensor) -> Tuple[Tensor, Tensor]:
+    dev = require_device(que, key, val, aij_eh, bij_ehd, edge_ij_e, e_start_i)
+    que, key, val = _f32(que, "que"), _f32(key, "key"), _f32(val, "val")
+    aij_eh, bij_ehd = _f32(aij_eh, "aij_eh"), _f32(bij_ehd, "bij_ehd")
+    edge_ij_e, e_start_i = _i64(edge_ij_e, "edge_ij_e"), _i64(e_start_i, "e_start_i")
+    N, H, Dk = que.shape
+    Dv = val.shape[-1]
+    E = edge_ij_e.shape[1]
+    if key.shape != (key.shape[0], H, Dk) or val.shape[:2] != (key.shape[0], H):
+        raise _lib.CrystalformerHipError("fused_dpa_fwd: inconsistent q/k/v shapes")
+    if key.shape[0] != N:
+        raise _lib.CrystalformerHipError("fused_dpa_fwd: self-attention only (same atoms for q and k/v)")
+    if aij_eh is not None and aij_eh.shape != (E, H):
+        raise _lib.CrystalformerHipError("fused_dpa_fwd: aij_eh must be (E,H)")
+    if bij_ehd is not None and bij_ehd.shape != (E, H, Dv):
+        raise _lib.CrystalformerHipError("fused_dpa_fwd: bij_ehd must be (E,H,Dv)")
+    if e_start_i.shape != (N + 1,):
+        raise _lib.CrystalformerHipError("fused_dpa_fwd: e_start_i must be (N+1,)")
+    prob = torch.empty((E, H), dtype=torch.float32, device=dev)
+    out = torch.empty((N, H, Dv), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_fused_dpa_fwd(ptr(que), ptr(key), ptr(val), ptr(aij_eh), ptr(bij_ehd),
+                                          ptr(edge_ij_e), ptr(e_start_i), N, H, E, Dk, Dv, ptr(prob),
+                                          ptr(out), stream_handle(dev))
+    check(rc, "cf_fused_dpa_fwd")
+    return out, prob
+
+
+def fused_dpa_bwd(que: Tensor, key: Tensor, val: Tensor, bij_ehd: Optional[Tensor], batch_i: Tensor,
+                  edge_ij_e: Tensor, e_start_i: Tensor, prob_eh: Tensor, out: Tensor, gout: Tensor,
+                  atom_start_n: Optional[Tensor] = None, edge_start_n: Optional[Tensor] = None):
+    dev = require_device(que, key, val, bij_ehd, batch_i, edge_ij_e, e_start_i, prob_eh, out, gout)
+    que, key, val, bij_ehd = _f32(que, "que"), _f32(key, "key"), _f32(val, "val"), _f32(bij_ehd, "bij_ehd")
+    prob_eh, out, gout = _f32(prob_eh, "prob_eh"), _f32(out, "out"), _f32(gout, "gout")
+    batch_i, edge_ij_e, e_start_i = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e"), \
+        _i64(e_start_i, "e_start_i")
+    N, H, Dk = que.shape
+    Dv = val.shape[-1]
+    E = edge_ij_e.shape[1]
+    if atom_start_n is None or edge_start_n is None:
+        atom_start_n, edge_start_n = crystal_offsets(batch_i)
+    atom_start_n, edge_start_n = _i64(atom_start_n, "atom_start_n"), _i64(edge_start_n, "edge_start_n")
+    B = atom_start_n.numel() - 1
+    gq, gk, gv = torch.empty_like(que), torch.empty_like(key), torch.empty_like(val)
+    ga = torch.empty((E, H), dtype=torch.float32, device=dev)
+    gb = torch.empty((E, H, Dv), dtype=torch.float32, device=dev) if bij_ehd is not None else None
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_fused_dpa_bwd(
+            ptr(que), ptr(key), ptr(val), ptr(bij_ehd), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i),
+            ptr(atom_start_n), ptr(edge_start_n), N, H, E, B, Dk, Dv, ptr(prob_eh), ptr(out), ptr(gout),
+            ptr(gq), ptr(gk), ptr(gv), ptr(ga), ptr(gb), stream_handle(dev))
+    check(rc, "cf_fused_dpa_bwd")
+    return gq, gk, gv, ga, gb
+
+
+def irregular_mean_fwd(x_ik: Tensor, start_n: Tensor) -> Tensor:
+    dev = require_device(x_ik, start_n)
+    x_ik, start_n = _f32(x_ik, "x_ik"), _i64(start_n, "start_n")
+    N = x_ik.shape[0]
+    B = start_n.numel() - 1
+    D = x_ik.numel() // N if N > 0 else 0
+    out = torch.empty((B,) + tuple(x_ik.shape[1:]), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_irregular_mean_fwd(ptr(x_ik), ptr(start_n), B, D, ptr(out), stream_handle(dev))
+    check(rc, "cf_irregular_mean_fwd")
+    return out
+
+
+def irregular_mean_bwd(go_nk: Tensor, batch_i: Tensor, start_n: Tensor) -> Tensor:
+    dev = require_device(go_nk, batch_i, start_n)
+    go_nk, batch_i, start_n = _f32(go_nk, "go_nk"), _i64(batch_i, "batch_i"), _i64(start_n, "start_n")
+    N = batch_i.numel()
+    D = go_nk.numel() // go_nk.shape[0] if go_nk.shape[0] > 0 else 0
+    gx = torch.empty((N,) + tuple(go_nk.shape[1:]), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_irregular_mean_bwd(ptr(go_nk), ptr(batch_i), ptr(start_n), N, D, ptr(gx),
+                                               stream_handle(dev))
+    check(rc, "cf_irregular_mean_bwd")
+    return gx
+
+
+def minimum_distance(rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor,
+                     rvlen_n: Optional[Tensor], cutoff_radius: float, lattice_range: int = 2,
+                     minimum_range: int = 0) -> Tensor:
+    dev = require_device(rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n)
+    rpos_ij_e, tvecs_n, rvlen_n = _f32(rpos_ij_e, "rpos_ij_e"), _f32(tvecs_n, "tvecs_n"), \
+        _f32(rvlen_n, "rvlen_n")
+    batch_i, edge_ij_e = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e")
+    E = edge_ij_e.shape[1]
+    out = torch.empty((E,), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_minimum_distance(ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), E,
+                                             ptr(rvlen_n), float(cutoff_radius), int(lattice_range),
+                                             int(minimum_range), ptr(out), stream_handle(dev))
+    check(rc, "cf_minimum_distance")
+    return out
+
+
+def edge_index(sizes: Tensor, pos: Optional[Tensor] = None,
+               num_edges: Optional[int] = None) -> Tuple[Tensor, Optional[Tensor]]:
+    """Dense intra-crystal edge list (2,E) and, with ``pos``, p_j - p_i (E,3),
+    built on the device.  ``num_edges`` (sum of sizes^2) avoids a host sync when
+    the caller already knows it."""
+    dev = require_device(sizes, pos)
+    sizes = _i64(sizes, "sizes")
+    pos = _f32(pos, "pos")
+    B = sizes.numel()
+    atom_start = F.pad(sizes.cumsum(0), (1, 0))
+    edge_start = F.pad((sizes * sizes).cumsum(0), (1, 0))
+    E = int(edge_start[-1].item()) if num_edges is None else int(num_edges)
+    edges = torch.empty((2, E), dtype=torch.int64, device=dev)
+    rpos = torch.empty((E, 3), dtype=torch.float32, device=dev) if pos is not None else None
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_edge_index(ptr(atom_start), ptr(edge_start), B, E, ptr(pos), ptr(edges),
+                                       ptr(rpos), stream_handle(dev))
+    check(rc, "cf_edge_index")
+    return edges, rpos

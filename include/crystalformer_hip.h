@@ -1,0 +1,199 @@
+/*
+ * C ABI of libcrystalformer_hip.so — MI355X (gfx950) kernels for Crystalformer's
+ * infinitely connected attention.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller, float32 data,
+ *     int64 indices, contiguous row-major tensors;
+ *   - `stream` is a hipStream_t (NULL = the default stream); calls are
+ *     asynchronous on it and never synchronise the device;
+ *   - the library allocates nothing unless a function's comment says so;
+ *   - return value 0 = success, negative = error (cf_last_error() gives the
+ *     text for the calling thread); no kernel is launched on error;
+ *   - optional pointers are documented as "nullable".
+ *
+ * Each entry point replaces one kernel launch of the reference's CuPy layer
+ * (file:line under the reference checkout given per function).
+ */
+#ifndef CRYSTALFORMER_HIP_H
+#define CRYSTALFORMER_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CF_OK 0
+#define CF_ERR_INVALID_ARGUMENT (-1)
+#define CF_ERR_UNSUPPORTED (-2)
+#define CF_ERR_HIP (-3)
+
+/* Library version, major*10000 + minor*100 + patch. */
+int cf_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *cf_last_error(void);
+
+/* Largest translation half-width a rule-B box may take per axis; larger
+ * values (or NaN exponents) are clamped so that a kernel always terminates. */
+int cf_max_translation_range(void);
+
+/*
+ * Real-space periodic encoding, forward.
+ * Replaces the launches of real_enc_fwd / real_enc_proj_fwd
+ * (models/cuda_funcs/real_space_enc.py:96-113,
+ *  models/cuda_funcs/real_space_enc_proj.py:70-88;
+ *  kernels models/kernels/real_enc_fwd.cu, real_enc_proj_fwd.cu).
+ *
+ *   a_ik      (N,H)    negative Gaussian exponents
+ *   rpos_ij_e (E,3)    p_j - p_i per edge
+ *   tvecs_n   (B,3,3)  lattice rows per crystal
+ *   batch_i   (N)      crystal of each atom
+ *   edge_ij_e (2,E)    edges (source i, target j)
+ *   K         number of Gaussian value-PE bins, 0 = bias only (1..128 supported)
+ *   D         rows of W (head dim of the projected value PE); ignored if W_k NULL
+ *   W_k       nullable, (W_num,H,D,K); W_num in {1,E,N}
+ *   rvlen_n   nullable, (B,3) lengths of the reciprocal lattice vectors
+ *   cutoff_radius  0: fixed cube [-lattice_range,lattice_range]^3 (rule A);
+ *                  <0: adaptive box from sqrt(-0.5/a)*|cutoff| per (atom,head);
+ *                  >0: adaptive box from that radius.  Non-zero needs rvlen_n.
+ *   minimum_range  lower bound of every adaptive half-width (0 = none)
+ * Outputs
+ *   z_ek  (E,H)                       log sum_n exp(a d^2)
+ *   v_ekd nullable if K==0; (E,H,K) when W_k is NULL, else (E,H,D)
+ */
+int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                    const int64_t *batch_i, const int64_t *edge_ij_e,
+                    int64_t N, int64_t H, int64_t E, int64_t B, int64_t K, int64_t D,
+                    double dist_max, double wscale, const float *W_k, int64_t W_num,
+                    const float *rvlen_n, double cutoff_radius, int lattice_range,
+                    int minimum_range, float *z_ek, float *v_ekd, void *stream);
+
+/*
+ * Bytes of device scratch cf_real_enc_bwd needs for the given sizes
+ * (pass want_gW != 0 when gW_k will be requested).
+ */
+int64_t cf_real_enc_bwd_workspace(int64_t N, int64_t H, int64_t E, int64_t K, int64_t D,
+                                  int64_t W_num, int want_gW);
+
+/*
+ * Real-space periodic encoding, backward wrt a_ik and W_k.
+ * Replaces the launches of real_enc_bwd / real_enc_proj_bwd
+ * (models/cuda_funcs/real_space_enc.py:222-241,
+ *  models/cuda_funcs/real_space_enc_proj.py:153-173;
+ *  kernels models/kernels/real_enc_bwd.cu, real_enc_proj_bwd.cu).
+ *
+ *   e_start_i (N+1)  CSR offsets of each source atom's edges
+ *   z_ek      (E,H)  forward output
+ *   gz_ek     (E,H)  gradient of z
+ *   gv_ekd    nullable; (E,H,K) when W_k is NULL else (E,H,D)
+ *   workspace device scratch of cf_real_enc_bwd_workspace() bytes (256-byte aligned)
+ * Outputs
+ *   ga_ik (N,H)
+ *   gW_k  nullable; (W_num,H,D,K) — already reduced to W's own shape (the
+ *         reference returns per-atom partial sums and lets autograd reduce them)
+ */
+int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                    const int64_t *batch_i, const int64_t *edge_ij_e,
+                    const int64_t *e_start_i, const float *z_ek, const float *gz_ek,
+                    const float *gv_ekd, int64_t N, int64_t H, int64_t E, int64_t B,
+                    int64_t K, int64_t D, double dist_max, double wscale,
+                    const float *W_k, int64_t W_num, const float *rvlen_n,
+                    double cutoff_radius, int lattice_range, int minimum_range,
+                    void *workspace, int64_t workspace_bytes,
+                    float *ga_ik, float *gW_k, void *stream);
+
+/*
+ * Per (atom, head) translation half-widths the encoding kernels use,
+ * R_out (N,H,3) int32.  Exposes the rule of models/kernels/real_enc_fwd.cu:58-85
+ * for bit-exact checks and work counting.
+ */
+int cf_translation_ranges(const float *a_ik, const float *rvlen_n, const int64_t *batch_i,
+                          int64_t N, int64_t H, double cutoff_radius, int lattice_range,
+                          int minimum_range, int32_t *R_out, void *stream);
+
+/*
+ * Fused edge-indexed dot-product attention, forward.
+ * Replaces the launch of fused_dpa_fwd / fused_dpa_fwd_v3
+ * (models/cuda_funcs/fused_dpa.py:40-57; kernel models/kernels/fused_dpa_fwd.cu).
+ * No limit on atoms per crystal.
+ *
+ *   que (N,H,Dk) already divided by sqrt(Dk); key (N,H,Dk); val (N,H,Dv)
+ *   aij_eh  nullable (E,H) additive logit bias
+ *   bij_ehd nullable (E,H,Dv) additive value term
+ *   edge_ij_e (2,E) sorted by source atom; e_start_i (N+1) CSR offsets
+ * Outputs
+ *   prob_eh (E,H) softmax over each source atom's edges
+ *   out     (N,H,Dv)
+ */
+int cf_fused_dpa_fwd(const float *que, const float *key, const float *val,
+                     const float *aij_eh, const float *bij_ehd, const int64_t *edge_ij_e,
+                     const int64_t *e_start_i, int64_t N, int64_t H, int64_t E,
+                     int64_t Dk, int64_t Dv, float *prob_eh, float *out, void *stream);
+
+/*
+ * Fused attention, backward.  Replaces irregular_transpose + fused_dpa_bwd +
+ * fused_dpa_bwd_q (models/cuda_funcs/fused_dpa.py:141-206; kernels
+ * models/kernels/fused_dpa_bwd.cu, fused_dpa_bwd_q.cu, irregular_transpose.cu).
+ * The edge list must be the dense per-crystal block layout produced by
+ * cf_edge_index (edge of (i,j) in a crystal of n atoms at e0 + i*n + j): the
+ * key-side sums walk a column of that block instead of transposing it.
+ *
+ *   batch_i (N); atom_start_n (B+1) first atom of each crystal;
+ *   edge_start_n (B+1) first edge of each crystal
+ *   prob_eh, out: forward outputs; gout (N,H,Dv)
+ * Outputs
+ *   gque (N,H,Dk) (gradient wrt the pre-scaled query), gkey, gval,
+ *   gaij (E,H), gbij nullable (E,H,Dv)
+ */
+int cf_fused_dpa_bwd(const float *que, const float *key, const float *val,
+                     const float *bij_ehd, const int64_t *batch_i,
+                     const int64_t *edge_ij_e, const int64_t *e_start_i,
+                     const int64_t *atom_start_n, const int64_t *edge_start_n,
+                     int64_t N, int64_t H, int64_t E, int64_t B, int64_t Dk, int64_t Dv,
+                     const float *prob_eh, const float *out, const float *gout,
+                     float *gque, float *gkey, float *gval, float *gaij, float *gbij,
+                     void *stream);
+
+/*
+ * Per-crystal mean over atoms.  Replaces the launch of irregular_mean_fwd
+ * (models/cuda_funcs/irregular_mean.py:43-54; kernel
+ * models/kernels/irregular_mean_fwd.cu).  No limit on atoms per crystal.
+ *   src (N,D); start_n (B+1) -> dst (B,D)
+ */
+int cf_irregular_mean_fwd(const float *src, const int64_t *start_n, int64_t B, int64_t D,
+                          float *dst, void *stream);
+
+/* Backward of the mean: gx[i,:] = go[batch_i[i],:] / len(batch_i[i])
+ * (models/cuda_funcs/irregular_mean.py:60-69). */
+int cf_irregular_mean_bwd(const float *go, const int64_t *batch_i, const int64_t *start_n,
+                          int64_t N, int64_t D, float *gx, void *stream);
+
+/*
+ * Per-edge minimum squared distance over the translation box.  Replaces the
+ * launch of minimum_distance (models/cuda_funcs/minimum_distance.py:30-40;
+ * kernel models/kernels/minimum_distance.cu).
+ */
+int cf_minimum_distance(const float *rpos_ij_e, const float *tvecs_n, const int64_t *batch_i,
+                        const int64_t *edge_ij_e, int64_t E, const float *rvlen_n,
+                        double cutoff_radius, int lattice_range, int minimum_range,
+                        float *dist2_min_e, void *stream);
+
+/*
+ * Dense intra-crystal edge list and relative positions on the device.
+ * Replaces the host loops of get_edge_index and the pos[j]-pos[i] gather
+ * (models/indexed_latticeformer_encoder.py:15-32, 214).
+ *   atom_start_n, edge_start_n (B+1): leading-zero cumulative sums of sizes
+ *   and sizes^2;  pos (N,3) nullable (then rpos_ij_e is not written)
+ * Outputs
+ *   edge_ij_e (2,E); rpos_ij_e nullable (E,3)
+ */
+int cf_edge_index(const int64_t *atom_start_n, const int64_t *edge_start_n, int64_t B,
+                  int64_t E, const float *pos, int64_t *edge_ij_e, float *rpos_ij_e,
+                  void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CRYSTALFORMER_HIP_H */
