@@ -165,6 +165,7 @@ void ref_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tv
                       float *ga_ik, float *gW_k)
 {
     static const float zero3[3] = {0, 0, 0};
+    (void)edge_ij_e;   /* rows are walked through e_start_i */
     const size_t Kn = (size_t)(K > 0 ? K : 1);
     double *sgv = (double *)malloc(sizeof(double) * Kn);
     double *sv = (double *)malloc(sizeof(double) * Kn);

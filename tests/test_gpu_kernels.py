@@ -1,0 +1,228 @@
+"""GPU parity tests: every HIP kernel, called through the C ABI (ctypes), against
+the CPU oracles on the same seeded inputs.  Integer outputs are compared
+bit-exactly; float32 outputs to 1e-5 relative (see tests/helpers.py)."""
+import math
+
+import pytest
+import torch
+
+from crystalformer_amd import lib, ops
+from oracle import kernel_semantics as ks
+from oracle import torch_path as tp
+from tests.helpers import Problem, assert_close, make_sized_batch, rel_err, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def enc_fwd_gpu(dev, p, K, W, cutoff, lr, mr, rvlen=True):
+    a, rpos, tv, bt, ed, Wd, rv = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, W,
+                                         p.rvlen if rvlen else None)
+    return ops.real_enc_fwd(a, rpos, tv, bt, ed, K, p.dist_max, p.wscale, Wd, rv, cutoff, lr, mr)
+
+
+def enc_fwd_ref(p, K, W, cutoff, lr, mr):
+    return ks.real_enc_fwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, K, p.dist_max, p.wscale, W, p.rvlen,
+                           cutoff, lr, mr)
+
+
+RULES = [(0.0, 2, 0), (-3.5, 2, 2), (-3.5, 1, 0), (5.0, 1, 1)]
+
+
+@pytest.mark.parametrize("cutoff,lr,mr", RULES)
+@pytest.mark.parametrize("H,K,D", [(8, 64, 16), (8, 0, 16), (4, 16, 8), (1, 7, 3), (2, 100, 4), (16, 32, 8)])
+def test_real_enc_fwd(dev, H, K, D, cutoff, lr, mr):
+    p = Problem([1, 3, 9, 2, 17], H=H, K=K, D=D, seed=21)
+    for W in ([p.W, None] if K > 0 else [None]):
+        z, v = enc_fwd_gpu(dev, p, K, W, cutoff, lr, mr)
+        z_ref, v_ref = enc_fwd_ref(p, K, W, cutoff, lr, mr)
+        assert_close(z, z_ref, "z")
+        if K > 0:
+            assert_close(v, v_ref, "v")
+        else:
+            assert v is None
+
+
+def test_real_enc_fwd_matches_torch_path_fixed_cube(dev):
+    """Against the reference's PyTorch-path semantics (dense (E,R) tensors)."""
+    p = Problem([2, 5, 1, 12], H=8, K=64, D=16, seed=22)
+    for r in (1, 2):
+        z, v = enc_fwd_gpu(dev, p, 64, p.W, 0.0, r, 0, rvlen=False)
+        z_ref, v_ref = tp.periodic_encoding(p.a, p.b.pos, p.b.batch, p.b.trans_vec, p.edges, r, 64, p.dist_max,
+                                            p.wscale, p.W)
+        assert_close(z, z_ref, "z")
+        assert_close(v, v_ref, "v")
+
+
+@pytest.mark.parametrize("mode", ["edge", "atom"])
+def test_real_enc_indexed_projection(dev, mode):
+    p = Problem([3, 4, 1], H=4, K=16, D=8, seed=23, W_mode=mode)
+    z, v = enc_fwd_gpu(dev, p, 16, p.W, -3.5, 2, 2)
+    z_ref, v_ref = enc_fwd_ref(p, 16, p.W, -3.5, 2, 2)
+    assert_close(z, z_ref, "z")
+    assert_close(v, v_ref, "v")
+    gz, gv = p.randn(p.E, 4), p.randn(p.E, 4, 8)
+    args = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv)
+    ga, gW = ops.real_enc_bwd(*args, 16, p.dist_max, p.wscale, p.W.to(dev), p.rvlen.to(dev), -3.5, 2, 2)
+    ga_ref, gW_ref = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv, 16,
+                                     p.dist_max, p.wscale, p.W, p.rvlen, -3.5, 2, 2)
+    assert_close(ga, ga_ref, "ga")
+    assert_close(gW, gW_ref, "gW")
+
+
+@pytest.mark.parametrize("cutoff,lr,mr", RULES[:3])
+@pytest.mark.parametrize("H,K,D", [(8, 64, 16), (8, 0, 16), (4, 16, 8), (2, 100, 4)])
+def test_real_enc_bwd(dev, H, K, D, cutoff, lr, mr):
+    p = Problem([1, 3, 9, 2, 14], H=H, K=K, D=D, seed=24)
+    for W in ([p.W, None] if K > 0 else [None]):
+        z_ref, v_ref = enc_fwd_ref(p, K, W, cutoff, lr, mr)
+        gz = p.randn(p.E, H)
+        gv = p.randn(*v_ref.shape) if K > 0 else None
+        args = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv)
+        ga, gW = ops.real_enc_bwd(*args, K, p.dist_max, p.wscale, None if W is None else W.to(dev),
+                                  p.rvlen.to(dev), cutoff, lr, mr)
+        ga_ref, gW_ref = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv,
+                                         K, p.dist_max, p.wscale, W, p.rvlen, cutoff, lr, mr)
+        assert_close(ga, ga_ref, "ga")
+        if W is not None:
+            assert_close(gW, gW_ref, "gW")
+        else:
+            assert gW is None
+
+
+def test_real_enc_bwd_without_value_gradient(dev):
+    p = Problem([4, 2], H=8, K=64, D=16, seed=25)
+    z_ref, _ = enc_fwd_ref(p, 64, p.W, 0.0, 2, 0)
+    gz = p.randn(p.E, 8)
+    args = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, None)
+    ga, gW = ops.real_enc_bwd(*args, 64, p.dist_max, p.wscale, p.W.to(dev), None, 0.0, 2, 0)
+    ga_ref, _ = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, None, 64,
+                                p.dist_max, p.wscale, p.W, None, 0.0, 2, 0)
+    assert_close(ga, ga_ref, "ga")
+    assert float(gW.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("cutoff,lr,mr", [(0.0, 2, 0), (-3.5, 2, 2), (-3.5, 2, 0), (4.0, 1, 0), (-1.0, 3, 1)])
+def test_translation_ranges_bit_exact(dev, cutoff, lr, mr):
+    p = Problem([5, 9, 1, 30], H=8, K=0, seed=26)
+    a = p.a * torch.logspace(-1.5, 1.0, p.N)[:, None]            # spread the exponents over decades
+    got = ops.translation_ranges(a.to(dev), p.rvlen.to(dev), p.b.batch.to(dev), cutoff, lr, mr).cpu()
+    ref = ks.translation_ranges(a, p.rvlen, p.b.batch, cutoff, lr, mr)
+    assert got.dtype == torch.int32 and torch.equal(got, ref)
+
+
+def test_empty_and_single_atom_inputs(dev):
+    # no crystals at all
+    z, v = ops.real_enc_fwd(torch.zeros(0, 8, device=dev), torch.zeros(0, 3, device=dev),
+                            torch.zeros(0, 3, 3, device=dev), torch.zeros(0, dtype=torch.long, device=dev),
+                            torch.zeros(2, 0, dtype=torch.long, device=dev), 64, 14.0, 1.0,
+                            torch.zeros(1, 8, 16, 64, device=dev))
+    assert z.shape == (0, 8) and v.shape == (0, 8, 16)
+    e, r = ops.edge_index(torch.zeros(0, dtype=torch.long, device=dev), torch.zeros(0, 3, device=dev))
+    assert e.shape == (2, 0) and r.shape == (0, 3)
+    # crystals of one atom: a single self edge with r_ij = 0
+    p = Problem([1, 1, 1], H=8, K=64, D=16, seed=27)
+    z, v = enc_fwd_gpu(dev, p, 64, p.W, 0.0, 2, 0, rvlen=False)
+    z_ref, v_ref = enc_fwd_ref(p, 64, p.W, 0.0, 2, 0)
+    assert_close(z, z_ref, "z")
+    assert_close(v, v_ref, "v")
+    assert bool((z.cpu() >= 0).all())      # the n = 0 term alone contributes exp(0) = 1
+
+
+# ------------------------------------------------------------ fused attention
+def dpa_problem(sizes, H, Dk, Dv, seed, bias=True, vals=True):
+    p = Problem(sizes, H=H, K=0, seed=seed)
+    q = p.randn(p.N, H, Dk) / math.sqrt(Dk)
+    k, v = p.randn(p.N, H, Dk), p.randn(p.N, H, Dv)
+    a = p.randn(p.E, H) * 2 if bias else None
+    b = p.randn(p.E, H, Dv) if vals else None
+    return p, q, k, v, a, b
+
+
+@pytest.mark.parametrize("bias,vals", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("H,Dk,Dv,sizes", [(8, 16, 16, [1, 5, 70, 2, 33]), (4, 8, 32, [3, 65]), (1, 5, 4, [7, 2]),
+                                           (16, 16, 16, [9, 1]), (2, 64, 64, [4])])
+def test_fused_dpa_fwd_bwd(dev, H, Dk, Dv, sizes, bias, vals):
+    p, q, k, v, a, b = dpa_problem(sizes, H, Dk, Dv, 31, bias, vals)
+    out, prob = ops.fused_dpa_fwd(*to_dev(dev, q, k, v, a, b, p.edges, p.e_start))
+    out_ref, prob_ref = ks.fused_dpa_fwd(q, k, v, a, b, p.edges, p.e_start)
+    assert_close(out, out_ref, "out")
+    assert_close(prob, prob_ref, "prob")
+    go = p.randn(p.N, H, Dv)
+    got = ops.fused_dpa_bwd(*to_dev(dev, q, k, v, b, p.b.batch, p.edges, p.e_start, prob_ref, out_ref, go))
+    ref = ks.fused_dpa_bwd(q, k, v, b, p.edges, p.e_start, prob_ref, out_ref, go)
+    for name, x, y in zip(("gq", "gk", "gv", "ga", "gb"), got, ref):
+        if y is None:
+            assert x is None
+        else:
+            assert_close(x, y, name)
+
+
+def test_fused_dpa_beyond_the_reference_size_limit(dev):
+    """The reference's kernels stop at 320 atoms per crystal; these do not."""
+    p, q, k, v, a, b = dpa_problem([444, 3], 8, 16, 16, 32)
+    out, prob = ops.fused_dpa_fwd(*to_dev(dev, q, k, v, a, b, p.edges, p.e_start))
+    out_ref, prob_ref = ks.fused_dpa_fwd(q, k, v, a, b, p.edges, p.e_start)
+    assert_close(out, out_ref, "out")
+    assert_close(prob, prob_ref, "prob")
+    go = p.randn(p.N, 8, 16)
+    got = ops.fused_dpa_bwd(*to_dev(dev, q, k, v, b, p.b.batch, p.edges, p.e_start, prob_ref, out_ref, go))
+    ref = ks.fused_dpa_bwd(q, k, v, b, p.edges, p.e_start, prob_ref, out_ref, go)
+    for name, x, y in zip(("gq", "gk", "gv", "ga", "gb"), got, ref):
+        assert_close(x, y, name)
+
+
+def test_fused_dpa_large_logits_are_stable(dev):
+    p, q, k, v, a, b = dpa_problem([20], 8, 16, 16, 33)
+    a = a * 200.0                                   # logits of +-1000: max-subtraction must hold
+    out, prob = ops.fused_dpa_fwd(*to_dev(dev, q, k, v, a, b, p.edges, p.e_start))
+    out_ref, prob_ref = ks.fused_dpa_fwd(q, k, v, a, b, p.edges, p.e_start)
+    assert_close(out, out_ref, "out")
+    assert_close(prob, prob_ref, "prob")
+
+
+# ------------------------------------------------------------ irregular ops
+@pytest.mark.parametrize("sizes,D", [([1, 5, 70, 2], 128), ([1500, 3], 7), ([2], 1)])
+def test_irregular_mean(dev, sizes, D):
+    b = make_sized_batch(sizes, seed=41)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(int(b.sizes.sum()), D, generator=g) + 3.0
+    start = tp.crystal_starts(b.sizes)
+    got = ops.irregular_mean_fwd(x.to(dev), start.to(dev))
+    assert_close(got, ks.irregular_mean(x, start), "mean")
+    assert_close(got, tp.avr_pool(x.double(), b.sizes).float(), "mean vs torch")
+    go = torch.randn(len(sizes), D, generator=g)
+    gx = ops.irregular_mean_bwd(go.to(dev), b.batch.to(dev), start.to(dev))
+    ref = (go / b.sizes.view(-1, 1).float())[b.batch]
+    assert_close(gx, ref, "mean bwd")
+
+
+@pytest.mark.parametrize("sizes", [[1], [3, 1, 4, 1, 5], [64, 1, 33], [200]])
+def test_edge_index_bit_exact(dev, sizes):
+    b = make_sized_batch(sizes, seed=42)
+    edges, rpos = ops.edge_index(b.sizes.to(dev), b.pos.to(dev))
+    ref = tp.get_edge_index(sizes)
+    assert edges.dtype == torch.int64 and torch.equal(edges.cpu(), ref)
+    assert torch.equal(rpos.cpu(), tp.relative_positions(b.pos, ref))      # one subtraction: bit-exact
+    assert torch.equal(ops.edge_row_offsets(edges, b.pos.shape[0]).cpu(), tp.edge_row_offsets(ref, b.pos.shape[0]))
+    atom_start, edge_start = ops.crystal_offsets(b.batch.to(dev))
+    B = len(sizes)
+    assert torch.equal(atom_start[:B + 1].cpu(), tp.crystal_starts(b.sizes))
+    assert torch.equal(edge_start[:B + 1].cpu(), tp.crystal_starts(b.sizes * b.sizes))
+
+
+def test_minimum_distance(dev):
+    p = Problem([3, 8, 1], H=1, K=0, seed=43)
+    for cutoff, lr, mr in [(0.0, 2, 0), (6.0, 1, 0), (2.0, 1, 2)]:
+        got = ops.minimum_distance(*to_dev(dev, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.rvlen), cutoff, lr, mr)
+        ref = ks.minimum_distance(p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.rvlen, cutoff, lr, mr)
+        assert_close(got, ref, "d2min")
+
+
+def test_errors_surface_as_exceptions(dev):
+    p = Problem([2], H=3, K=0, seed=44)           # three heads: not an instantiated width
+    with pytest.raises(lib.CrystalformerHipError, match="head count"):
+        enc_fwd_gpu(dev, p, 0, None, 0.0, 2, 0)
+    p = Problem([2], H=8, K=64, seed=44)
+    with pytest.raises(lib.CrystalformerHipError):
+        ops.real_enc_fwd(p.a.to(dev), p.rpos.to(dev).double(), p.b.trans_vec.to(dev), p.b.batch.to(dev),
+                         p.edges.to(dev), 64, 14.0, 1.0, p.W.to(dev))

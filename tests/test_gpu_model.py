@@ -1,0 +1,246 @@
+"""GPU parity of the operator boundary and of the stacked model: autograd
+Functions and the host modules on the HIP path against the CPU oracle, the
+reference-written golden vectors, and size-independent properties at the
+benchmark's full sizes."""
+import math
+import os
+import sys
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from crystalformer_amd import global_config, hip_funcs, ops
+from crystalformer_amd.latticeformer import Latticeformer, default_params
+from crystalformer_amd.synthetic import CONFIGS, make_config_batch
+from oracle import kernel_semantics as ks
+from oracle import torch_model as om
+from oracle import torch_path as tp
+from tests.helpers import Problem, assert_close, rel_err, to_dev
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+sys.path.insert(0, GOLD)
+from make_golden import small_cfg  # noqa: E402
+
+
+def ns_to(dev, ns):
+    return SimpleNamespace(**{k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in vars(ns).items()})
+
+
+# -------------------------------------------------------- autograd functions
+@pytest.mark.parametrize("fused_proj", [True, False])
+def test_encoding_function_gradients(dev, fused_proj):
+    p = Problem([3, 1, 6], H=4, K=16, D=8, seed=51)
+    hip_funcs.compile_kernels(2, 4, 8, 16, 8, False)
+    Fn = hip_funcs.RealPeriodicEncodingWithProjFuncCUDA if fused_proj else hip_funcs.RealPeriodicEncodingFuncCUDA
+    a = p.a.to(dev).requires_grad_(True)
+    W = p.W.to(dev).requires_grad_(True)
+    z, v = Fn.apply(a, p.rpos.to(dev), None, p.b.trans_vec.to(dev), p.b.batch.to(dev), p.edges.to(dev), 16,
+                    p.dist_max, p.wscale, W)
+    gz, gv = p.randn(*z.shape), p.randn(*v.shape)
+    ((z * gz.to(dev)).sum() + (v * gv.to(dev)).sum()).backward()
+    a64 = p.a.double().requires_grad_(True)
+    W64 = p.W.double().requires_grad_(True)
+    z_ref, v_ref = tp.periodic_encoding(a64, p.b.pos.double(), p.b.batch, p.b.trans_vec.double(), p.edges, 2, 16,
+                                        p.dist_max, p.wscale, W64)
+    ((z_ref * gz).sum() + (v_ref * gv).sum()).backward()
+    assert_close(z, z_ref.float(), "z")
+    assert_close(v, v_ref.float(), "v")
+    assert_close(a.grad, a64.grad.float(), "grad a")
+    assert_close(W.grad, W64.grad.float(), "grad W")
+    assert W.grad.shape == W.shape
+
+
+def test_encoding_function_bias_only_and_adaptive_signature(dev):
+    p = Problem([2, 5], H=8, K=0, seed=52)
+    hip_funcs.compile_kernels(2, 8, 16, 0, 16, True)
+    a = p.a.to(dev).requires_grad_(True)
+    out = hip_funcs.RealPeriodicEncodingWithProjFuncCUDA.apply(
+        a, p.rpos.to(dev), None, p.b.trans_vec.to(dev), p.b.batch.to(dev), p.edges.to(dev), 0, 14.0, 1.0, None,
+        p.rvlen.to(dev), -3.5)
+    assert len(out) == 1
+    gz = p.randn(p.E, 8)
+    (out[0] * gz.to(dev)).sum().backward()
+    z_ref, _ = ks.real_enc_fwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, 0, 14.0, 1.0, None, p.rvlen, -3.5, 2, 2)
+    ga_ref, _ = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, None, 0, 14.0,
+                                1.0, None, p.rvlen, -3.5, 2, 2)
+    assert_close(out[0], z_ref, "z")
+    assert_close(a.grad, ga_ref, "grad a")
+
+
+def test_fused_attention_function_gradients(dev):
+    p = Problem([4, 1, 7], H=4, K=0, seed=53)
+    D = 8
+    leaves = [p.randn(p.N, 4, D) for _ in range(3)] + [p.randn(p.E, 4), p.randn(p.E, 4, D)]
+    dl = [t.to(dev).requires_grad_(True) for t in leaves]
+    out = hip_funcs.FusedDotProductAttentionCUDA.apply(dl[0] / math.sqrt(D), dl[1], dl[2], dl[3], dl[4],
+                                                       p.b.batch.to(dev), p.edges.to(dev))
+    go = p.randn(*out.shape)
+    (out * go.to(dev)).sum().backward()
+    cl = [t.double().requires_grad_(True) for t in leaves]
+    ref, _ = tp.indexed_attention(cl[0], cl[1], cl[2], p.b.sizes, p.edges, cl[3], cl[4])
+    (ref * go).sum().backward()
+    assert_close(out, ref.float(), "out")
+    for name, x, y in zip(("q", "k", "v", "bias", "values"), dl, cl):
+        assert_close(x.grad, y.grad.float(), f"grad {name}")
+
+
+def test_irregular_mean_function(dev):
+    p = Problem([3, 9, 1], H=1, K=0, seed=54)
+    x = p.randn(p.N, 4, 5)
+    xd = x.to(dev).requires_grad_(True)
+    out = hip_funcs.IrregularMeanCUDA.apply(xd, p.b.batch.to(dev), None)       # sizes derived from batch
+    out2 = hip_funcs.IrregularMeanCUDA.apply(xd, p.b.batch.to(dev), p.b.sizes.to(dev))
+    ref = tp.avr_pool(x.double(), p.b.sizes)
+    assert_close(out, ref.float(), "mean")
+    assert torch.equal(out, out2)
+    go = p.randn(*out.shape)
+    (out * go.to(dev)).sum().backward()
+    assert_close(xd.grad, (go / p.b.sizes.view(-1, 1, 1).float())[p.b.batch], "grad x")
+
+
+# ----------------------------------------------------------- golden vectors
+@pytest.fixture(scope="module")
+def gold():
+    return torch.load(os.path.join(GOLD, "reference_small_model.pt"), weights_only=True)
+
+
+@pytest.mark.parametrize("low_memory", [True, False])
+@pytest.mark.parametrize("name,over", [("k16_r1", dict()), ("k0_r2", dict(value_pe_dist_real=0, lattice_range=2))])
+def test_model_matches_reference_golden_forward(dev, gold, name, over, low_memory):
+    """The reference's own outputs (its PyTorch path, fixed cube) reproduced by
+    the HIP path with the adaptive box switched off."""
+    cfg = small_cfg(adaptive_cutoff_sigma=0.0, use_low_memory=low_memory, **over)
+    model = Latticeformer(cfg)
+    model.load_state_dict(gold[f"{name}.state"])
+    model.to(dev).eval()
+    data = ns_to(dev, SimpleNamespace(**gold["batch"]))
+    captured = {}
+    for li, layer in enumerate(model.encoder.layers):
+        layer.self_attn.register_forward_hook(lambda m, i, o, li=li: captured.__setitem__(f"values{li}", o[1]))
+        layer.register_forward_hook(lambda m, i, o, li=li: captured.__setitem__(f"out{li}", o))
+    with torch.no_grad():
+        y = model(data)
+    assert_close(y, gold[f"{name}.eval.y"], "y")
+    for li in range(cfg.num_layers):
+        assert_close(captured[f"out{li}"], gold[f"{name}.eval.layer{li}.out"], f"layer {li} output")
+        key = f"{name}.eval.layer{li}.values"
+        if key in gold:
+            assert_close(captured[f"values{li}"], gold[key], f"layer {li} values")
+    assert float(model.encoder.layers[0].self_attn.gauss_scale.abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("name,over", [("k16_r1", dict()), ("k0_r2", dict(value_pe_dist_real=0, lattice_range=2))])
+def test_model_matches_reference_golden_training_step(dev, gold, name, over):
+    cfg = small_cfg(adaptive_cutoff_sigma=0.0, **over)
+    model = Latticeformer(cfg)
+    model.load_state_dict(gold[f"{name}.state"])
+    model.to(dev).train()
+    data = ns_to(dev, SimpleNamespace(**gold["batch"]))
+    y = model(data)
+    loss = torch.nn.functional.l1_loss(y.squeeze(-1), data.y)
+    loss.backward()
+    assert_close(y, gold[f"{name}.train.y"], "y")
+    assert abs(float(loss) - float(gold[f"{name}.train.loss"])) < 1e-6
+    params = dict(model.named_parameters())
+    for k, g in gold[f"{name}.train.grads"].items():
+        assert_close(params[k].grad, g, f"grad {k}", rtol=2e-5)
+    scales = torch.stack([l.self_attn.gauss_scale.detach() for l in model.encoder.layers])
+    assert_close(scales, gold[f"{name}.train.gauss_scale_after"], "gauss_scale")
+    model.eval()
+    with torch.no_grad():
+        assert_close(model(data), gold[f"{name}.eval2.y"], "second eval")
+
+
+def test_loop_attention_switch_matches_fused(dev, gold):
+    cfg = small_cfg(adaptive_cutoff_sigma=0.0)
+    model = Latticeformer(cfg)
+    model.load_state_dict(gold["k16_r1.state"])
+    model.to(dev).eval()
+    data = ns_to(dev, SimpleNamespace(**gold["batch"]))
+    old = global_config.REPRODUCIBLITY_STATE
+    try:
+        with torch.no_grad():
+            global_config.REPRODUCIBLITY_STATE = 3
+            y_fused = model(data)
+            global_config.REPRODUCIBLITY_STATE = 0
+            y_loop = model(data)
+    finally:
+        global_config.REPRODUCIBLITY_STATE = old
+    assert_close(y_fused, y_loop, "fused vs loop")
+    assert_close(y_loop, gold["k16_r1.eval.y"], "loop vs golden")
+
+
+# ------------------------------------------------- full-size configurations
+def build_model(name, seed=1, **over):
+    cfg = default_params(**CONFIGS[name]["model"], **over)
+    torch.manual_seed(seed)
+    return cfg, Latticeformer(cfg)
+
+
+@pytest.mark.parametrize("name", ["cfg1_simplified_b32", "cfg2_default_b128"])
+def test_full_model_forward_against_oracle(dev, name):
+    """Whole 4-block forward at the benchmark's batch, fixed cube, vs the CPU oracle."""
+    cfg, model = build_model(name, adaptive_cutoff_sigma=0.0)
+    b = make_config_batch(name)
+    P = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    cap = {}
+    with torch.no_grad():
+        y_ref = om.latticeformer_forward(P, cfg, b, capture=cap)
+    model.to(dev).eval()
+    outs = {}
+    for li, layer in enumerate(model.encoder.layers):
+        layer.register_forward_hook(lambda m, i, o, li=li: outs.__setitem__(li, o))
+    with torch.no_grad():
+        y = model(b.to(dev))
+    for li in range(cfg.num_layers):
+        assert_close(outs[li], cap[f"layer{li}.out"], f"layer {li}")
+    assert_close(y, y_ref, "model output")
+
+
+def test_full_size_properties_and_sampled_edges(dev):
+    """Config 2 and the 444-atom stress cells at full size: sampled edges
+    against the C oracle under the adaptive box, plus properties that hold at any
+    size (softmax rows sum to one, constant values pass through, equal
+    exponents give a symmetric bias, the adaptive box only adds positive terms)."""
+    for name, nsample in [("cfg2_default_b128", 300), ("cfg5_stress_b16", 60)]:
+        b = make_config_batch(name)
+        r0 = CONFIGS[name]["model"]["scale_real"][0]
+        p = Problem(b, H=8, K=64, D=16, seed=61)
+        p.dist_max = 10.0 * r0
+        p.a = p.a / (r0 * r0) * 2.0
+        dv = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.W, p.rvlen)
+        zA, vA = ops.real_enc_fwd(dv[0], dv[1], dv[2], dv[3], dv[4], 64, p.dist_max, 1.0, dv[5], None, 0.0, 2, 0)
+        zB, vB = ops.real_enc_fwd(dv[0], dv[1], dv[2], dv[3], dv[4], 64, p.dist_max, 1.0, dv[5], dv[6], -3.5, 2, 2)
+        assert bool(torch.isfinite(zB).all()) and bool(torch.isfinite(vB).all())
+        assert bool((zB >= zA - 1e-5).all())                     # box B contains cube A
+        sel = torch.randperm(p.E, generator=p.g)[:nsample].sort().values
+        sub = p.edges[:, sel]
+        for cut, lr, mr, z, v in [(0.0, 2, 0, zA, vA), (-3.5, 2, 2, zB, vB)]:
+            z_ref, v_ref = ks.real_enc_fwd(p.a, p.rpos[sel], p.b.trans_vec, p.b.batch, sub, 64, p.dist_max, 1.0, p.W,
+                                           p.rvlen, cut, lr, mr)
+            assert_close(z[sel.to(dev)], z_ref, f"{name} z")
+            assert_close(v[sel.to(dev)], v_ref, f"{name} v")
+        # equal exponents -> z(i,j) == z(j,i)
+        a_eq = torch.full_like(p.a, -0.3 / (r0 * r0))
+        zS, _ = ops.real_enc_fwd(a_eq.to(dev), dv[1], dv[2], dv[3], dv[4], 0, 1.0, 1.0, None, None, 0.0, 2, 0)
+        atom_start, edge_start = tp.crystal_starts(b.sizes), tp.crystal_starts(b.sizes * b.sizes)
+        for c in (0, len(b.sizes) // 2, len(b.sizes) - 1):
+            n = int(b.sizes[c])
+            blk = zS[int(edge_start[c]):int(edge_start[c + 1])].view(n, n, 8)
+            assert rel_err(blk, blk.transpose(0, 1)) < 1e-5
+        # attention: rows of prob sum to one; constant values pass through unchanged
+        q = p.randn(p.N, 8, 16).to(dev) / 4.0
+        k = p.randn(p.N, 8, 16).to(dev)
+        const = torch.full((p.N, 8, 16), 1.25, device=dev)
+        es = ops.edge_row_offsets(dv[4], p.N)
+        out, prob = ops.fused_dpa_fwd(q, k, const, zB, None, dv[4], es)
+        rows = torch.zeros(p.N, 8, device=dev).index_add_(0, dv[4][0], prob)
+        assert float((rows - 1).abs().max()) < 1e-5
+        assert float((out - 1.25).abs().max()) < 1e-5
+        # linear in the value term: out(v, b) - out(v, 0) == out(0, b)
+        out_vb, _ = ops.fused_dpa_fwd(q, k, const, zB, vB, dv[4], es)
+        out_0b, _ = ops.fused_dpa_fwd(q, k, torch.zeros_like(const), zB, vB, dv[4], es)
+        assert rel_err(out_vb - out, out_0b) < 1e-5
