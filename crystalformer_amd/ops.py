@@ -14,6 +14,56 @@ from . import lib as _lib
 from .lib import check, ptr, require_device, stream_handle
 
 
+# Optional kernel timing: when a list is installed, every encoding / attention
+# launch is bracketed by a pair of HIP events recorded on the launch stream and
+# (name, start, stop, info) is appended to it.
+_event_log: Optional[list] = None
+
+
+def set_event_log(log: Optional[list]) -> None:
+    global _event_log
+    _event_log = log
+
+
+# Optional work counter: when a list is installed, every encoding launch appends
+# the number of (edge, translation) pairs its kernel walks (the box of an edge is
+# the union over heads of the per-head boxes).  Costs a host sync; not for timed runs.
+_eval_counter: Optional[list] = None
+
+
+def set_eval_counter(counter: Optional[list]) -> None:
+    global _eval_counter
+    _eval_counter = counter
+
+
+def count_translation_evals(a_ik: Tensor, rvlen_n: Optional[Tensor], batch_i: Tensor, edge_ij_e: Tensor,
+                            cutoff: float, lattice_range: int, minimum_range: int) -> float:
+    E = edge_ij_e.shape[1]
+    if cutoff == 0.0 or rvlen_n is None:
+        return float(E) * (2 * lattice_range + 1) ** 3
+    R = translation_ranges(a_ik, rvlen_n, batch_i, cutoff, lattice_range, minimum_range)
+    T = (2 * R.max(dim=1).values.long() + 1).prod(dim=1).double()          # per source atom
+    return float(T[edge_ij_e[0]].sum().item())
+
+
+class _timed:
+    def __init__(self, name: str, **info):
+        self.name, self.info = name, info
+
+    def __enter__(self):
+        if _event_log is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.stop = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+        return self
+
+    def __exit__(self, *exc):
+        if _event_log is not None:
+            self.stop.record()
+            _event_log.append((self.name, self.start, self.stop, self.info))
+        return False
+
+
 def _f32(t: Optional[Tensor], name: str) -> Optional[Tensor]:
     if t is None:
         return None
@@ -83,7 +133,10 @@ def real_enc_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
     v = None
     if K > 0:
         v = torch.empty((E, H, D if W_k is not None else K), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    if _eval_counter is not None:
+        _eval_counter.append(count_translation_evals(a_ik, rvlen_n, batch_i, edge_ij_e, cutoff,
+                                                     int(lattice_range), int(minimum_range)))
+    with torch.cuda.device(dev), _timed("real_enc_fwd", E=E, H=H, K=K, D=D, proj=W_k is not None):
         rc = _lib.load().cf_real_enc_fwd(
             ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), N, H, E, B, K, D,
             float(dist_max), float(wscale), ptr(W_k if K > 0 else None), W_num,
@@ -126,7 +179,7 @@ def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
     L = _lib.load()
     ws_bytes = int(L.cf_real_enc_bwd_workspace(N, H, E, K, D, W_num, 1 if want_gW else 0))
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with torch.cuda.device(dev), _timed("real_enc_bwd", E=E, H=H, K=K, D=D, proj=W_k is not None):
         rc = L.cf_real_enc_bwd(
             ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i),
             ptr(z_ek), ptr(gz_ek), ptr(gv_ekd if K > 0 else None), N, H, E, B, K, D, float(dist_max),
@@ -172,7 +225,7 @@ def fused_dpa_fwd(que: Tensor, key: Tensor, val: Tensor, aij_eh: Optional[Tensor
         raise _lib.CrystalformerHipError("fused_dpa_fwd: e_start_i must be (N+1,)")
     prob = torch.empty((E, H), dtype=torch.float32, device=dev)
     out = torch.empty((N, H, Dv), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with torch.cuda.device(dev), _timed("fused_dpa_fwd", E=E, H=H, Dk=Dk, Dv=Dv, bij=bij_ehd is not None):
         rc = _lib.load().cf_fused_dpa_fwd(ptr(que), ptr(key), ptr(val), ptr(aij_eh), ptr(bij_ehd),
                                           ptr(edge_ij_e), ptr(e_start_i), N, H, E, Dk, Dv, ptr(prob),
                                           ptr(out), stream_handle(dev))
@@ -198,7 +251,7 @@ def fused_dpa_bwd(que: Tensor, key: Tensor, val: Tensor, bij_ehd: Optional[Tenso
     gq, gk, gv = torch.empty_like(que), torch.empty_like(key), torch.empty_like(val)
     ga = torch.empty((E, H), dtype=torch.float32, device=dev)
     gb = torch.empty((E, H, Dv), dtype=torch.float32, device=dev) if bij_ehd is not None else None
-    with torch.cuda.device(dev):
+    with torch.cuda.device(dev), _timed("fused_dpa_bwd", E=E, H=H, Dk=Dk, Dv=Dv, bij=bij_ehd is not None):
         rc = _lib.load().cf_fused_dpa_bwd(
             ptr(que), ptr(key), ptr(val), ptr(bij_ehd), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i),
             ptr(atom_start_n), ptr(edge_start_n), N, H, E, B, Dk, Dv, ptr(prob_eh), ptr(out), ptr(gout),
