@@ -49,10 +49,12 @@ def gaussian_exponents(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, ga
     """a[i,h] = -rho(normalised alpha) / (2 r0^2), alpha from the un-scaled
     per-head query (models/indexed_lattice_multi_head_attention_cuda.py:636-722)."""
     n, h, d = q.shape
+    # (per-head dot products; written as a product + sum rather than the reference's
+    # batch of N*H 1xd @ dx1 matmuls, which is two orders of magnitude slower on hipBLASLt)
     if params.gauss_state.startswith("q"):
-        alpha = q.reshape(n, h, 1, d) @ lattice_pos_weights.reshape(h, d, 1)
+        alpha = (q * lattice_pos_weights.reshape(1, h, d)).sum(-1)
     elif params.gauss_state == "1":
-        alpha = torch.ones_like(q).reshape(n, h, 1, d) @ lattice_pos_weights.reshape(h, d, 1)
+        alpha = lattice_pos_weights.reshape(1, h, d).sum(-1).expand(n, h)
     else:
         alpha = F.linear(query, lattice_pos_weights)
     alpha = alpha.view(n, h)

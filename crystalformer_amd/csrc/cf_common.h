@@ -23,6 +23,13 @@ void set_error(const char *fmt, ...);
 int hip_failed(hipError_t err, const char *what);
 int device_cu_count();
 
+// real_enc_mfma.hip
+int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,
+                              const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
+                              int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
+                              int64_t W_num, const float *rvlen, float cutoff, int lattice_range,
+                              int min_range, float *z, float *v, hipStream_t st);
+
 #define CF_REQUIRE(cond, code, ...)            \
     do {                                       \
         if (!(cond)) {                         \

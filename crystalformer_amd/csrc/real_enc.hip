@@ -846,8 +846,8 @@ extern "C" int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const 
                                const int64_t *batch_i, const int64_t *edge_ij_e, int64_t N, int64_t H,
                                int64_t E, int64_t B, int64_t K, int64_t D, double dist_max,
                                double wscale, const float *W_k, int64_t W_num, const float *rvlen_n,
-                               double cutoff_radius, int lattice_range, int minimum_range, float *z_ek,
-                               float *v_ekd, void *stream)
+                               double cutoff_radius, int lattice_range, int minimum_range,
+                               const int64_t *pairs_u, int64_t U, float *z_ek, float *v_ekd, void *stream)
 {
     EncArgs p;
     int rc = fill_args(p, "cf_real_enc_fwd", a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, N, H, E, B, K,
@@ -857,8 +857,21 @@ extern "C" int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const 
     if (E == 0) return CF_OK;
     CF_REQUIRE(z_ek, CF_ERR_INVALID_ARGUMENT, "cf_real_enc_fwd: z_ek is null");
     CF_REQUIRE(K == 0 || v_ekd, CF_ERR_INVALID_ARGUMENT, "cf_real_enc_fwd: v_ekd is null with K>0");
+    CF_REQUIRE(!pairs_u || 2 * U == E + N, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_fwd: a pair list over dense crystal blocks has (E+N)/2 = %lld entries, got %lld",
+               (long long)((E + N) / 2), (long long)U);
     p.z = z_ek;
     p.v = v_ekd;
+    if (pairs_u && K > 0) {
+        rc = launch_real_enc_fwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, N, H, E, K, D,
+                                       p.bin_step, p.s_scale, p.W, W_num, rvlen_n, p.cutoff, lattice_range,
+                                       minimum_range, z_ek, v_ekd, (hipStream_t)stream);
+        if (rc == CF_OK) {
+            CF_CHECK_LAUNCH("cf_real_enc_fwd (pairs)");
+            return CF_OK;
+        }
+        if (rc != CF_ERR_UNSUPPORTED) return rc;   // otherwise: shape not instantiated, use the per-edge kernel
+    }
     rc = CF_DISPATCH_H(H, launch_fwd, p, (hipStream_t)stream);
     if (rc) return rc;
     CF_CHECK_LAUNCH("cf_real_enc_fwd");

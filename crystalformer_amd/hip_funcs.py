@@ -56,6 +56,12 @@ class KernelManager:
     MAX_SYSTEM_SIZE: int = 1 << 30
     MAX_SYSTEM_SIZE_POW2: int = 1 << 30
     RUNNING_SUM_LEN: int = 8
+    # The edge list is the dense per-crystal block layout of get_edge_index
+    # (edge (i,j) of a crystal with n atoms at e0 + i*n + j).  The reference's
+    # transposes assume it too (models/cuda_funcs/fused_dpa.py:141-159).  With it
+    # the encoding evaluates both directions of an atom pair together; set False
+    # for arbitrary edge lists (per-edge kernels; attention backward unavailable).
+    DENSE_EDGE_BLOCKS: bool = True
     compiled: bool = False
 
 
@@ -77,6 +83,12 @@ def compile_kernels(lattice_range: int, head_num: int, key_head_dim: int, value_
     KernelManager.VPE_DIM = int(value_pe_dim)
     _lib.load()
     KernelManager.compiled = True
+
+
+def _pairs(batch_i: Tensor, edge_ij_e: Tensor, tvecs_n: Tensor, K: int) -> Optional[Tensor]:
+    if K <= 0 or not KernelManager.DENSE_EDGE_BLOCKS or edge_ij_e.shape[1] == 0:
+        return None
+    return ops.cached_edge_pairs(batch_i, edge_ij_e, tvecs_n.shape[0])
 
 
 def _w_leading(W_k: Optional[Tensor]) -> int:
@@ -110,7 +122,8 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         W_k = W_k.detach().contiguous() if W_k is not None else None
         z_ek, v_ekd = ops.real_enc_fwd(
             a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, W_k, rvlen_n,
-            cutoff_radius, KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
+            cutoff_radius, KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE,
+            pairs_u=_pairs(batch_i, edge_ij_e, tvecs_n, K))
         ctx.save_for_backward(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, W_k, z_ek)
         ctx.K, ctx.dist_max, ctx.wscale, ctx.cutoff_radius = K, dist_max, wscale, cutoff_radius
         ctx.ranges = (KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
@@ -122,7 +135,7 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gz_ek, gv_ekd=None):
         a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, W_k, z_ek = ctx.saved_tensors
-        e_start_i = ops.edge_row_offsets(edge_ij_e, a_ik.shape[0])
+        e_start_i = ops.cached_edge_row_offsets(edge_ij_e, a_ik.shape[0])
         gz = gz_ek.detach().contiguous() if gz_ek is not None else None
         gv = gv_ekd.detach().contiguous() if gv_ekd is not None else None
         ga_ik, gW_k = ops.real_enc_bwd(
@@ -148,7 +161,8 @@ class RealPeriodicEncodingFuncCUDA(torch.autograd.Function):
         E = edge_ij_e.shape[1]
         z_ek, s_ekk = ops.real_enc_fwd(
             a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, None, rvlen_n,
-            cutoff_radius, KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
+            cutoff_radius, KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE,
+            pairs_u=_pairs(batch_i, edge_ij_e, tvecs_n, K))
         v_out = s_ekk
         if W_k is not None and K > 0:
             W_k = W_k.detach().contiguous()
@@ -168,7 +182,7 @@ class RealPeriodicEncodingFuncCUDA(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gz_ek, gv_ekd=None):
         a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, W_k, z_ek, s_ekk = ctx.saved_tensors
-        e_start_i = ops.edge_row_offsets(edge_ij_e, a_ik.shape[0])
+        e_start_i = ops.cached_edge_row_offsets(edge_ij_e, a_ik.shape[0])
         gW_k = None
         gv = gv_ekd.detach().contiguous() if gv_ekd is not None else None
         if W_k is not None and gv is not None:
@@ -195,7 +209,7 @@ class FusedDotProductAttentionCUDA(torch.autograd.Function):
         bij_ehk = bij_ehk.contiguous().detach() if bij_ehk is not None else None
         batch_i = batch_i.contiguous()
         edge_ij_e = edge_ij_e.contiguous()
-        e_start_i = ops.edge_row_offsets(edge_ij_e, que_ihk.shape[0])
+        e_start_i = ops.cached_edge_row_offsets(edge_ij_e, que_ihk.shape[0])
         output, prob_eh = ops.fused_dpa_fwd(que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, edge_ij_e, e_start_i)
         ctx.save_for_backward(que_ihk, key_ihk, val_ihk, bij_ehk, batch_i, edge_ij_e, e_start_i, prob_eh,
                               output)

@@ -114,8 +114,12 @@ def crystal_offsets(batch_i: Tensor, num_slots: Optional[int] = None) -> Tuple[T
 def real_enc_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor,
                  K: int, dist_max: float, wscale: float, W_k: Optional[Tensor] = None,
                  rvlen_n: Optional[Tensor] = None, cutoff_radius: Optional[float] = None,
-                 lattice_range: int = 2, minimum_range: int = 0) -> Tuple[Tensor, Optional[Tensor]]:
-    dev = require_device(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, W_k, rvlen_n)
+                 lattice_range: int = 2, minimum_range: int = 0,
+                 pairs_u: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
+    """``pairs_u`` (U,2) from :func:`edge_pairs` selects the matrix-core kernel
+    that evaluates both directions of an atom pair together."""
+    dev = require_device(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, W_k, rvlen_n, pairs_u)
+    pairs_u = _i64(pairs_u, "pairs_u")
     a_ik, rpos_ij_e, tvecs_n = _f32(a_ik, "a_ik"), _f32(rpos_ij_e, "rpos_ij_e"), _f32(tvecs_n, "tvecs_n")
     batch_i, edge_ij_e = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e")
     W_k, rvlen_n = _f32(W_k, "W_k"), _f32(rvlen_n, "rvlen_n")
@@ -140,8 +144,8 @@ def real_enc_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
         rc = _lib.load().cf_real_enc_fwd(
             ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), N, H, E, B, K, D,
             float(dist_max), float(wscale), ptr(W_k if K > 0 else None), W_num,
-            ptr(rvlen_n), cutoff, int(lattice_range), int(minimum_range), ptr(z), ptr(v),
-            stream_handle(dev))
+            ptr(rvlen_n), cutoff, int(lattice_range), int(minimum_range), ptr(pairs_u),
+            0 if pairs_u is None else pairs_u.shape[0], ptr(z), ptr(v), stream_handle(dev))
     check(rc, "cf_real_enc_fwd")
     return z, v
 
@@ -245,7 +249,7 @@ def fused_dpa_bwd(que: Tensor, key: Tensor, val: Tensor, bij_ehd: Optional[Tenso
     Dv = val.shape[-1]
     E = edge_ij_e.shape[1]
     if atom_start_n is None or edge_start_n is None:
-        atom_start_n, edge_start_n = crystal_offsets(batch_i)
+        atom_start_n, edge_start_n = cached_crystal_offsets(batch_i)
     atom_start_n, edge_start_n = _i64(atom_start_n, "atom_start_n"), _i64(edge_start_n, "edge_start_n")
     B = atom_start_n.numel() - 1
     gq, gk, gv = torch.empty_like(que), torch.empty_like(key), torch.empty_like(val)
@@ -322,3 +326,72 @@ def edge_index(sizes: Tensor, pos: Optional[Tensor] = None,
                                        ptr(rpos), stream_handle(dev))
     check(rc, "cf_edge_index")
     return edges, rpos
+
+
+def edge_pairs(sizes: Tensor, num_atoms: Optional[int] = None, num_edges: Optional[int] = None) -> Tensor:
+    """(U,2) int64: for every unordered atom pair of each crystal's dense edge
+    block the edge (i->j), i <= j, and its reverse (j->i).  U = (E + N)/2; pass
+    ``num_atoms`` and ``num_edges`` when known to avoid a host sync."""
+    dev = require_device(sizes)
+    sizes = _i64(sizes, "sizes")
+    B = sizes.numel()
+    atom_start = F.pad(sizes.cumsum(0), (1, 0))
+    edge_start = F.pad((sizes * sizes).cumsum(0), (1, 0))
+    unit_start = F.pad((sizes * (sizes + 1) // 2).cumsum(0), (1, 0))
+    if num_atoms is None or num_edges is None:
+        tail = torch.stack([atom_start[-1], edge_start[-1]]).tolist() if B > 0 else [0, 0]
+        num_atoms, num_edges = int(tail[0]), int(tail[1])
+    U = (num_edges + num_atoms) // 2
+    pairs = torch.empty((U, 2), dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_edge_pairs(ptr(atom_start), ptr(edge_start), ptr(unit_start), B, num_edges,
+                                       ptr(pairs), stream_handle(dev))
+    check(rc, "cf_edge_pairs")
+    return pairs
+
+
+# Small caches of per-batch index structures derived from (batch_i, edge_ij_e):
+# the attention blocks of one forward all see the same tensors, so the pair list
+# and the CSR offsets are built once.  Entries keep their key tensors alive, so a
+# recycled address can never alias a stale entry.
+_index_cache: list = []
+_INDEX_CACHE_SIZE = 8
+
+
+def _cache_lookup(kind: str, *keys: Tensor):
+    sig = (kind,) + tuple((k.data_ptr(), tuple(k.shape), k._version) for k in keys)
+    for entry in _index_cache:
+        if entry[0] == sig:
+            return sig, entry[2]
+    return sig, None
+
+
+def _cache_store(sig, keys, value):
+    _index_cache.insert(0, (sig, keys, value))
+    del _index_cache[_INDEX_CACHE_SIZE:]
+    return value
+
+
+def cached_edge_row_offsets(edge_ij_e: Tensor, num_atoms: int) -> Tensor:
+    sig, hit = _cache_lookup("e_start", edge_ij_e)
+    if hit is not None and hit.numel() == num_atoms + 1:
+        return hit
+    return _cache_store(sig, (edge_ij_e,), edge_row_offsets(edge_ij_e, num_atoms))
+
+
+def cached_edge_pairs(batch_i: Tensor, edge_ij_e: Tensor, num_crystals: int) -> Tensor:
+    """Pair list for a dense per-crystal edge layout (see :func:`edge_pairs`)."""
+    sig, hit = _cache_lookup("pairs", batch_i, edge_ij_e)
+    if hit is not None:
+        return hit
+    sizes = torch.zeros(num_crystals, dtype=torch.int64, device=batch_i.device)
+    sizes.scatter_add_(0, batch_i, torch.ones_like(batch_i))
+    pairs = edge_pairs(sizes, batch_i.numel(), edge_ij_e.shape[1])
+    return _cache_store(sig, (batch_i, edge_ij_e), pairs)
+
+
+def cached_crystal_offsets(batch_i: Tensor) -> Tuple[Tensor, Tensor]:
+    sig, hit = _cache_lookup("offsets", batch_i)
+    if hit is not None:
+        return hit
+    return _cache_store(sig, (batch_i,), crystal_offsets(batch_i))

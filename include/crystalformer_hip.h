@@ -59,6 +59,13 @@ int cf_max_translation_range(void);
  *                  <0: adaptive box from sqrt(-0.5/a)*|cutoff| per (atom,head);
  *                  >0: adaptive box from that radius.  Non-zero needs rvlen_n.
  *   minimum_range  lower bound of every adaptive half-width (0 = none)
+ *   pairs_u   nullable, (U,2): for every unordered pair of atoms of a crystal
+ *             (self pairs included) the edge (i->j), i <= j, and its reverse
+ *             (j->i), as written by cf_edge_pairs.  When given (and K > 0) the
+ *             two directions of a pair are evaluated together on the matrix
+ *             cores; every edge must appear in exactly one pair and its reverse
+ *             must carry rpos = -rpos.  NULL selects the per-edge kernels,
+ *             which accept any edge list.
  * Outputs
  *   z_ek  (E,H)                       log sum_n exp(a d^2)
  *   v_ekd nullable if K==0; (E,H,K) when W_k is NULL, else (E,H,D)
@@ -68,7 +75,8 @@ int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvec
                     int64_t N, int64_t H, int64_t E, int64_t B, int64_t K, int64_t D,
                     double dist_max, double wscale, const float *W_k, int64_t W_num,
                     const float *rvlen_n, double cutoff_radius, int lattice_range,
-                    int minimum_range, float *z_ek, float *v_ekd, void *stream);
+                    int minimum_range, const int64_t *pairs_u, int64_t U,
+                    float *z_ek, float *v_ekd, void *stream);
 
 /*
  * Bytes of device scratch cf_real_enc_bwd needs for the given sizes
@@ -191,6 +199,20 @@ int cf_minimum_distance(const float *rpos_ij_e, const float *tvecs_n, const int6
  */
 int cf_edge_index(const int64_t *atom_start_n, const int64_t *edge_start_n, int64_t B,
                   int64_t E, const float *pos, int64_t *edge_ij_e, float *rpos_ij_e,
+                  void *stream);
+
+/*
+ * Pair list of the dense per-crystal edge blocks: for each crystal of n atoms
+ * the n(n+1)/2 pairs (i <= j) in row-major order of the upper triangle.
+ * No counterpart in the reference (its kernels treat the two directions of an
+ * edge independently, models/kernels/real_enc_proj_fwd.cu:24-31).
+ *   atom_start_n, edge_start_n, unit_start_n (B+1): leading-zero cumulative
+ *   sums of sizes, sizes^2 and sizes*(sizes+1)/2
+ * Output
+ *   pairs_u (U,2) with U = unit_start_n[B] = (E + N) / 2
+ */
+int cf_edge_pairs(const int64_t *atom_start_n, const int64_t *edge_start_n,
+                  const int64_t *unit_start_n, int64_t B, int64_t E, int64_t *pairs_u,
                   void *stream);
 
 #ifdef __cplusplus
