@@ -10,15 +10,21 @@
 // v_mfma_f32_16x16x4_f32: 4 translations per instruction, 16 bins x 16 columns
 // per tile, K/16 tiles.
 //
+// A work-group is 8 wavefronts; in every round each wavefront owns one unit.
 // Lane roles inside a wavefront (q = lane / 16, c = lane % 16):
-//   wide phase   lane = translation (64 at a time): decode, d^2, sqrt, in-box
-//                bits of the 16 columns -> a 1 KB LDS ring per wave;
-//   deep phase   for each group of 4 translations, lane (q, c) reads translation
+//   staging      lane = translation (64 at a time): decode, d^2, sqrt, in-box
+//                bits of the 16 columns and "which 16-bin tiles can this distance
+//                reach" bits -> per-wave LDS ring.  Translations out of reach of
+//                every bin are packed at the back of the ring so that whole
+//                groups of 4 skip the Gaussians;
+//   accumulation for each group of 4 translations, lane (q, c) reads translation
 //                q of the group, forms column c's weight exp(a_c (d^2 - d^2min_c))
-//                (B operand) and the Gaussians of bins 16m + c (A operands);
-//   epilogue     lane (q, c) owns bins 16m + 4q + r of column c (the MFMA
-//                accumulator layout); the D x K projection is applied from LDS
-//                and reduced over q with two cross-lane adds.
+//                (B operand) and, for the tiles the group can reach, the Gaussians
+//                of bins 16m + c (A operands);
+//   projection   v = W_h S: the 8 wavefronts park their normalised S in LDS; then
+//                wavefront w multiplies head w's D x K matrix (held in registers
+//                as MFMA A operands for the whole kernel) with the 16 columns of
+//                that head (8 units x 2 directions) and stores 16-byte rows of v.
 #include "cf_common.h"
 
 namespace {
@@ -45,6 +51,8 @@ struct PairArgs {
     float cutoff;
     int lattice_range, min_range;
     float bin_step, s_scale;
+    float inv_bin_step;     // distance argument -> fractional bin coordinate
+    float window;           // bins beyond which a Gaussian is below 2^-40 and is not evaluated
 };
 
 struct Cell {
@@ -60,19 +68,29 @@ __device__ __forceinline__ float dist2(const Cell &c, float n1, float n2, float 
     return dx * dx + dy * dy + dz * dz;
 }
 
-__device__ __forceinline__ void decode(int idx, int S2, int S3, int U1, int U2, int U3, int &n1, int &n2,
-                                       int &n3)
+// Box geometry of one unit (wave-uniform).
+struct BoxDims {
+    int U1, U2, U3, S2, S3, plane, T;
+    float inv_plane, inv_S3;
+};
+
+// idx -> (n1,n2,n3), first index slowest; float reciprocals with one correction
+// step instead of integer division (idx < 2^21).
+__device__ __forceinline__ void decode(const BoxDims &bx, int idx, int &n1, int &n2, int &n3)
 {
-    int plane = S2 * S3;
-    int q1 = idx / plane;
-    int rem = idx - q1 * plane;
-    int q2 = rem / S3;
-    n1 = q1 - U1;
-    n2 = q2 - U2;
-    n3 = rem - q2 * S3 - U3;
+    int q1 = (int)(((float)idx + 0.5f) * bx.inv_plane);
+    int rem = idx - q1 * bx.plane;
+    if (rem < 0) { q1--; rem += bx.plane; }
+    if (rem >= bx.plane) { q1++; rem -= bx.plane; }
+    int q2 = (int)(((float)rem + 0.5f) * bx.inv_S3);
+    int r3 = rem - q2 * bx.S3;
+    if (r3 < 0) { q2--; r3 += bx.S3; }
+    if (r3 >= bx.S3) { q2++; r3 -= bx.S3; }
+    n1 = q1 - bx.U1;
+    n2 = q2 - bx.U2;
+    n3 = r3 - bx.U3;
 }
 
-// max over the 16 lanes that share q (xor 1,2,4,8) and then over q (xor 16,32)
 __device__ __forceinline__ int wave_max_int(int v)
 {
 #pragma unroll
@@ -80,148 +98,292 @@ __device__ __forceinline__ int wave_max_int(int v)
     return v;
 }
 
-// W staged as [h][d][KP] with KP = 16*NT + 4 floats (16-byte aligned rows).
-template <int NT, bool UNIFORM, bool PROJ>
-__global__ __launch_bounds__(256) void real_enc_fwd_pair_kernel(PairArgs p)
+constexpr int RING_CAP = 256;            // translations staged per pass
+constexpr int RING_SLOTS = RING_CAP + 16; // + neutral padding (last groups, look-ahead) between the two blocks
+
+constexpr int WPB = 8;                   // wavefronts per work-group = units per round
+
+// Projection modes
+constexpr int PROJ_NONE = 0;             // v = normalised Gaussian averages (E,H,K)
+constexpr int PROJ_SHARED = 1;           // one W per head: batched on the matrix cores
+constexpr int PROJ_INDEXED = 2;          // W per edge or per atom: read from global memory
+
+// Bin handled by reduction step s (0..4*NT-1) and sub-lane kk (0..3) of the projection:
+// chosen so that a lane's 4 consecutive steps read 4 consecutive bins (one 16-byte load).
+__device__ __forceinline__ int proj_bin(int s, int kk) { return 16 * (s >> 2) + 4 * kk + (s & 3); }
+
+// LDS per work-group: per wave three ring arrays of RING_SLOTS words (d^2, distance
+// argument, flag bits); for PROJ_SHARED also WPB x 16 staged columns of 16*NT+1 floats
+// and WPB x 2 edge ids.
+template <int NT, bool UNIFORM, int PROJ, int DT>
+__global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
 {
     extern __shared__ __align__(16) float lds[];
-    constexpr int KP = 16 * NT + 4;
+    constexpr int SROW = 16 * NT + 1;     // floats per staged column, odd stride
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int wpb = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform by construction
     const int q = lane >> 4;
     const int c = lane & 15;
     const int H = p.H, K = p.K, D = p.D;
-    const bool w_shared = PROJ && p.W_num == 1;
-    float *Wl = lds;
-    float4_t *ring = reinterpret_cast<float4_t *>(lds + (w_shared ? H * D * KP : 0)) + wave * WAVE;
+    // read-only inputs: plain restrict pointers let per-unit descriptors use scalar loads
+    const int64_t *__restrict__ g_pairs = p.pairs;
+    const int64_t *__restrict__ g_edges = p.edges;
+    const int64_t *__restrict__ g_batch = p.batch;
+    const float *__restrict__ g_rpos = p.rpos;
+    const float *__restrict__ g_tvecs = p.tvecs;
+    const float *__restrict__ g_a = p.a_ik;
+    const float *__restrict__ g_rvlen = p.rvlen;
+    float *ring_d2 = lds + wave * (3 * RING_SLOTS);
+    float *ring_s = ring_d2 + RING_SLOTS;
+    int *ring_bits = reinterpret_cast<int *>(ring_s + RING_SLOTS);
+    float *Sbuf = lds + WPB * 3 * RING_SLOTS;                        // [WPB][16][SROW]
+    int64_t *meta = reinterpret_cast<int64_t *>(Sbuf + WPB * 16 * SROW);   // [WPB][2]
 
-    if (w_shared) {
-        for (int x = threadIdx.x; x < H * D * KP; x += blockDim.x) {
-            int hd = x / KP, k = x - hd * KP;
-            Wl[x] = (k < K) ? p.W[hd * K + k] : 0.f;
-        }
-        __syncthreads();
-    }
     // Gaussian argument of bin 16m + c at distance 0
     float ck[NT];
 #pragma unroll
     for (int m = 0; m < NT; m++) ck[m] = p.bin_step * (float)(16 * m + c + 1);
 
-    const int64_t items = p.U * p.head_groups;
-    for (int64_t it = (int64_t)blockIdx.x * wpb + wave; it < items; it += (int64_t)gridDim.x * wpb) {
-        const int64_t u = it / p.head_groups;
-        const int hg = (int)(it - u * p.head_groups);
-        const int64_t e_ij = p.pairs[2 * u], e_ji = p.pairs[2 * u + 1];
-        const int64_t i = p.edges[e_ij], j = p.edges[p.E + e_ij];
-        const int64_t n = p.batch[i];
-        Cell cell;
-        cell.rx = p.rpos[e_ij * 3 + 0];
-        cell.ry = p.rpos[e_ij * 3 + 1];
-        cell.rz = p.rpos[e_ij * 3 + 2];
+    // projection operands of this wave's head, reloaded when the head group changes
+    float Wa[PROJ == PROJ_SHARED ? DT : 1][PROJ == PROJ_SHARED ? 4 * NT : 1];
+    int wa_hg = -1;
+
+    const int64_t rounds_per_hg = (p.U + WPB - 1) / WPB;
+    const int64_t rounds = rounds_per_hg * p.head_groups;
+    // unit descriptor of the coming round, fetched one round ahead
+    struct Desc { int64_t e_ij, e_ji, i, j, n; };
+    auto fetch = [&](int64_t rd_) {
+        Desc dsc;
+        const int hg_ = (int)(rd_ / rounds_per_hg);
+        int64_t u_ = (rd_ - (int64_t)hg_ * rounds_per_hg) * WPB + wave;
+        if (rd_ >= rounds || u_ >= p.U) u_ = 0;
+        dsc.e_ij = g_pairs[2 * u_];
+        dsc.e_ji = g_pairs[2 * u_ + 1];
+        dsc.i = g_edges[dsc.e_ij];
+        dsc.j = g_edges[p.E + dsc.e_ij];
+        dsc.n = g_batch[dsc.i];
+        return dsc;
+    };
+    Desc next = fetch(blockIdx.x);
+    for (int64_t rd = blockIdx.x; rd < rounds; rd += gridDim.x) {
+        const int hg = (int)(rd / rounds_per_hg);
+        const int64_t u = (rd - (int64_t)hg * rounds_per_hg) * WPB + wave;
+        const bool unit_on = u < p.U;
+        const Desc cur = next;
+        next = fetch(rd + gridDim.x);
+        if (PROJ == PROJ_SHARED && hg != wa_hg) {
+            const int hw = hg * 8 + wave;
 #pragma unroll
-        for (int x = 0; x < 9; x++) cell.t[x] = p.tvecs[n * 9 + x];
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int s = 0; s < 4 * NT; s++) {
+                    const int d = 16 * dt + c, k = proj_bin(s, q);
+                    Wa[dt][s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
+                }
+            wa_hg = hg;
+        }
+        const int64_t e_ij = cur.e_ij, e_ji = cur.e_ji, i = cur.i, j = cur.j, n = cur.n;
+        Cell cell;
+        cell.rx = g_rpos[e_ij * 3 + 0];
+        cell.ry = g_rpos[e_ij * 3 + 1];
+        cell.rz = g_rpos[e_ij * 3 + 2];
+#pragma unroll
+        for (int x = 0; x < 9; x++) cell.t[x] = g_tvecs[n * 9 + x];
 
         // column c: head (hg*8 + c%8) of atom i (c < 8) or atom j (c >= 8)
         const int h = hg * 8 + (c & 7);
-        const bool col_on = h < H && (c < 8 || e_ji != e_ij);
+        const bool col_on = unit_on && h < H && (c < 8 || e_ji != e_ij);
         const int64_t atom = (c < 8) ? i : j;
-        const float a = col_on ? p.a_ik[atom * H + h] : -1.0f;
+        const float a = col_on ? g_a[atom * H + h] : -1.0f;
         const float a2 = a * LOG2E;
 
         // translation box: union over the 16 columns; per-column boxes when they differ
-        int U1 = p.lattice_range, U2 = U1, U3 = U1;
-        int R1 = U1, R2 = U1, R3 = U1;
+        BoxDims bx;
+        bx.U1 = bx.U2 = bx.U3 = p.lattice_range;
+        int R1 = bx.U1, R2 = bx.U1, R3 = bx.U1;
         if (!UNIFORM) {
-            float rvl[3] = {p.rvlen[n * 3 + 0], p.rvlen[n * 3 + 1], p.rvlen[n * 3 + 2]};
+            float rvl[3] = {g_rvlen[n * 3 + 0], g_rvlen[n * 3 + 1], g_rvlen[n * 3 + 2]};
             range_rule(a, p.cutoff, rvl, p.lattice_range, p.min_range, R1, R2, R3);
             if (!col_on) R1 = R2 = R3 = 0;
-            U1 = wave_max_int(R1);
-            U2 = wave_max_int(R2);
-            U3 = wave_max_int(R3);
+            bx.U1 = __builtin_amdgcn_readfirstlane(wave_max_int(R1));
+            bx.U2 = __builtin_amdgcn_readfirstlane(wave_max_int(R2));
+            bx.U3 = __builtin_amdgcn_readfirstlane(wave_max_int(R3));
         }
-        const int S3 = 2 * U3 + 1, S2 = 2 * U2 + 1;
-        const int T = (2 * U1 + 1) * S2 * S3;
+        bx.S3 = 2 * bx.U3 + 1;
+        bx.S2 = 2 * bx.U2 + 1;
+        bx.plane = bx.S2 * bx.S3;
+        bx.T = (2 * bx.U1 + 1) * bx.plane;
+        bx.inv_plane = 1.0f / (float)bx.plane;
+        bx.inv_S3 = 1.0f / (float)bx.S3;
+        const int T = bx.T;
 
-        // pass 1: minimum of d^2 over each column's own box
-        float d2min;
-        {
-            float mloc[UNIFORM ? 1 : 16];
+        // geometry of one translation: d^2 and the in-box bits of the 16 columns
+        auto geometry = [&](int idx, bool valid, float &d2, int &colbits) {
+            int n1, n2, n3;
+            decode(bx, valid ? idx : 0, n1, n2, n3);
+            d2 = dist2(cell, (float)n1, (float)n2, (float)n3);
+            colbits = 0;
+            if (valid) {
+                if (UNIFORM) {
+                    colbits = 0xFFFF;
+                } else {
 #pragma unroll
-            for (int x = 0; x < (UNIFORM ? 1 : 16); x++) mloc[x] = 1e10f;
-            for (int c0 = 0; c0 < T; c0 += WAVE) {
-                int idx = c0 + lane;
-                if (idx < T) {
-                    int n1, n2, n3;
-                    decode(idx, S2, S3, U1, U2, U3, n1, n2, n3);
-                    float d2 = dist2(cell, (float)n1, (float)n2, (float)n3);
-                    if (UNIFORM) {
-                        mloc[0] = fminf(mloc[0], d2);
-                    } else {
-#pragma unroll
-                        for (int x = 0; x < 16; x++) {
-                            int r1 = __builtin_amdgcn_readlane(R1, x);
-                            int r2 = __builtin_amdgcn_readlane(R2, x);
-                            int r3 = __builtin_amdgcn_readlane(R3, x);
-                            if (abs(n1) <= r1 && abs(n2) <= r2 && abs(n3) <= r3) mloc[x] = fminf(mloc[x], d2);
-                        }
+                    for (int x = 0; x < 16; x++) {
+                        int r1 = __builtin_amdgcn_readlane(R1, x);
+                        int r2 = __builtin_amdgcn_readlane(R2, x);
+                        int r3 = __builtin_amdgcn_readlane(R3, x);
+                        if (abs(n1) <= r1 && abs(n2) <= r2 && abs(n3) <= r3) colbits |= (1 << x);
                     }
                 }
             }
-            if (UNIFORM) {
-                d2min = wave_min(mloc[0]);
-            } else {
-                d2min = 1e10f;
+        };
+        // per-column minimum of d^2 over the column's own box
+        float mloc[UNIFORM ? 1 : 16];
 #pragma unroll
-                for (int x = 0; x < 16; x++) {
-                    float mx = wave_min(mloc[x]);
-                    if (c == x) d2min = mx;
+        for (int x = 0; x < (UNIFORM ? 1 : 16); x++) mloc[x] = 1e10f;
+        auto track_min = [&](float d2, int colbits) {
+            if (UNIFORM) {
+                if (colbits) mloc[0] = fminf(mloc[0], d2);
+            } else {
+#pragma unroll
+                for (int x = 0; x < 16; x++)
+                    if ((colbits >> x) & 1) mloc[x] = fminf(mloc[x], d2);
+            }
+        };
+        // boxes of up to RING_CAP translations are evaluated once and kept in registers
+        constexpr int NCACHE = RING_CAP / WAVE;
+        float d2c[NCACHE];
+        int bitsc[UNIFORM ? 1 : NCACHE];
+        const bool cached = T <= RING_CAP;
+        if (cached) {
+#pragma unroll
+            for (int ch = 0; ch < NCACHE; ch++) {
+                d2c[ch] = 0.f;
+                if (ch * WAVE < T) {
+                    int cb;
+                    geometry(ch * WAVE + lane, ch * WAVE + lane < T, d2c[ch], cb);
+                    track_min(d2c[ch], cb);
+                    if (!UNIFORM) bitsc[ch] = cb;
                 }
             }
+        } else {
+            for (int c0 = 0; c0 < T; c0 += WAVE) {
+                float d2;
+                int cb;
+                geometry(c0 + lane, c0 + lane < T, d2, cb);
+                track_min(d2, cb);
+            }
         }
+        float d2min;
+        if (UNIFORM) {
+            d2min = wave_min(mloc[0]);
+        } else {
+            d2min = 1e10f;
+#pragma unroll
+            for (int x = 0; x < 16; x++) {
+                float mx = wave_min(mloc[x]);
+                if (c == x) d2min = mx;
+            }
+        }
+        // A translation out of reach of every bin whose weight is below 2^-40 of the leading
+        // term in EVERY column cannot change an fp32 sum and is dropped.  For all columns
+        // a2_c (d2 - d2min_c) <= a2_weak (d2 - d2min_far) with the weakest decay and the
+        // largest per-column minimum.
+        const float a2_weak = wave_max(col_on ? a2 : -3.0e38f);
+        const float d2min_far = wave_max(col_on ? d2min : 0.f);
 
-        // pass 2: accumulate
         float4_t acc[NT];
 #pragma unroll
         for (int m = 0; m < NT; m++) acc[m] = float4_t{0.f, 0.f, 0.f, 0.f};
         float sum = 0.f;
-        for (int c0 = 0; c0 < T; c0 += WAVE) {
-            {   // wide phase: lane = translation
-                int idx = c0 + lane;
-                bool valid = idx < T;
-                int n1, n2, n3;
-                decode(valid ? idx : 0, S2, S3, U1, U2, U3, n1, n2, n3);
-                float d2 = dist2(cell, (float)n1, (float)n2, (float)n3);
-                float s = sqrt_hw(d2) * p.s_scale;
-                int bits = 0;
+        for (int s0 = 0; s0 < T; s0 += RING_CAP) {
+            const int cnt = min(RING_CAP, T - s0);
+            // ---- staging, lane = translation.  "Near" translations (some bin within reach)
+            // are packed upwards from slot 0, the remaining live ones downwards from the top
+            // of the ring, so that the second kind never enters the Gaussian loop.
+            int near_cnt = 0, far_cnt = 0;
+            auto stage = [&](float d2, int colbits, bool valid) {
+                const float s = sqrt_hw(d2) * p.s_scale;
+                const float xb = s * p.inv_bin_step - 1.0f;          // fractional bin coordinate
+                int bits = colbits;
                 if (valid) {
-                    if (UNIFORM) {
-                        bits = 0xFFFF;
-                    } else {
 #pragma unroll
-                        for (int x = 0; x < 16; x++) {
-                            int r1 = __builtin_amdgcn_readlane(R1, x);
-                            int r2 = __builtin_amdgcn_readlane(R2, x);
-                            int r3 = __builtin_amdgcn_readlane(R3, x);
-                            if (abs(n1) <= r1 && abs(n2) <= r2 && abs(n3) <= r3) bits |= (1 << x);
+                    for (int m = 0; m < NT; m++)
+                        if (xb >= (float)(16 * m) - p.window && xb <= (float)(16 * m + 15) + p.window)
+                            bits |= (0x10000 << m);
+                }
+                const bool is_near = valid && (bits >> 16) != 0;
+                const bool is_far = valid && !is_near && colbits != 0 && a2_weak * (d2 - d2min_far) > -40.0f;
+                const unsigned long long near_mask = __ballot(is_near);
+                const unsigned long long far_mask = __ballot(is_far);
+                const unsigned long long below = (1ull << lane) - 1ull;
+                int pos = -1;
+                if (is_near) pos = near_cnt + __popcll(near_mask & below);
+                else if (is_far) pos = RING_SLOTS - 1 - (far_cnt + __popcll(far_mask & below));
+                if (pos >= 0) {
+                    ring_d2[pos] = d2;
+                    ring_s[pos] = s;
+                    ring_bits[pos] = bits;
+                }
+                near_cnt += __popcll(near_mask);
+                far_cnt += __popcll(far_mask);
+            };
+            if (cached) {
+#pragma unroll
+                for (int ch = 0; ch < NCACHE; ch++)
+                    if (ch * WAVE < T) stage(d2c[ch], UNIFORM ? (ch * WAVE + lane < T ? 0xFFFF : 0) : bitsc[UNIFORM ? 0 : ch],
+                                             ch * WAVE + lane < T);
+            } else {
+                for (int c0 = 0; c0 < cnt; c0 += WAVE) {
+                    float d2;
+                    int cb;
+                    geometry(s0 + c0 + lane, c0 + lane < cnt, d2, cb);
+                    stage(d2, cb, c0 + lane < cnt);
+                }
+            }
+            // neutral records: 8 after the near block (last group + look-ahead), 4 below the far block
+            if (lane < 12) {
+                const int pos = lane < 8 ? near_cnt + lane : RING_SLOTS - far_cnt - 1 - (lane - 8);
+                ring_d2[pos] = __builtin_inff();
+                ring_s[pos] = 0.f;
+                ring_bits[pos] = 0;
+            }
+            wave_mem_sync();
+            // ---- accumulation over the near block: 4 translations per MFMA; the record of the
+            // next group is loaded while the current one is in use
+            {
+                const int groups = (near_cnt + 3) >> 2;
+                float d2n = ring_d2[q], sn = ring_s[q];
+                int bitsn = ring_bits[q];
+                for (int g = 0; g < groups; g++) {
+                    const float d2t = d2n, st = sn;
+                    const int bits = bitsn;
+                    const int slot = 4 * (g + 1) + q;
+                    d2n = ring_d2[slot];
+                    sn = ring_s[slot];
+                    bitsn = ring_bits[slot];
+                    float w = exp2_hw(a2 * (d2t - d2min));
+                    w = (col_on && ((bits >> c) & 1)) ? w : 0.f;
+                    sum += w;
+#pragma unroll
+                    for (int m = 0; m < NT; m++) {
+                        if (__ballot((bits & (0x10000 << m)) != 0) != 0ull) {     // wave-uniform
+                            float b = ck[m] - st;
+                            float gm = exp2_hw(-(b * b));
+                            acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, w, acc[m], 0, 0, 0);
                         }
                     }
                 }
-                ring[lane] = float4_t{d2, s, __int_as_float(bits), 0.f};
             }
-            wave_mem_sync();
-            const int groups = (min(WAVE, T - c0) + 3) >> 2;
-            for (int g = 0; g < groups; g++) {
-                const float4_t rec = ring[4 * g + q];
-                const int bits = __float_as_int(rec.z);
-                float w = exp2_hw(a2 * (rec.x - d2min));
-                w = (col_on && ((bits >> c) & 1)) ? w : 0.f;
-                sum += w;
-#pragma unroll
-                for (int m = 0; m < NT; m++) {
-                    float b = ck[m] - rec.y;
-                    float gm = exp2_hw(-(b * b));
-                    acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, w, acc[m], 0, 0, 0);
+            // ---- the far block only feeds the column sums
+            {
+                const int groups = (far_cnt + 3) >> 2;
+                for (int g = 0; g < groups; g++) {
+                    const int slot = RING_SLOTS - 4 * (g + 1) + q;
+                    const float d2t = ring_d2[slot];
+                    const int bits = ring_bits[slot];
+                    float w = exp2_hw(a2 * (d2t - d2min));
+                    sum += (col_on && ((bits >> c) & 1)) ? w : 0.f;
                 }
             }
             wave_mem_sync();
@@ -234,7 +396,7 @@ __global__ __launch_bounds__(256) void real_enc_fwd_pair_kernel(PairArgs p)
         if (col_on && q == 0) p.z[e_col * H + h] = log2_hw(sum) * LN2 + d2min * a;
 
         // epilogue: lane (q,c) holds S[bin = 16m + 4q + r][column c] in acc[m][r]
-        if (!PROJ) {
+        if (PROJ == PROJ_NONE) {
             if (col_on) {
 #pragma unroll
                 for (int m = 0; m < NT; m++) {
@@ -245,47 +407,91 @@ __global__ __launch_bounds__(256) void real_enc_fwd_pair_kernel(PairArgs p)
                         if (k0 + r < K) dst[r] = acc[m][r] * inv;
                 }
             }
+        } else if (PROJ == PROJ_SHARED) {
+            // park the normalised column (zero for inactive columns), then project per head
+            float *col = Sbuf + (wave * 16 + c) * SROW;
+#pragma unroll
+            for (int m = 0; m < NT; m++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) col[16 * m + 4 * q + r] = col_on ? acc[m][r] * inv : 0.f;
+            if (lane == 0) {
+                meta[2 * wave + 0] = unit_on ? e_ij : -1;
+                meta[2 * wave + 1] = (unit_on && e_ji != e_ij) ? e_ji : -1;
+            }
+            __syncthreads();
+            {
+                // this wave: head hw; column j of the product = direction j/8 of unit j%8
+                const int hw = hg * 8 + wave;
+                const int j = c, unit_j = j & 7, dir_j = j >> 3;
+                const float *src = Sbuf + (unit_j * 16 + dir_j * 8 + wave) * SROW;
+                float4_t out[DT];
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++) out[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t4 = 0; t4 < NT; t4++) {
+                    float sb[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) sb[r] = src[16 * t4 + 4 * q + r];
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+#pragma unroll
+                        for (int dt = 0; dt < DT; dt++)
+                            out[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(Wa[dt][4 * t4 + r], sb[r], out[dt], 0, 0, 0);
+                }
+                // lane (q, j) holds components 16dt + 4q + r of column j
+                const int64_t e_out = meta[2 * unit_j + dir_j];
+                if (e_out >= 0 && hw < H) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++) {
+                        const int dbase = 16 * dt + 4 * q;
+                        float *dst = p.v + (e_out * H + hw) * D + dbase;
+                        if (dbase + 3 < D) {
+                            *reinterpret_cast<float4_t *>(dst) = out[dt];
+                        } else {
+#pragma unroll
+                            for (int r = 0; r < 3; r++)
+                                if (dbase + r < D) dst[r] = out[dt][r];
+                        }
+                    }
+                }
+            }
+            __syncthreads();
         } else {
             int64_t w_ind = 0;
-            if (p.W_num == 1) w_ind = 0;
-            else if (p.W_num == p.E) w_ind = e_col;
+            if (p.W_num == p.E) w_ind = e_col;
             else if (p.W_num == p.N) w_ind = atom;
             const float *Wg = p.W + (w_ind * H + (col_on ? h : 0)) * (int64_t)D * K;
-            const float *Wh = Wl + (col_on ? h : 0) * D * KP;
             for (int d0 = 0; d0 < D; d0 += 16) {
-                float out[16];
+                float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;   // this lane's 4 output components
 #pragma unroll
                 for (int dd = 0; dd < 16; dd++) {
                     float o = 0.f;
-                    if (d0 + dd < D) {
+                    if (col_on && d0 + dd < D) {
 #pragma unroll
                         for (int m = 0; m < NT; m++) {
                             const int k0 = 16 * m + 4 * q;
-                            if (w_shared) {
-                                const float4_t wv = *reinterpret_cast<const float4_t *>(Wh + (d0 + dd) * KP + k0);
-                                o = fmaf(wv.x, acc[m][0], o);
-                                o = fmaf(wv.y, acc[m][1], o);
-                                o = fmaf(wv.z, acc[m][2], o);
-                                o = fmaf(wv.w, acc[m][3], o);
-                            } else {
 #pragma unroll
-                                for (int r = 0; r < 4; r++)
-                                    if (k0 + r < K) o = fmaf(Wg[(int64_t)(d0 + dd) * K + k0 + r], acc[m][r], o);
-                            }
+                            for (int r = 0; r < 4; r++)
+                                if (k0 + r < K) o = fmaf(Wg[(int64_t)(d0 + dd) * K + k0 + r], acc[m][r], o);
                         }
                     }
                     o += __shfl_xor(o, 16, WAVE);
                     o += __shfl_xor(o, 32, WAVE);
-                    out[dd] = o * inv;
-                }
-                // lane q writes components d0 + 4q .. d0 + 4q + 3
-                if (col_on) {
-                    float *dst = p.v + (e_col * H + h) * D + d0 + 4 * q;
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        float val = q == 0 ? out[r] : q == 1 ? out[4 + r] : q == 2 ? out[8 + r] : out[12 + r];
-                        if (d0 + 4 * q + r < D) dst[r] = val;
+                    // lane q keeps components 4q .. 4q+3
+                    if ((dd >> 2) == q) {
+                        if ((dd & 3) == 0) o0 = o;
+                        else if ((dd & 3) == 1) o1 = o;
+                        else if ((dd & 3) == 2) o2 = o;
+                        else o3 = o;
                     }
+                }
+                if (col_on) {
+                    const int dbase = d0 + 4 * q;
+                    float *dst = p.v + (e_col * H + h) * D + dbase;
+                    if (dbase + 0 < D) dst[0] = o0 * inv;
+                    if (dbase + 1 < D) dst[1] = o1 * inv;
+                    if (dbase + 2 < D) dst[2] = o2 * inv;
+                    if (dbase + 3 < D) dst[3] = o3 * inv;
                 }
             }
         }
@@ -327,8 +533,8 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
                               int64_t W_num, const float *rvlen, float cutoff, int lattice_range,
                               int min_range, float *z, float *v, hipStream_t st)
 {
-    if (K < 1 || K > 128 || (K > 64 && W)) return CF_ERR_UNSUPPORTED;
-    if (W && (D < 1 || D > 64 || (D % 4) != 0)) return CF_ERR_UNSUPPORTED;
+    if (K < 1 || K > 128) return CF_ERR_UNSUPPORTED;
+    if (W && (D < 1 || D > 64)) return CF_ERR_UNSUPPORTED;
     PairArgs p{};
     p.a_ik = a_ik; p.rpos = rpos; p.tvecs = tvecs; p.batch = batch; p.edges = edges; p.pairs = pairs;
     p.W = W; p.rvlen = rvlen; p.z = z; p.v = v;
@@ -337,29 +543,34 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     p.head_groups = (int)((H + 7) / 8);
     p.cutoff = cutoff; p.lattice_range = lattice_range; p.min_range = min_range;
     p.bin_step = bin_step; p.s_scale = s_scale;
+    p.inv_bin_step = 1.0f / bin_step;
+    p.window = sqrtf(40.0f) / bin_step;                 // exp2(-(bin_step*x)^2) < 2^-40 beyond it
     const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
-    const int KP = 16 * NT + 4;
-    const int wpb = 4;
-    const bool proj = W != nullptr;
     const bool uniform = cutoff == 0.0f;
-    size_t lds = sizeof(float) * ((proj && W_num == 1 ? (size_t)H * D * KP : 0) + (size_t)wpb * WAVE * 4);
-    if (lds > 64 * 1024) return CF_ERR_UNSUPPORTED;
-    const int64_t items = U * p.head_groups;
-    int64_t blocks = (items + wpb - 1) / wpb;
-    int64_t cap = (int64_t)device_cu_count() * 4;      // 16 waves per CU
+    int mode = PROJ_NONE;
+    if (W) mode = (W_num == 1) ? PROJ_SHARED : PROJ_INDEXED;
+    if (mode == PROJ_SHARED && D > 32) return CF_ERR_UNSUPPORTED;
+    const int DT = (mode == PROJ_SHARED && D > 16) ? 2 : 1;
+    size_t lds = sizeof(float) * (size_t)WPB * 3 * RING_SLOTS;
+    if (mode == PROJ_SHARED) lds += sizeof(float) * (size_t)WPB * 16 * (16 * NT + 1) + sizeof(int64_t) * WPB * 2 + 8;
+    const int64_t rounds = ((U + WPB - 1) / WPB) * p.head_groups;
+    int64_t blocks = rounds;
+    int64_t cap = (int64_t)device_cu_count() * 2;      // 16 waves per CU
     if (blocks > cap) blocks = cap;
     if (blocks < 1) return CF_OK;
-#define CF_PAIR(NTV, UNI, PRJ) \
-    real_enc_fwd_pair_kernel<NTV, UNI, PRJ><<<(int)blocks, wpb * WAVE, lds, st>>>(p)
-#define CF_PAIR_NT(NTV)                                     \
-    do {                                                    \
-        if (uniform) {                                      \
-            if (proj) CF_PAIR(NTV, true, true);             \
-            else CF_PAIR(NTV, true, false);                 \
-        } else {                                            \
-            if (proj) CF_PAIR(NTV, false, true);            \
-            else CF_PAIR(NTV, false, false);                \
-        }                                                   \
+#define CF_PAIR(NTV, UNI, PRJ, DTV) \
+    real_enc_fwd_pair_kernel<NTV, UNI, PRJ, DTV><<<(int)blocks, WPB * WAVE, lds, st>>>(p)
+#define CF_PAIR_MODE(NTV, UNI)                                        \
+    do {                                                              \
+        if (mode == PROJ_NONE) CF_PAIR(NTV, UNI, PROJ_NONE, 1);       \
+        else if (mode == PROJ_INDEXED) CF_PAIR(NTV, UNI, PROJ_INDEXED, 1); \
+        else if (DT == 1) CF_PAIR(NTV, UNI, PROJ_SHARED, 1);          \
+        else CF_PAIR(NTV, UNI, PROJ_SHARED, 2);                       \
+    } while (0)
+#define CF_PAIR_NT(NTV)                       \
+    do {                                      \
+        if (uniform) CF_PAIR_MODE(NTV, true); \
+        else CF_PAIR_MODE(NTV, false);        \
     } while (0)
     switch (NT) {
         case 1: CF_PAIR_NT(1); break;
@@ -368,6 +579,7 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
         default: CF_PAIR_NT(8); break;
     }
 #undef CF_PAIR_NT
+#undef CF_PAIR_MODE
 #undef CF_PAIR
     return CF_OK;
 }
