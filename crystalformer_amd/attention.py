@@ -59,17 +59,15 @@ def gaussian_exponents(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, ga
         alpha = F.linear(query, lattice_pos_weights)
     alpha = alpha.view(n, h)
     if params.normalize_gauss:
-        stored = bool(gauss_scale[0] > 0)
-        if stored:
-            scale, shift = gauss_scale[0], gauss_scale[1]
-        else:
-            scale = torch.reciprocal(alpha.detach().std())
-            shift = -alpha.detach().mean()
+        # Stored statistics (gauss_scale[0] > 0) win over the statistics of this batch.
+        # Selected on the device: no host synchronisation in the attention block.
+        stored = gauss_scale[0] > 0
+        scale = torch.where(stored, gauss_scale[0], torch.reciprocal(alpha.detach().std()))
+        shift = torch.where(stored, gauss_scale[1], -alpha.detach().mean())
         alpha = (alpha + shift) * scale
-        if training and not stored:   # stored once, in the first training step
+        if training:   # written once, by the first training step
             with torch.no_grad():
-                gauss_scale[0] = scale
-                gauss_scale[1] = shift
+                gauss_scale.copy_(torch.stack([scale, shift]))
     rho = make_positive_func(params.positive_func)(alpha, params.gauss_lb_real)
     return rho * (-0.5 * params.scale_real ** -2)
 
@@ -211,11 +209,12 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             if dist_max < 0:
                 dist_max = (-dist_max) * P.scale_real
             adaptive = ()
-            if P.adaptive_cutoff_sigma < 0:
-                adaptive = (torch.norm(rvecs, 2, dim=-1), P.adaptive_cutoff_sigma)
-            elif P.adaptive_cutoff_sigma > 0:
-                adaptive = (torch.norm(rvecs, 2, dim=-1),
-                            P.scale_real * P.gauss_lb_real ** (-0.5) * P.adaptive_cutoff_sigma)
+            if P.adaptive_cutoff_sigma != 0:
+                # lengths of the reciprocal vectors; the encoder passes them precomputed as (B,3)
+                rvlen = rvecs if rvecs.dim() == 2 else torch.norm(rvecs, 2, dim=-1)
+                cutoff = P.adaptive_cutoff_sigma if P.adaptive_cutoff_sigma < 0 else \
+                    P.scale_real * P.gauss_lb_real ** (-0.5) * P.adaptive_cutoff_sigma
+                adaptive = (rvlen, cutoff)
             if proj is not None and not P.value_pe_headed:
                 proj = proj.expand(proj.shape[0], H, proj.shape[2], proj.shape[3])
             enc = RealPeriodicEncodingWithProjFuncCUDA if P.use_low_memory else RealPeriodicEncodingFuncCUDA

@@ -159,9 +159,11 @@ class CrystalformerEncoderCUDA(Module):
         P = self.lattice_params
         pos_ij, dist2_min, kr_base, rvecs, vcell, edges = compute_lattice_distances_for_cuda(
             pos, batch, trans, sizes, P.lattice_range, -1, output_real=True, output_reci=False)
+        # every block needs only the lengths of the reciprocal vectors: take the norm once
+        rvlen = torch.norm(rvecs, 2, dim=-1).contiguous()
         output = src
         for layer in self.layers:
-            output = layer(output, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot)
+            output = layer(output, batch, edges, pos_ij, dist2_min, trans, kr_base, rvlen, vcell, onehot)
         if self.norm is not None:
             output = self.norm(output)
         return output

@@ -64,6 +64,28 @@ class _timed:
         return False
 
 
+# Small caches of per-batch index structures derived from (batch_i, edge_ij_e):
+# the attention blocks of one forward all see the same tensors, so the pair list
+# and the CSR offsets are built once.  Entries keep their key tensors alive, so a
+# recycled address can never alias a stale entry.
+_index_cache: list = []
+_INDEX_CACHE_SIZE = 8
+
+
+def _cache_lookup(kind: str, *keys: Tensor):
+    sig = (kind,) + tuple((k.data_ptr(), tuple(k.shape), k._version) for k in keys)
+    for entry in _index_cache:
+        if entry[0] == sig:
+            return sig, entry[2]
+    return sig, None
+
+
+def _cache_store(sig, keys, value):
+    _index_cache.insert(0, (sig, keys, value))
+    del _index_cache[_INDEX_CACHE_SIZE:]
+    return value
+
+
 def _f32(t: Optional[Tensor], name: str) -> Optional[Tensor]:
     if t is None:
         return None
@@ -318,7 +340,14 @@ def edge_index(sizes: Tensor, pos: Optional[Tensor] = None,
     B = sizes.numel()
     atom_start = F.pad(sizes.cumsum(0), (1, 0))
     edge_start = F.pad((sizes * sizes).cumsum(0), (1, 0))
-    E = int(edge_start[-1].item()) if num_edges is None else int(num_edges)
+    if num_edges is None:
+        # one host read per distinct ``sizes`` tensor; repeated forwards over the same batch
+        # (and stream capture after a warm-up) find the count in the cache
+        sig, hit = _cache_lookup("num_edges", sizes)
+        if hit is None:
+            hit = _cache_store(sig, (sizes,), int(edge_start[-1].item()))
+        num_edges = hit
+    E = int(num_edges)
     edges = torch.empty((2, E), dtype=torch.int64, device=dev)
     rpos = torch.empty((E, 3), dtype=torch.float32, device=dev) if pos is not None else None
     with torch.cuda.device(dev):
@@ -348,28 +377,6 @@ def edge_pairs(sizes: Tensor, num_atoms: Optional[int] = None, num_edges: Option
                                        ptr(pairs), stream_handle(dev))
     check(rc, "cf_edge_pairs")
     return pairs
-
-
-# Small caches of per-batch index structures derived from (batch_i, edge_ij_e):
-# the attention blocks of one forward all see the same tensors, so the pair list
-# and the CSR offsets are built once.  Entries keep their key tensors alive, so a
-# recycled address can never alias a stale entry.
-_index_cache: list = []
-_INDEX_CACHE_SIZE = 8
-
-
-def _cache_lookup(kind: str, *keys: Tensor):
-    sig = (kind,) + tuple((k.data_ptr(), tuple(k.shape), k._version) for k in keys)
-    for entry in _index_cache:
-        if entry[0] == sig:
-            return sig, entry[2]
-    return sig, None
-
-
-def _cache_store(sig, keys, value):
-    _index_cache.insert(0, (sig, keys, value))
-    del _index_cache[_INDEX_CACHE_SIZE:]
-    return value
 
 
 def cached_edge_row_offsets(edge_ij_e: Tensor, num_atoms: int) -> Tensor:

@@ -175,7 +175,7 @@ def test_loop_attention_switch_matches_fused(dev, gold):
 
 # ------------------------------------------------- full-size configurations
 def build_model(name, seed=1, **over):
-    cfg = default_params(**CONFIGS[name]["model"], **over)
+    cfg = default_params(**{**CONFIGS[name]["model"], **over})
     torch.manual_seed(seed)
     return cfg, Latticeformer(cfg)
 
@@ -244,3 +244,30 @@ def test_full_size_properties_and_sampled_edges(dev):
         out_vb, _ = ops.fused_dpa_fwd(q, k, const, zB, vB, dv[4], es)
         out_0b, _ = ops.fused_dpa_fwd(q, k, torch.zeros_like(const), zB, vB, dv[4], es)
         assert rel_err(out_vb - out, out_0b) < 1e-5
+
+
+def test_graph_replay_matches_eager(dev):
+    """The step captured as one HIP graph: several replays, interleaved with eager work and
+    synchronisations, each equal to the eager result; new inputs of the same layout too."""
+    from crystalformer_amd.graphs import GraphedForward
+    cfg, model = build_model("cfg1_simplified_b32", num_layers=2, value_pe_dist_real=64)
+    model.to(dev).eval()
+    b = make_config_batch("cfg1_simplified_b32").to(dev)
+    with torch.no_grad():
+        y_eager = model(b).clone()
+    graphed = GraphedForward(model, b)
+    for _ in range(3):
+        y = graphed().clone()
+        torch.cuda.synchronize()
+        assert torch.equal(y, y_eager)
+        with torch.no_grad():
+            assert torch.equal(model(b), y_eager)          # eager work between replays
+        torch.cuda.synchronize()
+    b2 = make_config_batch("cfg1_simplified_b32").to(dev)
+    b2.pos.mul_(1.07)
+    b2.trans_vec.mul_(1.07)
+    with torch.no_grad():
+        y2 = model(b2).clone()
+    assert float((y2 - y_eager).abs().max()) > 1e-6        # really different physics
+    assert torch.equal(graphed(b2), y2)
+    assert torch.equal(graphed(b), y_eager)
