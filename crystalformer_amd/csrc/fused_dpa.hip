@@ -113,6 +113,128 @@ __global__ __launch_bounds__(256) void fused_dpa_fwd_kernel(DpaArgs p)
     }
 }
 
+
+// ------------------------------------------------- forward, streaming version
+// One work-group of 4 wavefronts per query atom, single pass over the edge row
+// with a running (max, sum, output) per head ("online" softmax).  Lane = (edge
+// slot, head, 4 components): the H*Dv/4 lanes of a slot read one edge's key row,
+// value row and b_ij row as consecutive 16-byte pieces (fully coalesced);
+// 4*ES = 4*64/(H*Dv/4) edges are in flight per step, the loop is unrolled 4x and
+// the key indices of the next step are fetched one step ahead.  The partial
+// (max, sum, output) of slots and wavefronts are merged through shuffles and LDS.
+// Raw logits are parked in prob[e,h] and normalised by a second, cheap sweep
+// (4*H bytes per edge).  Needs Dk == Dv, Dv/4 a power of two, H*Dv/4 <= 64.
+typedef float float4_v __attribute__((ext_vector_type(4)));
+
+constexpr int DPA_WPQ = 4;     // wavefronts per query row
+
+__global__ __launch_bounds__(256) void fused_dpa_fwd_stream_kernel(DpaArgs p, int DV4, int LPE)
+{
+    __shared__ float part[DPA_WPQ][WAVE][6];
+    __shared__ float fin[2][MAXH];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t i = blockIdx.x;
+    const int H = p.H;
+    const int HD4 = LPE;                       // float4 pieces per edge row
+    const int ES = WAVE / LPE;                 // edge slots per wavefront
+    const int es = lane / LPE;
+    const int piece = lane - es * LPE;         // which float4 of the (H,Dv) row
+    const int h = piece / DV4;
+    const bool lead = (piece - h * DV4) == 0;  // first piece of its head: owns the logit
+    const int64_t e0 = p.e_start[i], e1 = p.e_start[i + 1];
+    const int64_t *dst = p.edges + p.E;
+    const float4_v *key4 = reinterpret_cast<const float4_v *>(p.key);
+    const float4_v *val4 = reinterpret_cast<const float4_v *>(p.val);
+    const float4_v *bij4 = reinterpret_cast<const float4_v *>(p.bij);
+    const float4_v q4 = reinterpret_cast<const float4_v *>(p.que)[i * HD4 + piece];
+
+    float m = -1.0e30f, l = 0.f;
+    float4_v acc = {0.f, 0.f, 0.f, 0.f};
+    auto step = [&](int64_t e, int64_t j) {
+        const float4_v k4 = key4[j * HD4 + piece];
+        float4_v v4 = val4[j * HD4 + piece];
+        if (bij4) {
+            const float4_v b4 = bij4[e * HD4 + piece];
+            v4 += b4;
+        }
+        float s = q4.x * k4.x + q4.y * k4.y + q4.z * k4.z + q4.w * k4.w;
+        for (int off = DV4 >> 1; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
+        if (p.aij) s += p.aij[e * H + h];
+        if (lead) p.prob[e * H + h] = s;
+        const float m_new = fmaxf(m, s);
+        const float sc = exp2_hw((m - m_new) * LOG2E);
+        const float pe = exp2_hw((s - m_new) * LOG2E);
+        l = l * sc + pe;
+        acc = acc * sc + v4 * pe;
+        m = m_new;
+    };
+    const int stride = DPA_WPQ * ES;
+    int64_t e = e0 + wave * ES + es;
+    // key indices one step (4 edges per slot) ahead
+    int64_t jn[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) jn[u] = (e + u * stride < e1) ? dst[e + u * stride] : 0;
+    for (; e + 3 * stride < e1; e += 4 * stride) {
+        int64_t jc[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) jc[u] = jn[u];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int64_t en = e + (4 + u) * stride;
+            jn[u] = (en < e1) ? dst[en] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) step(e + u * stride, jc[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        if (e + u * stride < e1) step(e + u * stride, jn[u]);
+    // merge the edge slots of this wavefront
+    auto merge = [&](float mo, float lo, float4_v ao) {
+        const float m_new = fmaxf(m, mo);
+        const float s1 = exp2_hw((m - m_new) * LOG2E), s2 = exp2_hw((mo - m_new) * LOG2E);
+        l = l * s1 + lo * s2;
+        acc = acc * s1 + ao * s2;
+        m = m_new;
+    };
+    for (int off = LPE; off < WAVE; off <<= 1) {
+        const float mo = __shfl_xor(m, off, WAVE);
+        const float lo = __shfl_xor(l, off, WAVE);
+        float4_v ao;
+        ao.x = __shfl_xor(acc.x, off, WAVE);
+        ao.y = __shfl_xor(acc.y, off, WAVE);
+        ao.z = __shfl_xor(acc.z, off, WAVE);
+        ao.w = __shfl_xor(acc.w, off, WAVE);
+        merge(mo, lo, ao);
+    }
+    // merge the wavefronts (fixed order 0,1,2,3) in wavefront 0
+    if (es == 0) {
+        float *dstp = part[wave][piece];
+        dstp[0] = m; dstp[1] = l; dstp[2] = acc.x; dstp[3] = acc.y; dstp[4] = acc.z; dstp[5] = acc.w;
+    }
+    __syncthreads();
+    if (wave == 0 && es == 0) {
+        for (int w = 1; w < DPA_WPQ; w++) {
+            const float *src = part[w][piece];
+            merge(src[0], src[1], float4_v{src[2], src[3], src[4], src[5]});
+        }
+        const float inv = l > 0.f ? 1.0f / l : 0.f;     // an atom without edges yields zeros
+        reinterpret_cast<float4_v *>(p.out)[i * HD4 + piece] = acc * inv;
+        if (lead) {
+            fin[0][h] = m;
+            fin[1][h] = inv;
+        }
+    }
+    __syncthreads();
+    // normalise the parked logits: element x of the row's (n,H) block belongs to head x % H
+    const int hx = threadIdx.x % H;
+    const float mh = fin[0][hx], ih = fin[1][hx];
+    float *row = p.prob + e0 * H;
+    const int64_t total = (e1 - e0) * H;
+    for (int64_t x = threadIdx.x; x < total; x += blockDim.x) row[x] = exp2_hw((row[x] - mh) * LOG2E) * ih;
+}
+
 // ----------------------------------------------------------------- backward
 // rows: per query i, lane = (head, value component); Dv is a power of two <= 64
 // so that the lanes of one head form an aligned group.
@@ -240,6 +362,14 @@ extern "C" int cf_fused_dpa_fwd(const float *que, const float *key, const float 
     p.prob = prob_eh; p.out = out;
     p.N = N; p.E = E; p.H = (int)H; p.Dk = (int)Dk; p.Dv = (int)Dv;
     hipStream_t st = (hipStream_t)stream;
+    // streaming kernel when a head's components split into 16-byte pieces that tile a wavefront
+    const int64_t dv4 = Dv / 4, lpe = H * dv4;
+    const bool pow2 = (dv4 & (dv4 - 1)) == 0 && (H & (H - 1)) == 0;
+    if (Dk == Dv && Dv % 4 == 0 && pow2 && lpe >= 1 && lpe <= 64) {
+        fused_dpa_fwd_stream_kernel<<<(int)N, DPA_WPQ * WAVE, 0, st>>>(p, (int)dv4, (int)lpe);
+        CF_CHECK_LAUNCH("cf_fused_dpa_fwd");
+        return CF_OK;
+    }
     switch (H) {
         case 1: launch_fwd<1>(p, st); break;
         case 2: launch_fwd<2>(p, st); break;
