@@ -881,11 +881,15 @@ extern "C" int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const 
 extern "C" int64_t cf_real_enc_bwd_workspace(int64_t N, int64_t H, int64_t E, int64_t K, int64_t D,
                                              int64_t W_num, int want_gW)
 {
-    (void)N;
     int64_t bytes = align256(E * H * 4);                       // per-edge ga
     if (K > 0 && want_gW) {
-        bytes += align256(E * H * K * 4);                      // normalised Gaussian averages
-        if (W_num == 1) bytes += align256((int64_t)GW_SPLITS * H * D * K * 4);
+        // per-edge kernels: normalised Gaussian averages + split partial sums of gW
+        int64_t generic = align256(E * H * K * 4);
+        if (W_num == 1) generic += align256((int64_t)GW_SPLITS * H * D * K * 4);
+        // pair kernel: one H x D x K block per work-group
+        int64_t paired = 0;
+        if (W_num == 1) paired = align256((int64_t)real_enc_bwd_pairs_blocks((E + N) / 2, H) * H * D * K * 4);
+        bytes += generic > paired ? generic : paired;
     }
     return bytes;
 }
@@ -896,8 +900,8 @@ extern "C" int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const 
                                const float *gv_ekd, int64_t N, int64_t H, int64_t E, int64_t B, int64_t K,
                                int64_t D, double dist_max, double wscale, const float *W_k, int64_t W_num,
                                const float *rvlen_n, double cutoff_radius, int lattice_range,
-                               int minimum_range, void *workspace, int64_t workspace_bytes,
-                               float *ga_ik, float *gW_k, void *stream)
+                               int minimum_range, const int64_t *pairs_u, int64_t U, void *workspace,
+                               int64_t workspace_bytes, float *ga_ik, float *gW_k, void *stream)
 {
     EncArgs p;
     int rc = fill_args(p, "cf_real_enc_bwd", a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, N, H, E, B, K,
@@ -919,7 +923,29 @@ extern "C" int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const 
                "cf_real_enc_bwd: workspace of %lld bytes needed, %lld given", (long long)need,
                (long long)workspace_bytes);
     CF_REQUIRE(E == 0 || z_ek, CF_ERR_INVALID_ARGUMENT, "cf_real_enc_bwd: z_ek is null");
+    CF_REQUIRE(!pairs_u || 2 * U == E + N, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_bwd: a pair list over dense crystal blocks has (E+N)/2 = %lld entries, got %lld",
+               (long long)((E + N) / 2), (long long)U);
     char *ws = (char *)workspace;
+    if (pairs_u && E > 0 && K > 0 && W_k && W_num == 1 && gv_ekd) {
+        float *ga_edge = (float *)ws;
+        float *gW_part = want_gW ? (float *)(ws + align256(E * H * 4)) : nullptr;
+        if (gW_part && H > 8) {     // a work-group only writes the head groups it visits
+            int64_t total = (int64_t)real_enc_bwd_pairs_blocks(U, H) * H * D * K;
+            fill_zero_kernel<<<(int)((total + 255) / 256), 256, 0, st>>>(gW_part, total);
+        }
+        rc = launch_real_enc_bwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, z_ek, gz_ek,
+                                       gv_ekd, N, H, E, K, D, p.bin_step, p.s_scale, W_k, rvlen_n, p.cutoff,
+                                       lattice_range, minimum_range, ga_edge, gW_part, gW_k, st);
+        if (rc == CF_OK) {
+            CF_CHECK_LAUNCH("cf_real_enc_bwd (pairs)");
+            int64_t total = N * H;
+            reduce_ga_kernel<<<(int)((total + 255) / 256), 256, 0, st>>>(ga_edge, e_start_i, N, (int)H, ga_ik);
+            CF_CHECK_LAUNCH("cf_real_enc_bwd: reduce_ga");
+            return CF_OK;
+        }
+        if (rc != CF_ERR_UNSUPPORTED) return rc;
+    }
     p.e_start = e_start_i;
     p.z_in = z_ek;
     p.gz = gz_ek;

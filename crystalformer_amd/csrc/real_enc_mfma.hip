@@ -25,92 +25,22 @@
 //                wavefront w multiplies head w's D x K matrix (held in registers
 //                as MFMA A operands for the whole kernel) with the 16 columns of
 //                that head (8 units x 2 directions) and stores 16-byte rows of v.
-#include "cf_common.h"
+#include "real_enc_pair.h"
 
 namespace {
 
 using namespace cf;
-
-typedef float float4_t __attribute__((ext_vector_type(4)));
-
-struct PairArgs {
-    const float *a_ik;
-    const float *rpos;
-    const float *tvecs;
-    const int64_t *batch;
-    const int64_t *edges;
-    const int64_t *pairs;   // (U,2): edge (i->j) with i <= j and its reverse
-    const float *W;
-    const float *rvlen;
-    float *z;
-    float *v;
-    int64_t N, E, U;
-    int64_t W_num;
-    int H, K, D;
-    int head_groups;        // ceil(H / 8)
-    float cutoff;
-    int lattice_range, min_range;
-    float bin_step, s_scale;
-    float inv_bin_step;     // distance argument -> fractional bin coordinate
-    float window;           // bins beyond which a Gaussian is below 2^-40 and is not evaluated
-};
-
-struct Cell {
-    float rx, ry, rz;
-    float t[9];
-};
-
-__device__ __forceinline__ float dist2(const Cell &c, float n1, float n2, float n3)
-{
-    float dx = c.rx + c.t[0] * n1 + c.t[3] * n2 + c.t[6] * n3;
-    float dy = c.ry + c.t[1] * n1 + c.t[4] * n2 + c.t[7] * n3;
-    float dz = c.rz + c.t[2] * n1 + c.t[5] * n2 + c.t[8] * n3;
-    return dx * dx + dy * dy + dz * dz;
-}
-
-// Box geometry of one unit (wave-uniform).
-struct BoxDims {
-    int U1, U2, U3, S2, S3, plane, T;
-    float inv_plane, inv_S3;
-};
-
-// idx -> (n1,n2,n3), first index slowest; float reciprocals with one correction
-// step instead of integer division (idx < 2^21).
-__device__ __forceinline__ void decode(const BoxDims &bx, int idx, int &n1, int &n2, int &n3)
-{
-    int q1 = (int)(((float)idx + 0.5f) * bx.inv_plane);
-    int rem = idx - q1 * bx.plane;
-    if (rem < 0) { q1--; rem += bx.plane; }
-    if (rem >= bx.plane) { q1++; rem -= bx.plane; }
-    int q2 = (int)(((float)rem + 0.5f) * bx.inv_S3);
-    int r3 = rem - q2 * bx.S3;
-    if (r3 < 0) { q2--; r3 += bx.S3; }
-    if (r3 >= bx.S3) { q2++; r3 -= bx.S3; }
-    n1 = q1 - bx.U1;
-    n2 = q2 - bx.U2;
-    n3 = r3 - bx.U3;
-}
-
-__device__ __forceinline__ int wave_max_int(int v)
-{
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, WAVE));
-    return v;
-}
+using namespace cfpair;
 
 constexpr int RING_CAP = 256;            // translations staged per pass
 constexpr int RING_SLOTS = RING_CAP + 16; // + neutral padding (last groups, look-ahead) between the two blocks
 
-constexpr int WPB = 8;                   // wavefronts per work-group = units per round
 
 // Projection modes
 constexpr int PROJ_NONE = 0;             // v = normalised Gaussian averages (E,H,K)
 constexpr int PROJ_SHARED = 1;           // one W per head: batched on the matrix cores
 constexpr int PROJ_INDEXED = 2;          // W per edge or per atom: read from global memory
 
-// Bin handled by reduction step s (0..4*NT-1) and sub-lane kk (0..3) of the projection:
-// chosen so that a lane's 4 consecutive steps read 4 consecutive bins (one 16-byte load).
-__device__ __forceinline__ int proj_bin(int s, int kk) { return 16 * (s >> 2) + 4 * kk + (s & 3); }
 
 // LDS per work-group: per wave three ring arrays of RING_SLOTS words (d^2, distance
 // argument, flag bits); for PROJ_SHARED also WPB x 16 staged columns of 16*NT+1 floats

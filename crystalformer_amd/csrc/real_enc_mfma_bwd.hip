@@ -1,0 +1,403 @@
+// Real-space periodic encoding, backward, matrix-core version for gfx950
+// (shared projection W of shape (H,D,K), the default model path).
+//
+// Per directed edge and head, with p_t = exp(a d2_t - z):
+//     PX = sum_t p_t d2_t,  S_k = sum_t p_t g_k(t),  Q_k = sum_t p_t d2_t g_k(t)
+//     ga_edge = gz PX + gv.(W Q) - PX gv.(W S)          (gradient wrt the exponent a)
+//     gW     += gv (x) S                                 (gradient wrt the projection)
+// Same decomposition as the forward kernel: a unit is an unordered atom pair, its
+// Gaussians are evaluated once per translation for 2 x 16 weight columns
+// (8 heads of i and of j, each with p and p*d2), S and Q accumulate on
+// v_mfma_f32_16x16x4_f32.  A work-group is 8 wavefronts; per round every
+// wavefront owns one unit, then the 8 wavefronts exchange S and Q through LDS
+// and wavefront w does head w for all 8 units: W S and W Q (the forward's
+// projection, twice), the two dot products with gv, and the rank-16 update of
+// that head's D x K block of gW, which stays in registers for the whole kernel
+// and is written once per work-group; a second kernel adds the per-work-group
+// blocks in a fixed order.  No atomics.
+#include "real_enc_pair.h"
+
+namespace {
+
+using namespace cf;
+using namespace cfpair;
+
+constexpr int BRING_CAP = 128;              // translations staged per pass
+constexpr int BRING_SLOTS = BRING_CAP + 16;
+
+template <int NT, bool UNIFORM>
+__global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
+{
+    extern __shared__ __align__(16) float lds[];
+    constexpr int SROW = 16 * NT + 1;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane >> 4;
+    const int c = lane & 15;
+    const int H = p.H, K = p.K, D = p.D;
+    const int64_t *__restrict__ g_pairs = p.pairs;
+    const int64_t *__restrict__ g_edges = p.edges;
+    const int64_t *__restrict__ g_batch = p.batch;
+    const float *__restrict__ g_rpos = p.rpos;
+    const float *__restrict__ g_tvecs = p.tvecs;
+    const float *__restrict__ g_a = p.a_ik;
+    const float *__restrict__ g_rvlen = p.rvlen;
+    const float *__restrict__ g_z = p.z_in;
+    const float *__restrict__ g_gz = p.gz;
+    const float *__restrict__ g_gv = p.gv;
+    float *ring_d2 = lds + wave * (3 * BRING_SLOTS);
+    float *ring_s = ring_d2 + BRING_SLOTS;
+    int *ring_bits = reinterpret_cast<int *>(ring_s + BRING_SLOTS);
+    float *Sbuf = lds + WPB * 3 * BRING_SLOTS;                          // [8 heads][2 dirs][8 units][SROW]
+    float *PXbuf = Sbuf + WPB * 16 * SROW;                              // [8 units][16 cols]
+    int64_t *meta = reinterpret_cast<int64_t *>(PXbuf + WPB * 16);      // [8 units][2]
+
+    float ck[NT];
+#pragma unroll
+    for (int m = 0; m < NT; m++) ck[m] = p.bin_step * (float)(16 * m + c + 1);
+
+    // this wave's head: projection operands and the running block of gW
+    float Wa[4 * NT];
+    float4_t gWacc[NT];
+    int wa_hg = -1;
+
+    const int64_t rounds_per_hg = (p.U + WPB - 1) / WPB;
+    const int64_t rounds = rounds_per_hg * p.head_groups;
+    struct Desc { int64_t e_ij, e_ji, i, j, n; };
+    auto fetch = [&](int64_t rd_) {
+        Desc dsc;
+        const int hg_ = (int)(rd_ / rounds_per_hg);
+        int64_t u_ = (rd_ - (int64_t)hg_ * rounds_per_hg) * WPB + wave;
+        if (rd_ >= rounds || u_ >= p.U) u_ = 0;
+        dsc.e_ij = g_pairs[2 * u_];
+        dsc.e_ji = g_pairs[2 * u_ + 1];
+        dsc.i = g_edges[dsc.e_ij];
+        dsc.j = g_edges[p.E + dsc.e_ij];
+        dsc.n = g_batch[dsc.i];
+        return dsc;
+    };
+    auto flush_gW = [&](int hg_) {
+        // lane (q, j) holds gW[d = 4q + r][bin = 16t + j] of head hg_*8 + wave
+        const int hw = hg_ * 8 + wave;
+        if (p.gW_part && hw < H) {
+            float *dst = p.gW_part + ((int64_t)blockIdx.x * H + hw) * D * K;
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int d = 4 * q + r, k = 16 * t + c;
+                    if (d < D && k < K) dst[d * K + k] = gWacc[t][r];
+                }
+        }
+    };
+    Desc next = fetch(blockIdx.x);
+    for (int64_t rd = blockIdx.x; rd < rounds; rd += gridDim.x) {
+        const int hg = (int)(rd / rounds_per_hg);
+        const int64_t u = (rd - (int64_t)hg * rounds_per_hg) * WPB + wave;
+        const bool unit_on = u < p.U;
+        const Desc cur = next;
+        next = fetch(rd + gridDim.x);
+        if (hg != wa_hg) {
+            if (wa_hg >= 0) flush_gW(wa_hg);
+            const int hw = hg * 8 + wave;
+#pragma unroll
+            for (int s = 0; s < 4 * NT; s++) {
+                const int d = c, k = proj_bin(s, q);
+                Wa[s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
+            }
+#pragma unroll
+            for (int t = 0; t < NT; t++) gWacc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+            wa_hg = hg;
+        }
+        const int64_t e_ij = cur.e_ij, e_ji = cur.e_ji, i = cur.i, j = cur.j, n = cur.n;
+        Cell cell;
+        cell.rx = g_rpos[e_ij * 3 + 0];
+        cell.ry = g_rpos[e_ij * 3 + 1];
+        cell.rz = g_rpos[e_ij * 3 + 2];
+#pragma unroll
+        for (int x = 0; x < 9; x++) cell.t[x] = g_tvecs[n * 9 + x];
+
+        const int h = hg * 8 + (c & 7);
+        const bool col_on = unit_on && h < H && (c < 8 || e_ji != e_ij);
+        const int64_t atom = (c < 8) ? i : j;
+        const int64_t e_col = (c < 8) ? e_ij : e_ji;
+        const float a = col_on ? g_a[atom * H + h] : -1.0f;
+        const float a2 = a * LOG2E;
+        const float z2 = col_on ? g_z[e_col * H + h] * LOG2E : 0.f;
+
+        BoxDims bx;
+        bx.U1 = bx.U2 = bx.U3 = p.lattice_range;
+        int R1 = bx.U1, R2 = bx.U1, R3 = bx.U1;
+        if (!UNIFORM) {
+            float rvl[3] = {g_rvlen[n * 3 + 0], g_rvlen[n * 3 + 1], g_rvlen[n * 3 + 2]};
+            range_rule(a, p.cutoff, rvl, p.lattice_range, p.min_range, R1, R2, R3);
+            if (!col_on) R1 = R2 = R3 = 0;
+            bx.U1 = __builtin_amdgcn_readfirstlane(wave_max_int(R1));
+            bx.U2 = __builtin_amdgcn_readfirstlane(wave_max_int(R2));
+            bx.U3 = __builtin_amdgcn_readfirstlane(wave_max_int(R3));
+        }
+        bx.S3 = 2 * bx.U3 + 1;
+        bx.S2 = 2 * bx.U2 + 1;
+        bx.plane = bx.S2 * bx.S3;
+        bx.T = (2 * bx.U1 + 1) * bx.plane;
+        bx.inv_plane = 1.0f / (float)bx.plane;
+        bx.inv_S3 = 1.0f / (float)bx.S3;
+        const int T = bx.T;
+
+        // p_t <= 2^-40 in every column when a2_weak d2 - z2_floor <= -40
+        const float a2_weak = wave_max(col_on ? a2 : -3.0e38f);
+        const float z2_floor = wave_min(col_on ? z2 : 3.0e38f);
+
+        float4_t accS[NT], accQ[NT];
+#pragma unroll
+        for (int m = 0; m < NT; m++) accS[m] = accQ[m] = float4_t{0.f, 0.f, 0.f, 0.f};
+        float px = 0.f;
+        for (int s0 = 0; s0 < T; s0 += BRING_CAP) {
+            const int cnt = min(BRING_CAP, T - s0);
+            int near_cnt = 0, far_cnt = 0;
+            for (int c0 = 0; c0 < cnt; c0 += WAVE) {
+                const bool valid = c0 + lane < cnt;
+                int n1, n2, n3;
+                decode(bx, valid ? s0 + c0 + lane : 0, n1, n2, n3);
+                const float d2 = dist2(cell, (float)n1, (float)n2, (float)n3);
+                int bits = 0;
+                if (valid) {
+                    if (UNIFORM) {
+                        bits = 0xFFFF;
+                    } else {
+#pragma unroll
+                        for (int x = 0; x < 16; x++) {
+                            int r1 = __builtin_amdgcn_readlane(R1, x);
+                            int r2 = __builtin_amdgcn_readlane(R2, x);
+                            int r3 = __builtin_amdgcn_readlane(R3, x);
+                            if (abs(n1) <= r1 && abs(n2) <= r2 && abs(n3) <= r3) bits |= (1 << x);
+                        }
+                    }
+                }
+                const int colbits = bits;
+                const float s = sqrt_hw(d2) * p.s_scale;
+                const float xb = s * p.inv_bin_step - 1.0f;
+                if (valid) {
+#pragma unroll
+                    for (int m = 0; m < NT; m++)
+                        if (xb >= (float)(16 * m) - p.window && xb <= (float)(16 * m + 15) + p.window)
+                            bits |= (0x10000 << m);
+                }
+                const bool is_near = valid && (bits >> 16) != 0;
+                const bool is_far = valid && !is_near && colbits != 0 && a2_weak * d2 - z2_floor > -40.0f;
+                const unsigned long long near_mask = __ballot(is_near);
+                const unsigned long long far_mask = __ballot(is_far);
+                const unsigned long long below = (1ull << lane) - 1ull;
+                int pos = -1;
+                if (is_near) pos = near_cnt + __popcll(near_mask & below);
+                else if (is_far) pos = BRING_SLOTS - 1 - (far_cnt + __popcll(far_mask & below));
+                if (pos >= 0) {
+                    ring_d2[pos] = d2;
+                    ring_s[pos] = s;
+                    ring_bits[pos] = bits;
+                }
+                near_cnt += __popcll(near_mask);
+                far_cnt += __popcll(far_mask);
+            }
+            if (lane < 12) {
+                const int pos = lane < 8 ? near_cnt + lane : BRING_SLOTS - far_cnt - 1 - (lane - 8);
+                ring_d2[pos] = __builtin_inff();
+                ring_s[pos] = 0.f;
+                ring_bits[pos] = 0;
+            }
+            wave_mem_sync();
+            {
+                const int groups = (near_cnt + 3) >> 2;
+                float d2n = ring_d2[q], sn = ring_s[q];
+                int bitsn = ring_bits[q];
+                for (int g = 0; g < groups; g++) {
+                    const float d2t = d2n, st = sn;
+                    const int bits = bitsn;
+                    const int slot = 4 * (g + 1) + q;
+                    d2n = ring_d2[slot];
+                    sn = ring_s[slot];
+                    bitsn = ring_bits[slot];
+                    const bool on = col_on && ((bits >> c) & 1);
+                    // padding records carry d2 = +inf: keep them out of p*d2
+                    const float w = on ? exp2_hw(a2 * d2t - z2) : 0.f;
+                    const float wd = on ? w * d2t : 0.f;
+                    px += wd;
+#pragma unroll
+                    for (int m = 0; m < NT; m++) {
+                        if (__ballot((bits & (0x10000 << m)) != 0) != 0ull) {
+                            float b = ck[m] - st;
+                            float gm = exp2_hw(-(b * b));
+                            accS[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, w, accS[m], 0, 0, 0);
+                            accQ[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, wd, accQ[m], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            {
+                const int groups = (far_cnt + 3) >> 2;
+                for (int g = 0; g < groups; g++) {
+                    const int slot = BRING_SLOTS - 4 * (g + 1) + q;
+                    const float d2t = ring_d2[slot];
+                    const int bits = ring_bits[slot];
+                    if (col_on && ((bits >> c) & 1)) px += exp2_hw(a2 * d2t - z2) * d2t;
+                }
+            }
+            wave_mem_sync();
+        }
+        px += __shfl_xor(px, 16, WAVE);
+        px += __shfl_xor(px, 32, WAVE);
+
+        // ---- exchange: column (dir, head) of unit `wave` -> row ((head*2 + dir)*8 + wave)
+        const int srow = ((c & 7) * 2 + (c >> 3)) * WPB + wave;
+        if (q == 0) PXbuf[wave * 16 + c] = px;
+        if (lane == 0) {
+            meta[2 * wave + 0] = unit_on ? e_ij : -1;
+            meta[2 * wave + 1] = (unit_on && e_ji != e_ij) ? e_ji : -1;
+        }
+        const int hw = hg * 8 + wave;
+        const int jcol = c, unit_j = jcol & 7, dir_j = jcol >> 3;    // product column j = dir*8 + unit
+        const float *src = Sbuf + ((wave * 2 + dir_j) * WPB + unit_j) * SROW;
+        float dotS = 0.f, dotQ = 0.f;
+        float4_t gv4 = {0.f, 0.f, 0.f, 0.f};
+        int64_t e_out = -1;
+#pragma unroll
+        for (int pass = 0; pass < 2; pass++) {
+            // pass 0 exchanges S (also feeds gW), pass 1 exchanges Q
+            {
+                float *col = Sbuf + srow * SROW;
+#pragma unroll
+                for (int m = 0; m < NT; m++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const float val = pass == 0 ? accS[m][r] : accQ[m][r];
+                        col[16 * m + 4 * q + r] = col_on ? val : 0.f;
+                    }
+            }
+            __syncthreads();
+            if (pass == 0) {
+                e_out = meta[2 * unit_j + dir_j];
+                if (e_out >= 0 && hw < H && g_gv) {
+                    const float *gp = g_gv + (e_out * H + hw) * D + 4 * q;
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (4 * q + r < D) gv4[r] = gp[r];
+                }
+            }
+            float4_t out = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t4 = 0; t4 < NT; t4++) {
+                float sb[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) sb[r] = src[16 * t4 + 4 * q + r];
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    out = __builtin_amdgcn_mfma_f32_16x16x4f32(Wa[4 * t4 + r], sb[r], out, 0, 0, 0);
+            }
+            // lane (q, j): components d = 4q + r of (W S) or (W Q) for column j; dot with gv
+            float dot = out[0] * gv4[0] + out[1] * gv4[1] + out[2] * gv4[2] + out[3] * gv4[3];
+            dot += __shfl_xor(dot, 16, WAVE);
+            dot += __shfl_xor(dot, 32, WAVE);
+            if (pass == 0) {
+                dotS = dot;
+            } else {
+                dotQ = dot;
+                if (q == 0 && e_out >= 0 && hw < H) {
+                    const float PX = PXbuf[unit_j * 16 + dir_j * 8 + wave];
+                    const float gz = g_gz ? g_gz[e_out * H + hw] : 0.f;
+                    p.ga_edge[e_out * H + hw] = PX * gz + (dotQ - PX * dotS);
+                }
+            }
+            if (pass == 0 && p.gW_part) {
+                // gW_h[d][bin] += sum over the 16 columns of gv[col][d] * S[bin][col]
+                // A[i = d][k = col], B[k = col][j = bin]; column 4*s4 + kk
+#pragma unroll
+                for (int s4 = 0; s4 < 4; s4++) {
+                    const int colk = 4 * s4 + q;                    // this lane's reduction index
+                    const int64_t e_k = meta[2 * (colk & 7) + (colk >> 3)];
+                    float av = 0.f;
+                    if (e_k >= 0 && hw < H && g_gv && c < D) av = g_gv[(e_k * H + hw) * D + c];
+                    const float *srck = Sbuf + ((wave * 2 + (colk >> 3)) * WPB + (colk & 7)) * SROW;
+#pragma unroll
+                    for (int t = 0; t < NT; t++)
+                        gWacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, srck[16 * t + c], gWacc[t], 0, 0, 0);
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (wa_hg >= 0) flush_gW(wa_hg);
+}
+
+// gW[x] = sum over work-groups of part[b][x], fixed order.
+__global__ void gw_blocks_reduce_kernel(const float *part, int blocks, int64_t HDK, float *gW)
+{
+    int64_t x = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (x >= HDK) return;
+    float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+    int b = 0;
+    for (; b + 4 <= blocks; b += 4) {
+        acc0 += part[(int64_t)b * HDK + x];
+        acc1 += part[(int64_t)(b + 1) * HDK + x];
+        acc2 += part[(int64_t)(b + 2) * HDK + x];
+        acc3 += part[(int64_t)(b + 3) * HDK + x];
+    }
+    for (; b < blocks; b++) acc0 += part[(int64_t)b * HDK + x];
+    gW[x] = (acc0 + acc1) + (acc2 + acc3);
+}
+
+}  // namespace
+
+namespace cf {
+
+int real_enc_bwd_pairs_blocks(int64_t U, int64_t H)
+{
+    const int64_t rounds = ((U + WPB - 1) / WPB) * ((H + 7) / 8);
+    int64_t blocks = rounds;
+    const int64_t cap = (int64_t)device_cu_count() * 2;
+    if (blocks > cap) blocks = cap;
+    return (int)(blocks < 1 ? 1 : blocks);
+}
+
+// Returns CF_ERR_UNSUPPORTED (no error text) for shapes this kernel does not cover.
+int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,
+                              const int64_t *edges, const int64_t *pairs, int64_t U, const float *z,
+                              const float *gz, const float *gv, int64_t N, int64_t H, int64_t E, int64_t K,
+                              int64_t D, float bin_step, float s_scale, const float *W, const float *rvlen,
+                              float cutoff, int lattice_range, int min_range, float *ga_edge,
+                              float *gW_part, float *gW, hipStream_t st)
+{
+    if (K < 1 || K > 64 || !W || D < 1 || D > 16) return CF_ERR_UNSUPPORTED;
+    PairArgs p{};
+    p.a_ik = a_ik; p.rpos = rpos; p.tvecs = tvecs; p.batch = batch; p.edges = edges; p.pairs = pairs;
+    p.W = W; p.rvlen = rvlen; p.z_in = z; p.gz = gz; p.gv = gv; p.ga_edge = ga_edge; p.gW_part = gW_part;
+    p.N = N; p.E = E; p.U = U; p.W_num = 1;
+    p.H = (int)H; p.K = (int)K; p.D = (int)D;
+    p.head_groups = (int)((H + 7) / 8);
+    p.cutoff = cutoff; p.lattice_range = lattice_range; p.min_range = min_range;
+    p.bin_step = bin_step; p.s_scale = s_scale;
+    p.inv_bin_step = 1.0f / bin_step;
+    p.window = sqrtf(40.0f) / bin_step;
+    const int NT = K <= 16 ? 1 : K <= 32 ? 2 : 4;
+    const bool uniform = cutoff == 0.0f;
+    const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)WPB * 16 * (16 * NT + 1) + WPB * 16) +
+                       sizeof(int64_t) * WPB * 2 + 8;
+    const int blocks = real_enc_bwd_pairs_blocks(U, H);
+#define CF_BPAIR(NTV)                                                                              \
+    do {                                                                                           \
+        if (uniform) real_enc_bwd_pair_kernel<NTV, true><<<blocks, WPB * WAVE, lds, st>>>(p);      \
+        else real_enc_bwd_pair_kernel<NTV, false><<<blocks, WPB * WAVE, lds, st>>>(p);             \
+    } while (0)
+    switch (NT) {
+        case 1: CF_BPAIR(1); break;
+        case 2: CF_BPAIR(2); break;
+        default: CF_BPAIR(4); break;
+    }
+#undef CF_BPAIR
+    if (gW_part && gW) {
+        const int64_t HDK = H * D * K;
+        gw_blocks_reduce_kernel<<<(int)((HDK + 255) / 256), 256, 0, st>>>(gW_part, blocks, HDK, gW);
+    }
+    return CF_OK;
+}
+
+}  // namespace cf

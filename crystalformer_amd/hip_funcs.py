@@ -141,7 +141,8 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         ga_ik, gW_k = ops.real_enc_bwd(
             a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz, gv, ctx.K, ctx.dist_max,
             ctx.wscale, W_k, rvlen_n, ctx.cutoff_radius, ctx.ranges[0], ctx.ranges[1],
-            want_gW=W_k is not None and ctx.needs_input_grad[9])
+            want_gW=W_k is not None and ctx.needs_input_grad[9],
+            pairs_u=_pairs(batch_i, edge_ij_e, tvecs_n, ctx.K))
         return _enc_backward_tail(ga_ik, gW_k, ctx.adaptive_args)
 
 

@@ -177,9 +177,10 @@ def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
                  K: int, dist_max: float, wscale: float, W_k: Optional[Tensor] = None,
                  rvlen_n: Optional[Tensor] = None, cutoff_radius: Optional[float] = None,
                  lattice_range: int = 2, minimum_range: int = 0,
-                 want_gW: bool = True) -> Tuple[Tensor, Optional[Tensor]]:
+                 want_gW: bool = True, pairs_u: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
     dev = require_device(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd,
-                         W_k, rvlen_n)
+                         W_k, rvlen_n, pairs_u)
+    pairs_u = _i64(pairs_u, "pairs_u")
     a_ik, rpos_ij_e, tvecs_n = _f32(a_ik, "a_ik"), _f32(rpos_ij_e, "rpos_ij_e"), _f32(tvecs_n, "tvecs_n")
     batch_i, edge_ij_e, e_start_i = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e"), \
         _i64(e_start_i, "e_start_i")
@@ -210,7 +211,8 @@ def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
             ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i),
             ptr(z_ek), ptr(gz_ek), ptr(gv_ekd if K > 0 else None), N, H, E, B, K, D, float(dist_max),
             float(wscale), ptr(W_k if K > 0 else None), W_num, ptr(rvlen_n), cutoff, int(lattice_range),
-            int(minimum_range), ptr(ws), ws_bytes, ptr(ga), ptr(gW), stream_handle(dev))
+            int(minimum_range), ptr(pairs_u), 0 if pairs_u is None else pairs_u.shape[0], ptr(ws), ws_bytes,
+            ptr(ga), ptr(gW), stream_handle(dev))
     check(rc, "cf_real_enc_bwd")
     return ga, gW
 

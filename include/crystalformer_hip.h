@@ -97,6 +97,9 @@ int64_t cf_real_enc_bwd_workspace(int64_t N, int64_t H, int64_t E, int64_t K, in
  *   gz_ek     (E,H)  gradient of z
  *   gv_ekd    nullable; (E,H,K) when W_k is NULL else (E,H,D)
  *   workspace device scratch of cf_real_enc_bwd_workspace() bytes (256-byte aligned)
+ *   pairs_u   nullable, (U,2) pair list as for cf_real_enc_fwd; with it (and a shared
+ *             W_k, K <= 64, D <= 16) the two directions of a pair are evaluated together
+ *             on the matrix cores
  * Outputs
  *   ga_ik (N,H)
  *   gW_k  nullable; (W_num,H,D,K) — already reduced to W's own shape (the
@@ -109,6 +112,7 @@ int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tvec
                     int64_t K, int64_t D, double dist_max, double wscale,
                     const float *W_k, int64_t W_num, const float *rvlen_n,
                     double cutoff_radius, int lattice_range, int minimum_range,
+                    const int64_t *pairs_u, int64_t U,
                     void *workspace, int64_t workspace_bytes,
                     float *ga_ik, float *gW_k, void *stream);
 
