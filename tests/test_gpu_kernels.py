@@ -14,10 +14,11 @@ from tests.helpers import Problem, assert_close, make_sized_batch, rel_err, to_d
 pytestmark = pytest.mark.gpu
 
 
-def enc_fwd_gpu(dev, p, K, W, cutoff, lr, mr, rvlen=True):
+def enc_fwd_gpu(dev, p, K, W, cutoff, lr, mr, rvlen=True, pairs=False):
     a, rpos, tv, bt, ed, Wd, rv = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, W,
                                          p.rvlen if rvlen else None)
-    return ops.real_enc_fwd(a, rpos, tv, bt, ed, K, p.dist_max, p.wscale, Wd, rv, cutoff, lr, mr)
+    pr = ops.edge_pairs(p.b.sizes.to(dev)) if pairs else None
+    return ops.real_enc_fwd(a, rpos, tv, bt, ed, K, p.dist_max, p.wscale, Wd, rv, cutoff, lr, mr, pairs_u=pr)
 
 
 def enc_fwd_ref(p, K, W, cutoff, lr, mr):
@@ -40,6 +41,92 @@ def test_real_enc_fwd(dev, H, K, D, cutoff, lr, mr):
             assert_close(v, v_ref, "v")
         else:
             assert v is None
+
+
+@pytest.mark.parametrize("cutoff,lr,mr", RULES + [(-3.5, 3, 3)])
+@pytest.mark.parametrize("H,K,D", [(8, 64, 16), (4, 16, 8), (1, 7, 3), (2, 100, 4), (16, 32, 8), (8, 64, 32),
+                                   (8, 48, 20), (8, 64, 64)])
+def test_real_enc_fwd_pair_kernel(dev, H, K, D, cutoff, lr, mr):
+    """Matrix-core path: both directions of an atom pair evaluated together (pair list given)."""
+    p = Problem([1, 3, 9, 2, 17, 1], H=H, K=K, D=D, seed=28)
+    z_ref, v_ref = enc_fwd_ref(p, K, p.W, cutoff, lr, mr)
+    _, s_ref = enc_fwd_ref(p, K, None, cutoff, lr, mr)
+    z, v = enc_fwd_gpu(dev, p, K, p.W, cutoff, lr, mr, pairs=True)
+    assert_close(z, z_ref, "z")
+    assert_close(v, v_ref, "v")
+    z2, s = enc_fwd_gpu(dev, p, K, None, cutoff, lr, mr, pairs=True)
+    assert torch.equal(z2, z) or rel_err(z2, z) < 1e-6
+    assert_close(s, s_ref, "s")
+
+
+def test_real_enc_pair_kernel_large_boxes_and_indexed_projection(dev):
+    """Boxes beyond the staging capacity (several passes per unit) and per-edge / per-atom W."""
+    p = Problem([4, 7], H=8, K=64, D=16, seed=29)
+    p.a = p.a * 0.05                                  # slow decay -> wide adaptive boxes
+    for mr in (0, 4):
+        z, v = enc_fwd_gpu(dev, p, 64, p.W, -3.5, 2, mr, pairs=True)
+        z_ref, v_ref = enc_fwd_ref(p, 64, p.W, -3.5, 2, mr)
+        R = ks.translation_ranges(p.a, p.rvlen, p.b.batch, -3.5, 2, mr)
+        assert int((2 * R.max(dim=1).values + 1).prod(dim=1).max()) > 256
+        assert_close(z, z_ref, "z")
+        assert_close(v, v_ref, "v")
+    for mode in ("edge", "atom"):
+        pm = Problem([3, 4, 1], H=4, K=16, D=8, seed=23, W_mode=mode)
+        z, v = enc_fwd_gpu(dev, pm, 16, pm.W, -3.5, 2, 2, pairs=True)
+        z_ref, v_ref = enc_fwd_ref(pm, 16, pm.W, -3.5, 2, 2)
+        assert_close(z, z_ref, "z")
+        assert_close(v, v_ref, "v")
+
+
+@pytest.mark.parametrize("cutoff,lr,mr", RULES[:3])
+@pytest.mark.parametrize("H,K,D", [(8, 64, 16), (4, 16, 8), (16, 32, 16), (1, 7, 12), (8, 64, 32)])
+def test_real_enc_bwd_pair_kernel(dev, H, K, D, cutoff, lr, mr):
+    p = Problem([1, 3, 9, 2, 14, 1, 1, 1, 1, 20], H=H, K=K, D=D, seed=30)
+    z_ref, v_ref = enc_fwd_ref(p, K, p.W, cutoff, lr, mr)
+    gz, gv = p.randn(p.E, H), p.randn(*v_ref.shape)
+    args = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv)
+    pairs = ops.edge_pairs(p.b.sizes.to(dev))
+    ga, gW = ops.real_enc_bwd(*args, K, p.dist_max, p.wscale, p.W.to(dev), p.rvlen.to(dev), cutoff, lr, mr,
+                              pairs_u=pairs)
+    ga_ref, gW_ref = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv, K,
+                                     p.dist_max, p.wscale, p.W, p.rvlen, cutoff, lr, mr)
+    assert_close(ga, ga_ref, "ga")
+    assert_close(gW, gW_ref, "gW")
+    # without the gradient of W
+    ga2, none = ops.real_enc_bwd(*args, K, p.dist_max, p.wscale, p.W.to(dev), p.rvlen.to(dev), cutoff, lr, mr,
+                                 want_gW=False, pairs_u=pairs)
+    assert none is None and torch.equal(ga2, ga)
+
+
+def test_pair_kernels_are_bit_stable(dev):
+    """No atomics: repeated launches give identical bits, forward and backward."""
+    p = Problem([5, 11, 2, 30], H=8, K=64, D=16, seed=31)
+    pairs = ops.edge_pairs(p.b.sizes.to(dev))
+    a, rpos, tv, bt, ed, W, rv, es = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.W, p.rvlen,
+                                            p.e_start)
+    runs = [ops.real_enc_fwd(a, rpos, tv, bt, ed, 64, p.dist_max, 1.0, W, rv, -3.5, 2, 2, pairs_u=pairs)
+            for _ in range(3)]
+    assert all(torch.equal(r[0], runs[0][0]) and torch.equal(r[1], runs[0][1]) for r in runs)
+    z, v = runs[0]
+    gz, gv = p.randn(p.E, 8).to(dev), p.randn(p.E, 8, 16).to(dev)
+    bruns = [ops.real_enc_bwd(a, rpos, tv, bt, ed, es, z, gz, gv, 64, p.dist_max, 1.0, W, rv, -3.5, 2, 2,
+                              pairs_u=pairs) for _ in range(3)]
+    assert all(torch.equal(r[0], bruns[0][0]) and torch.equal(r[1], bruns[0][1]) for r in bruns)
+
+
+def test_edge_pairs_bit_exact(dev):
+    for sizes in ([1], [3, 1, 4, 1, 5], [64, 1, 33]):
+        b = make_sized_batch(sizes, seed=45)
+        pairs = ops.edge_pairs(b.sizes.to(dev)).cpu()
+        edges = tp.get_edge_index(sizes)
+        ref, off, eoff = [], 0, 0
+        for n in sizes:
+            for i in range(n):
+                for j in range(i, n):
+                    ref.append((eoff + i * n + j, eoff + j * n + i))
+            eoff += n * n
+        assert pairs.dtype == torch.int64 and pairs.tolist() == [list(r) for r in ref]
+        assert torch.equal(edges[0][pairs[:, 0]], edges[1][pairs[:, 1]])
 
 
 def test_real_enc_fwd_matches_torch_path_fixed_cube(dev):
