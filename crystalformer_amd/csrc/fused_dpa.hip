@@ -235,6 +235,121 @@ __global__ __launch_bounds__(256) void fused_dpa_fwd_stream_kernel(DpaArgs p, in
     for (int64_t x = threadIdx.x; x < total; x += blockDim.x) row[x] = exp2_hw((row[x] - mh) * LOG2E) * ih;
 }
 
+// ------------------------------------------------- backward, streaming version
+// Same lane layout as the streaming forward (work-group of 4 wavefronts per atom,
+// lane = (edge slot, head, 4 components)), two kernels, fixed summation order:
+//   query side  per query i over its edge row: gb_ij = go_i p_ij (stored),
+//               gs_ij = sum_d (v_j + b_ij - o_i) gb_ij (stored as gaij),
+//               gq_i = sum_j gs_ij k_j;
+//   key side    per key j over the column (i, j) of the crystal's dense block:
+//               gv_j = sum_i go_i p_ij, gk_j = sum_i gs_ij q_i.
+__global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs p, int DV4, int LPE)
+{
+    __shared__ float part[DPA_WPQ][WAVE][4];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t i = blockIdx.x;
+    const int H = p.H;
+    const int HD4 = LPE;
+    const int ES = WAVE / LPE;
+    const int es = lane / LPE;
+    const int piece = lane - es * LPE;
+    const int h = piece / DV4;
+    const bool lead = (piece - h * DV4) == 0;
+    const int64_t e0 = p.e_start[i], e1 = p.e_start[i + 1];
+    const int64_t *dst = p.edges + p.E;
+    const float4_v *key4 = reinterpret_cast<const float4_v *>(p.key);
+    const float4_v *val4 = reinterpret_cast<const float4_v *>(p.val);
+    const float4_v *bij4 = reinterpret_cast<const float4_v *>(p.bij);
+    float4_v *gb4 = reinterpret_cast<float4_v *>(p.gbij);
+    const float4_v go4 = reinterpret_cast<const float4_v *>(p.gout)[i * HD4 + piece];
+    const float4_v o4 = reinterpret_cast<const float4_v *>(p.out_in)[i * HD4 + piece];
+    float4_v gq = {0.f, 0.f, 0.f, 0.f};
+    const int stride = DPA_WPQ * ES;
+    for (int64_t e = e0 + wave * ES + es; e < e1; e += stride) {
+        const int64_t j = dst[e];
+        const float pr = p.prob_in[e * H + h];
+        const float4_v k4 = key4[j * HD4 + piece];
+        float4_v m4 = val4[j * HD4 + piece];
+        if (bij4) m4 += bij4[e * HD4 + piece];
+        const float4_v t4 = go4 * pr;
+        if (gb4) gb4[e * HD4 + piece] = t4;
+        m4 -= o4;
+        float gs = m4.x * t4.x + m4.y * t4.y + m4.z * t4.z + m4.w * t4.w;
+        for (int off = DV4 >> 1; off > 0; off >>= 1) gs += __shfl_xor(gs, off, WAVE);
+        if (lead) p.gaij[e * H + h] = gs;
+        gq += k4 * gs;
+    }
+    for (int off = LPE; off < WAVE; off <<= 1) {
+        gq.x += __shfl_xor(gq.x, off, WAVE);
+        gq.y += __shfl_xor(gq.y, off, WAVE);
+        gq.z += __shfl_xor(gq.z, off, WAVE);
+        gq.w += __shfl_xor(gq.w, off, WAVE);
+    }
+    if (es == 0) {
+        float *d = part[wave][piece];
+        d[0] = gq.x; d[1] = gq.y; d[2] = gq.z; d[3] = gq.w;
+    }
+    __syncthreads();
+    if (wave == 0 && es == 0) {
+        for (int w = 1; w < DPA_WPQ; w++) {
+            const float *s = part[w][piece];
+            gq += float4_v{s[0], s[1], s[2], s[3]};
+        }
+        reinterpret_cast<float4_v *>(p.gque)[i * HD4 + piece] = gq;
+    }
+}
+
+__global__ __launch_bounds__(256) void fused_dpa_bwd_key_stream_kernel(DpaArgs p, int DV4, int LPE)
+{
+    __shared__ float part[DPA_WPQ][WAVE][8];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t j = blockIdx.x;
+    const int H = p.H;
+    const int HD4 = LPE;
+    const int ES = WAVE / LPE;
+    const int es = lane / LPE;
+    const int piece = lane - es * LPE;
+    const int h = piece / DV4;
+    const int64_t b = p.batch[j];
+    const int64_t ab = p.atom_start[b];
+    const int64_t n = p.atom_start[b + 1] - ab;
+    const int64_t eb = p.edge_start[b] + (j - ab);
+    const float4_v *que4 = reinterpret_cast<const float4_v *>(p.que);
+    const float4_v *go4 = reinterpret_cast<const float4_v *>(p.gout);
+    float4_v gv = {0.f, 0.f, 0.f, 0.f}, gk = {0.f, 0.f, 0.f, 0.f};
+    const int stride = DPA_WPQ * ES;
+    for (int64_t il = wave * ES + es; il < n; il += stride) {
+        const int64_t e = eb + il * n;
+        const float pr = p.prob_in[e * H + h];
+        const float gs = p.gaij[e * H + h];
+        gv += go4[(ab + il) * HD4 + piece] * pr;
+        gk += que4[(ab + il) * HD4 + piece] * gs;
+    }
+    for (int off = LPE; off < WAVE; off <<= 1) {
+        gv.x += __shfl_xor(gv.x, off, WAVE); gv.y += __shfl_xor(gv.y, off, WAVE);
+        gv.z += __shfl_xor(gv.z, off, WAVE); gv.w += __shfl_xor(gv.w, off, WAVE);
+        gk.x += __shfl_xor(gk.x, off, WAVE); gk.y += __shfl_xor(gk.y, off, WAVE);
+        gk.z += __shfl_xor(gk.z, off, WAVE); gk.w += __shfl_xor(gk.w, off, WAVE);
+    }
+    if (es == 0) {
+        float *d = part[wave][piece];
+        d[0] = gv.x; d[1] = gv.y; d[2] = gv.z; d[3] = gv.w;
+        d[4] = gk.x; d[5] = gk.y; d[6] = gk.z; d[7] = gk.w;
+    }
+    __syncthreads();
+    if (wave == 0 && es == 0) {
+        for (int w = 1; w < DPA_WPQ; w++) {
+            const float *s = part[w][piece];
+            gv += float4_v{s[0], s[1], s[2], s[3]};
+            gk += float4_v{s[4], s[5], s[6], s[7]};
+        }
+        reinterpret_cast<float4_v *>(p.gval)[j * HD4 + piece] = gv;
+        reinterpret_cast<float4_v *>(p.gkey)[j * HD4 + piece] = gk;
+    }
+}
+
 // ----------------------------------------------------------------- backward
 // rows: per query i, lane = (head, value component); Dv is a power of two <= 64
 // so that the lanes of one head form an aligned group.
@@ -409,6 +524,17 @@ extern "C" int cf_fused_dpa_bwd(const float *que, const float *key, const float 
     p.gque = gque; p.gkey = gkey; p.gval = gval; p.gaij = gaij; p.gbij = gbij;
     p.N = N; p.E = E; p.H = (int)H; p.Dk = (int)Dk; p.Dv = (int)Dv;
     hipStream_t st = (hipStream_t)stream;
+    {
+        const int64_t dv4 = Dv / 4, lpe = H * dv4;
+        const bool pow2 = (dv4 & (dv4 - 1)) == 0 && (H & (H - 1)) == 0;
+        if (Dk == Dv && Dv % 4 == 0 && pow2 && lpe >= 1 && lpe <= 64) {
+            fused_dpa_bwd_query_stream_kernel<<<(int)N, DPA_WPQ * WAVE, 0, st>>>(p, (int)dv4, (int)lpe);
+            CF_CHECK_LAUNCH("cf_fused_dpa_bwd: query side");
+            fused_dpa_bwd_key_stream_kernel<<<(int)N, DPA_WPQ * WAVE, 0, st>>>(p, (int)dv4, (int)lpe);
+            CF_CHECK_LAUNCH("cf_fused_dpa_bwd: key side");
+            return CF_OK;
+        }
+    }
     const int wpb = 4;
     const int grid = (int)((N + wpb - 1) / wpb);
     fused_dpa_bwd_rows_kernel<<<grid, wpb * WAVE, 0, st>>>(p);
