@@ -20,7 +20,7 @@ from torch.nn import Module, Parameter
 from torch.nn.init import constant_, normal_, xavier_uniform_
 
 from . import global_config as config
-from .hip_funcs import (FusedDotProductAttentionCUDA, RealPeriodicEncodingFuncCUDA,
+from .hip_funcs import (FusedDotProductAttentionCUDA, GaussianExponentsHIP, RealPeriodicEncodingFuncCUDA,
                         RealPeriodicEncodingWithProjFuncCUDA)
 from .params import LatticeformerParams
 
@@ -70,6 +70,16 @@ def gaussian_exponents(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, ga
                 gauss_scale.copy_(torch.stack([scale, shift]))
     rho = make_positive_func(params.positive_func)(alpha, params.gauss_lb_real)
     return rho * (-0.5 * params.scale_real ** -2)
+
+
+def fused_exponents_spec(params: LatticeformerParams):
+    """(name, beta) when the Gaussian-exponent kernel serves this configuration, else None."""
+    if not params.gauss_state.startswith("q"):
+        return None
+    name, _, beta = params.positive_func.partition("=")
+    if name not in ("elu", "abs", "exp"):
+        return None
+    return name, (float(beta) if beta else 1.0)
 
 
 def conditional_projection(proj: Tensor, onehot: Tensor, edges: Tensor, mode: str) -> Tensor:
@@ -199,12 +209,19 @@ class CrystalformerMultiheadAttentionCUDA(Module):
         k = F.linear(key, self.k_proj_weight, b_k).contiguous().view(key.shape[0], H, kd // H)
         v = F.linear(value, self.v_proj_weight, b_v).contiguous().view(value.shape[0], H, vd // H)
 
-        bias = values = None
+        bias = values = qs = None
         if P.domain == "real":
             proj = self.pe_dist_proj
             if proj is not None and P.value_pe_condproj != "no":
                 proj = conditional_projection(proj, onehot, edges, P.value_pe_condproj)
-            a = gaussian_exponents(q, query, self.lattice_pos_weights, self.gauss_scale, P, self.training)
+            spec = fused_exponents_spec(P) if q.is_cuda else None
+            if spec is not None:
+                # alpha, its normalisation, the positive map and the query scaling in two launches
+                a, qs = GaussianExponentsHIP.apply(
+                    q, self.lattice_pos_weights, self.gauss_scale, P.normalize_gauss, self.training, spec[0],
+                    spec[1], P.gauss_lb_real, -0.5 * P.scale_real ** -2, 1.0 / math.sqrt(q.shape[-1]))
+            else:
+                a = gaussian_exponents(q, query, self.lattice_pos_weights, self.gauss_scale, P, self.training)
             dist_max = P.value_pe_dist_max
             if dist_max < 0:
                 dist_max = (-dist_max) * P.scale_real
@@ -227,7 +244,8 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             raise NotImplementedError("norm_func_mode != 0 is not served by the HIP path")
         if self.training and self.dropout > 0.0:
             raise NotImplementedError("attention dropout is not served by the HIP path")
-        qs = q / math.sqrt(q.shape[-1])
+        if qs is None:
+            qs = q / math.sqrt(q.shape[-1])
         if config.REPRODUCIBLITY_STATE >= 2 and batch_q is batch_kv:
             attn = FusedDotProductAttentionCUDA.apply(qs, k, v, bias, values, batch_q, edges)
         else:

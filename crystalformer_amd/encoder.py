@@ -31,6 +31,15 @@ def det_3x3(m: Tensor) -> Tensor:
             - m[:, 0, 0] * m[:, 1, 2] * m[:, 2, 1] - m[:, 0, 1] * m[:, 1, 0] * m[:, 2, 2])
 
 
+def _sizes_on_device(sizes, batch: Tensor, num_crystals: int, device) -> Tensor:
+    if sizes is None:
+        sizes = torch.zeros(num_crystals, dtype=torch.long, device=device)
+        sizes.scatter_add_(0, batch, torch.ones_like(batch))
+    if not torch.is_tensor(sizes):
+        sizes = torch.tensor(sizes, dtype=torch.long, device=device)
+    return sizes.to(device=device, dtype=torch.long)
+
+
 def compute_lattice_distances_for_cuda(pos: Tensor, batch: Tensor, trans_vec: Tensor, sizes, lattice_range,
                                        cutoff_radius=0, output_real=False, output_reci=False):
     """Geometry prologue of the kernel path
@@ -41,18 +50,8 @@ def compute_lattice_distances_for_cuda(pos: Tensor, batch: Tensor, trans_vec: Te
     reciprocal-space kernel here)."""
     if output_reci:
         raise NotImplementedError("reciprocal-space outputs are not served by the HIP path")
-    if sizes is None:
-        sizes = torch.zeros(trans_vec.shape[0], dtype=torch.long, device=pos.device)
-        sizes.scatter_add_(0, batch, torch.ones_like(batch))
-    if not torch.is_tensor(sizes):
-        sizes = torch.tensor(sizes, dtype=torch.long, device=pos.device)
-    sizes = sizes.to(device=pos.device, dtype=torch.long)
-    vcell = det_3x3(trans_vec).contiguous()
-    recip_vec = (torch.stack([
-        torch.cross(trans_vec[:, 1], trans_vec[:, 2], dim=1),
-        torch.cross(trans_vec[:, 2], trans_vec[:, 0], dim=1),
-        torch.cross(trans_vec[:, 0], trans_vec[:, 1], dim=1),
-    ], dim=1) * (2.0 * math.pi / vcell[:, None, None])).contiguous()
+    sizes = _sizes_on_device(sizes, batch, trans_vec.shape[0], pos.device)
+    vcell, recip_vec, _ = ops.lattice_geometry(trans_vec)
     edges, pos_ij = ops.edge_index(sizes, pos.contiguous())
     return pos_ij, None, None, recip_vec, vcell, edges
 
@@ -157,10 +156,12 @@ class CrystalformerEncoderCUDA(Module):
             raise RuntimeError("the feature number of src and tgt must be equal to d_model")
         batch = batch - batch[0]
         P = self.lattice_params
-        pos_ij, dist2_min, kr_base, rvecs, vcell, edges = compute_lattice_distances_for_cuda(
-            pos, batch, trans, sizes, P.lattice_range, -1, output_real=True, output_reci=False)
-        # every block needs only the lengths of the reciprocal vectors: take the norm once
-        rvlen = torch.norm(rvecs, 2, dim=-1).contiguous()
+        # geometry prologue of compute_lattice_distances_for_cuda, plus the lengths of the
+        # reciprocal vectors (all a block needs of them), in two launches
+        sizes = _sizes_on_device(sizes, batch, trans.shape[0], pos.device)
+        vcell, _, rvlen = ops.lattice_geometry(trans)
+        edges, pos_ij = ops.edge_index(sizes, pos.contiguous())
+        dist2_min = kr_base = None
         output = src
         for layer in self.layers:
             output = layer(output, batch, edges, pos_ij, dist2_min, trans, kr_base, rvlen, vcell, onehot)

@@ -226,6 +226,52 @@ class FusedDotProductAttentionCUDA(torch.autograd.Function):
         return gque, gkey, gval, (gaij if ctx.has_aij else None), gbij, None, None
 
 
+class GaussianExponentsHIP(torch.autograd.Function):
+    """(a, q_scaled) from the per-head query: a = coef * rho(normalised <q, w>),
+    q_scaled = q * q_scale.  The normalisation statistics are constants of the
+    backward pass, as in the reference, which detaches them
+    (models/indexed_lattice_multi_head_attention_cuda.py:700-712)."""
+
+    @staticmethod
+    def forward(ctx, q_ihd, w_hd, gauss_scale, normalize, update_stats, positive_func, beta, lower_bound,
+                coef, q_scale):
+        q_ihd = q_ihd.contiguous().detach()
+        w_hd = w_hd.contiguous().detach()
+        need_grad = any(ctx.needs_input_grad[:2])
+        a, qs, alpha_n, used = ops.gauss_exponents(q_ihd, w_hd, gauss_scale, normalize, update_stats,
+                                                   positive_func, beta, lower_bound, coef, q_scale,
+                                                   want_alpha=need_grad)
+        if need_grad:
+            ctx.save_for_backward(q_ihd, w_hd, alpha_n, used)
+        ctx.conf = (positive_func, beta, lower_bound, coef, q_scale)
+        return a, qs
+
+    @staticmethod
+    def backward(ctx, ga, gqs):
+        q_ihd, w_hd, alpha_n, used = ctx.saved_tensors
+        func, beta, lb, coef, q_scale = ctx.conf
+        n, h, d = q_ihd.shape
+        if func == "elu":
+            x = alpha_n * (beta / (1.0 - lb))
+            slope = torch.where(x > 0, torch.ones_like(x), torch.exp(x)) * beta
+        elif func == "abs":
+            slope = torch.sign(alpha_n) * (1.0 - lb)
+        else:
+            slope = torch.exp(alpha_n * (beta / (1.0 - lb))) * beta
+        g_alpha = ga * slope * coef
+        if used is not None:
+            g_alpha = g_alpha * used[0]
+        w = w_hd.reshape(1, h, d)
+        gq = gw = None
+        if ctx.needs_input_grad[0]:
+            gq = g_alpha[..., None] * w
+            if gqs is not None:
+                gq = gq + gqs * q_scale
+        if ctx.needs_input_grad[1]:
+            gw = (g_alpha[..., None] * q_ihd).sum(0).reshape(w_hd.shape)
+        return gq, gw, None, None, None, None, None, None, None, None
+
+
 class IrregularMeanCUDA(torch.autograd.Function):
     """Per-crystal mean over atoms with a fixed summation order."""
 
@@ -235,7 +281,10 @@ class IrregularMeanCUDA(torch.autograd.Function):
             B = int(batch_i.max().item()) + 1
             sizes = torch.zeros(B, dtype=torch.long, device=x_ik.device)
             sizes.scatter_add_(0, batch_i, torch.ones_like(batch_i))
-        start_n = torch.constant_pad_nd(torch.cumsum(sizes, 0), (1, 0)).contiguous()
+        sig, start_n = ops._cache_lookup("mean_start", sizes)
+        if start_n is None:
+            start_n = ops._cache_store(
+                sig, (sizes,), torch.constant_pad_nd(torch.cumsum(sizes, 0), (1, 0)).contiguous())
         o_nk = ops.irregular_mean_fwd(x_ik.contiguous().detach(), start_n)
         ctx.save_for_backward(batch_i.contiguous(), start_n)
         return o_nk

@@ -21,6 +21,7 @@ CSRC_DIR = os.path.join(_PKG_DIR, "csrc")
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
 _dbl = ctypes.c_double
+_f32 = ctypes.c_float
 _ptr = ctypes.c_void_p
 
 # name -> (restype, argtypes); mirrors include/crystalformer_hip.h
@@ -41,6 +42,10 @@ SIGNATURES = {
     "cf_minimum_distance": (_int, [_ptr] * 4 + [_i64, _ptr, _dbl, _int, _int, _ptr, _ptr]),
     "cf_edge_index": (_int, [_ptr, _ptr, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "cf_edge_pairs": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _ptr, _ptr]),
+    "cf_lattice_geometry": (_int, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "cf_gauss_exponents_workspace": (_i64, [_i64, _i64]),
+    "cf_gauss_exponents": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _int, _int, _f32, _f32, _f32, _f32,
+                                  _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -404,3 +404,64 @@ def cached_crystal_offsets(batch_i: Tensor) -> Tuple[Tensor, Tensor]:
     if hit is not None:
         return hit
     return _cache_store(sig, (batch_i,), crystal_offsets(batch_i))
+
+
+def lattice_geometry(trans_n: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+    """(vcell (B), recip (B,3,3), rvlen (B,3)) of the lattices ``trans_n`` (B,3,3)
+    in one launch (models/indexed_latticeformer_encoder.py:34-44, 206-212)."""
+    dev = require_device(trans_n)
+    trans_n = _f32(trans_n, "trans_n")
+    if trans_n.dim() != 3 or trans_n.shape[1:] != (3, 3):
+        raise _lib.CrystalformerHipError(f"trans_n must be (B,3,3), got {tuple(trans_n.shape)}")
+    B = trans_n.shape[0]
+    vcell = torch.empty(B, dtype=torch.float32, device=dev)
+    recip = torch.empty((B, 3, 3), dtype=torch.float32, device=dev)
+    rvlen = torch.empty((B, 3), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_lattice_geometry(ptr(trans_n), B, ptr(vcell), ptr(recip), ptr(rvlen),
+                                             stream_handle(dev))
+    check(rc, "cf_lattice_geometry")
+    return vcell, recip, rvlen
+
+
+POSITIVE_FUNCS = {"elu": 0, "abs": 1, "exp": 2}
+
+
+def gauss_exponents(q_ihd: Tensor, w_hd: Tensor, gauss_scale: Optional[Tensor], normalize: bool,
+                    update_stats: bool, positive_func: str, beta: float, lower_bound: float, coef: float,
+                    q_scale: Optional[float] = None,
+                    want_alpha: bool = False) -> Tuple[Tensor, Optional[Tensor], Optional[Tensor], Optional[Tensor]]:
+    """a[i,h] = coef * rho(normalised <q[i,h], w[h]>), the scaled query and
+    (optionally) the normalised alpha, in two launches
+    (models/indexed_lattice_multi_head_attention_cuda.py:636-722).
+    ``gauss_scale`` (2,) is read, and written in place when ``update_stats``.
+    Returns ``(a, q_scaled, alpha_n, used)``; ``used`` is the (scale, shift) pair
+    applied (None without normalisation)."""
+    dev = require_device(q_ihd, w_hd, gauss_scale)
+    q_ihd = _f32(q_ihd, "q_ihd")
+    w_hd = _f32(w_hd, "w_hd")
+    if q_ihd.dim() != 3:
+        raise _lib.CrystalformerHipError("q_ihd must be (N,H,D)")
+    N, H, D = q_ihd.shape
+    if w_hd.numel() != H * D:
+        raise _lib.CrystalformerHipError(f"w_hd has {w_hd.numel()} elements, expected H*D = {H * D}")
+    if positive_func not in POSITIVE_FUNCS:
+        raise _lib.CrystalformerHipError(f"positive map {positive_func!r} has no kernel")
+    if normalize:
+        if gauss_scale is None or gauss_scale.numel() != 2 or gauss_scale.dtype != torch.float32 \
+                or not gauss_scale.is_contiguous():
+            raise _lib.CrystalformerHipError("gauss_scale must be a contiguous float32 tensor of 2 elements")
+    lib = _lib.load()
+    a = torch.empty((N, H), dtype=torch.float32, device=dev)
+    qs = torch.empty_like(q_ihd) if q_scale is not None else None
+    alpha_n = torch.empty((N, H), dtype=torch.float32, device=dev) if want_alpha else None
+    ws_bytes = int(lib.cf_gauss_exponents_workspace(N, H)) if normalize else 0
+    ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=dev) if normalize else None
+    with torch.cuda.device(dev):
+        rc = lib.cf_gauss_exponents(ptr(q_ihd), ptr(w_hd), ptr(gauss_scale) if normalize else None, N, H, D,
+                                    int(bool(normalize)), int(bool(update_stats)),
+                                    POSITIVE_FUNCS[positive_func], float(beta), float(lower_bound), float(coef),
+                                    float(q_scale if q_scale is not None else 1.0), ptr(ws), ws_bytes,
+                                    ptr(alpha_n), ptr(a), ptr(qs), stream_handle(dev))
+    check(rc, "cf_gauss_exponents")
+    return a, qs, alpha_n, (ws[-4:-2] if normalize else None)

@@ -219,6 +219,44 @@ int cf_edge_pairs(const int64_t *atom_start_n, const int64_t *edge_start_n,
                   const int64_t *unit_start_n, int64_t B, int64_t E, int64_t *pairs_u,
                   void *stream);
 
+/*
+ * Cell volume, reciprocal lattice vectors and their lengths, one launch:
+ *   vcell_n = det(trans_n)            (term order of models/indexed_latticeformer_encoder.py:34-44)
+ *   recip_n = 2 pi (a2 x a3, a3 x a1, a1 x a2) / vcell_n      (models/indexed_latticeformer_encoder.py:206-212)
+ *   rvlen_n = row norms of recip_n    (models/indexed_lattice_multi_head_attention_cuda.py:879, torch.norm)
+ * Replaces the ~25 elementwise launches those expressions take.
+ *   trans_n (B,3,3); outputs vcell_n (B), recip_n (B,3,3), rvlen_n (B,3), each nullable.
+ */
+int cf_lattice_geometry(const float *trans_n, int64_t B, float *vcell_n, float *recip_n,
+                        float *rvlen_n, void *stream);
+
+/*
+ * Gaussian exponents of the periodic encoding from the per-head query
+ * (models/indexed_lattice_multi_head_attention_cuda.py:636-722, gauss_state "q"):
+ *   alpha[i,h] = sum_d q[i,h,d] w[h,d]
+ *   normalize:  alpha = (alpha + shift) * scale, with (scale, shift) =
+ *               gauss_scale when gauss_scale[0] > 0, else (1/std, -mean) of
+ *               alpha over the whole batch (unbiased std); update_stats
+ *               stores the pair used back into gauss_scale
+ *   a[i,h]     = coef * rho(alpha),   coef = -1 / (2 r0^2)
+ *   rho        : 0 elu  (1-lb) elu(x beta/(1-lb)) + 1
+ *                1 abs  (1-lb) |x| + lb
+ *                2 exp  (1-lb) exp(x beta/(1-lb)) + lb
+ *                (models/indexed_lattice_multi_head_attention_cuda.py:675-692)
+ *   q_scaled   = q * q_scale (nullable), the query the attention consumes
+ *   alpha_n    = normalised alpha (nullable), what a backward pass needs
+ * Replaces ~14 elementwise / reduction launches per attention block.  Two
+ * launches, fixed summation order.
+ *   workspace: cf_gauss_exponents_workspace(N,H) bytes when normalize != 0; on
+ *              return floats [-4], [-3] of it hold the (scale, shift) pair used
+ */
+int64_t cf_gauss_exponents_workspace(int64_t N, int64_t H);
+int cf_gauss_exponents(const float *q_ihd, const float *w_hd, float *gauss_scale, int64_t N, int64_t H,
+                       int64_t D, int normalize, int update_stats, int positive_func, float beta,
+                       float lower_bound, float coef, float q_scale, void *workspace,
+                       int64_t workspace_bytes, float *alpha_n, float *a_ih, float *q_scaled,
+                       void *stream);
+
 #ifdef __cplusplus
 }
 #endif

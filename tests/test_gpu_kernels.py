@@ -313,3 +313,79 @@ def test_errors_surface_as_exceptions(dev):
     with pytest.raises(lib.CrystalformerHipError):
         ops.real_enc_fwd(p.a.to(dev), p.rpos.to(dev).double(), p.b.trans_vec.to(dev), p.b.batch.to(dev),
                          p.edges.to(dev), 64, 14.0, 1.0, p.W.to(dev))
+
+
+def test_lattice_geometry(dev):
+    """Cell volume bit-exact with the un-contracted elementwise expression; reciprocal
+    vectors and their lengths to float32 rounding."""
+    g = torch.Generator().manual_seed(5)
+    trans = torch.randn(257, 3, 3, generator=g) * 4 + torch.eye(3) * 6
+    vcell, recip, rvlen = ops.lattice_geometry(trans.to(dev))
+    rec_ref, v_ref = tp.reciprocal_vectors(trans)
+    assert torch.equal(vcell.cpu(), v_ref)
+    assert_close(recip, rec_ref, "recip", rtol=1e-6)
+    assert_close(rvlen, rec_ref.norm(dim=-1), "rvlen", rtol=1e-6)
+    # closed form: rows of recip are dual to the lattice rows, b_r . a_c = 2 pi delta_rc
+    dual = torch.einsum("brk,bck->brc", recip.cpu().double(), trans.double())
+    assert (dual - 2 * math.pi * torch.eye(3, dtype=torch.float64)).abs().max() < 1e-4
+
+
+@pytest.mark.parametrize("N,H,D", [(1900, 8, 16), (3, 1, 5), (57000, 8, 16), (33, 16, 8)])
+@pytest.mark.parametrize("stored", [False, True])
+def test_gauss_exponents(dev, N, H, D, stored):
+    g = torch.Generator().manual_seed(N + H)
+    q = torch.randn(N, H, D, generator=g) * 1.7 + 0.3
+    w = torch.randn(H * D, generator=g) * D ** -0.5
+    gs = torch.tensor([1.3, -0.2]) if stored else torch.zeros(2)
+    lb, beta, r0 = 0.5, 0.1, 1.4
+    gs_ref = gs.clone()
+    a_ref = tp.gaussian_exponents(q, w, gs_ref, True, True, lb, beta, r0)
+    gs_dev = gs.to(dev)
+    a, qs, alpha_n, used = ops.gauss_exponents(q.to(dev), w.to(dev), gs_dev, True, True, "elu", beta, lb,
+                                               -0.5 * r0 ** -2, 0.25, want_alpha=True)
+    assert_close(a, a_ref, "a")
+    assert torch.equal(qs.cpu(), q * 0.25)
+    assert_close(gs_dev, gs_ref, "stored statistics")           # written by the training call
+    assert_close(used, gs_ref, "statistics used")
+    # second call reads the stored pair, inference mode leaves it alone
+    before = gs_dev.clone()
+    a2, _, _, _ = ops.gauss_exponents(q.to(dev), w.to(dev), gs_dev, True, False, "elu", beta, lb,
+                                      -0.5 * r0 ** -2, None)
+    assert torch.equal(gs_dev, before)
+    assert_close(a2, a_ref, "a from stored statistics")
+    # normalised alpha has zero mean / unit std when the batch statistics were used
+    if not stored:
+        assert abs(float(alpha_n.double().mean())) < 1e-4 and abs(float(alpha_n.double().std()) - 1) < 1e-4
+
+
+@pytest.mark.parametrize("func", ["elu", "abs", "exp"])
+def test_gauss_exponents_positive_maps_and_plain_mode(dev, func):
+    from crystalformer_amd.attention import make_positive_func
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(40, 4, 12, generator=g)
+    w = torch.randn(4, 12, generator=g) * 0.3
+    spec = func if func == "abs" else func + "=0.3"
+    alpha = (q * w[None]).sum(-1)
+    ref = make_positive_func(spec)(alpha, 0.4) * -0.2
+    a, qs, _, used = ops.gauss_exponents(q.to(dev), w.to(dev), None, False, False, func, 0.3, 0.4, -0.2)
+    assert qs is None and used is None
+    assert_close(a, ref, "a")
+
+
+def test_gauss_exponents_autograd(dev):
+    from crystalformer_amd.hip_funcs import GaussianExponentsHIP
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(50, 8, 16, generator=g)
+    w = torch.randn(128, generator=g) * 0.25
+    ga = torch.randn(50, 8, generator=g)
+    gqs = torch.randn(50, 8, 16, generator=g)
+    qr, wr = q.clone().requires_grad_(), w.clone().requires_grad_()
+    a_ref = tp.gaussian_exponents(qr, wr, torch.zeros(2), False, True, 0.5, 0.1, 1.4)
+    ((a_ref * ga).sum() + (qr * 0.25 * gqs).sum()).backward()
+    qd, wd = q.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    a, qs = GaussianExponentsHIP.apply(qd, wd, torch.zeros(2, device=dev), True, False, "elu", 0.1, 0.5,
+                                       -0.5 * 1.4 ** -2, 0.25)
+    ((a * ga.to(dev)).sum() + (qs * gqs.to(dev)).sum()).backward()
+    assert_close(a, a_ref.detach(), "a")
+    assert_close(qd.grad, qr.grad, "gq")
+    assert_close(wd.grad, wr.grad, "gw")

@@ -143,7 +143,7 @@ def test_model_matches_reference_golden_training_step(dev, gold, name, over):
     loss = torch.nn.functional.l1_loss(y.squeeze(-1), data.y)
     loss.backward()
     assert_close(y, gold[f"{name}.train.y"], "y")
-    assert abs(float(loss) - float(gold[f"{name}.train.loss"])) < 1e-6
+    assert abs(float(loss.detach()) - float(gold[f"{name}.train.loss"])) < 1e-6
     params = dict(model.named_parameters())
     for k, g in gold[f"{name}.train.grads"].items():
         assert_close(params[k].grad, g, f"grad {k}", rtol=2e-5)
