@@ -57,8 +57,6 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
     const int H = p.H, K = p.K, D = p.D;
     // read-only inputs: plain restrict pointers let per-unit descriptors use scalar loads
     const int64_t *__restrict__ g_pairs = p.pairs;
-    const int64_t *__restrict__ g_edges = p.edges;
-    const int64_t *__restrict__ g_batch = p.batch;
     const float *__restrict__ g_rpos = p.rpos;
     const float *__restrict__ g_tvecs = p.tvecs;
     const float *__restrict__ g_a = p.a_ik;
@@ -80,27 +78,38 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
 
     const int64_t rounds_per_hg = (p.U + WPB - 1) / WPB;
     const int64_t rounds = rounds_per_hg * p.head_groups;
-    // unit descriptor of the coming round, fetched one round ahead
-    struct Desc { int64_t e_ij, e_ji, i, j, n; };
-    auto fetch = [&](int64_t rd_) {
-        Desc dsc;
-        const int hg_ = (int)(rd_ / rounds_per_hg);
-        int64_t u_ = (rd_ - (int64_t)hg_ * rounds_per_hg) * WPB + wave;
-        if (rd_ >= rounds || u_ >= p.U) u_ = 0;
-        dsc.e_ij = g_pairs[2 * u_];
-        dsc.e_ji = g_pairs[2 * u_ + 1];
-        dsc.i = g_edges[dsc.e_ij];
-        dsc.j = g_edges[p.E + dsc.e_ij];
-        dsc.n = g_batch[dsc.i];
-        return dsc;
+    // unit of round rd_ for this wave (0 when the round or the unit does not exist: loads stay valid)
+    auto unit_of = [&](int64_t rd_) -> int64_t {
+        const int64_t hg_ = rd_ / rounds_per_hg;
+        const int64_t u_ = (rd_ - hg_ * rounds_per_hg) * WPB + wave;
+        return (rd_ < rounds && u_ < p.U) ? u_ : 0;
     };
-    Desc next = fetch(blockIdx.x);
-    for (int64_t rd = blockIdx.x; rd < rounds; rd += gridDim.x) {
+    // exponent of column c of a unit in the head group of round rd_
+    auto load_a = [&](const UnitIds &d, int64_t rd_) -> float {
+        const int h_ = min((int)(rd_ / rounds_per_hg) * 8 + (c & 7), H - 1);
+        return g_a[((c < 8) ? d.i : d.j) * H + h_];
+    };
+    const int64_t stride = gridDim.x;
+    // fill the descriptor pipeline: current round complete, next round's ids known
+    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x), lane));
+    float a_cur;
+    UnitGeom geo;
+    UnitIds ids_next;
+    {
+        const float gv0 = load_unit_geom(ids, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
+        a_cur = load_a(ids, blockIdx.x);
+        const int64_t dv1 = load_unit_ids(g_pairs, unit_of(blockIdx.x + stride), lane);
+        geo = unit_geom(gv0, !UNIFORM);
+        ids_next = unit_ids(dv1);
+    }
+    for (int64_t rd = blockIdx.x; rd < rounds; rd += stride) {
         const int hg = (int)(rd / rounds_per_hg);
         const int64_t u = (rd - (int64_t)hg * rounds_per_hg) * WPB + wave;
         const bool unit_on = u < p.U;
-        const Desc cur = next;
-        next = fetch(rd + gridDim.x);
+        // loads for the coming rounds, consumed just before this round's epilogue
+        const float gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
+        const float a_next = load_a(ids_next, rd + stride);
+        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride), lane);
         if (PROJ == PROJ_SHARED && hg != wa_hg) {
             const int hw = hg * 8 + wave;
 #pragma unroll
@@ -112,19 +121,19 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 }
             wa_hg = hg;
         }
-        const int64_t e_ij = cur.e_ij, e_ji = cur.e_ji, i = cur.i, j = cur.j, n = cur.n;
+        const int64_t e_ij = ids.e_ij, e_ji = ids.e_ji, i = ids.i, j = ids.j;
         Cell cell;
-        cell.rx = g_rpos[e_ij * 3 + 0];
-        cell.ry = g_rpos[e_ij * 3 + 1];
-        cell.rz = g_rpos[e_ij * 3 + 2];
+        cell.rx = geo.rx;
+        cell.ry = geo.ry;
+        cell.rz = geo.rz;
 #pragma unroll
-        for (int x = 0; x < 9; x++) cell.t[x] = g_tvecs[n * 9 + x];
+        for (int x = 0; x < 9; x++) cell.t[x] = geo.t[x];
 
         // column c: head (hg*8 + c%8) of atom i (c < 8) or atom j (c >= 8)
         const int h = hg * 8 + (c & 7);
         const bool col_on = unit_on && h < H && (c < 8 || e_ji != e_ij);
         const int64_t atom = (c < 8) ? i : j;
-        const float a = col_on ? g_a[atom * H + h] : -1.0f;
+        const float a = col_on ? a_cur : -1.0f;
         const float a2 = a * LOG2E;
 
         // translation box: union over the 16 columns; per-column boxes when they differ
@@ -132,8 +141,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         bx.U1 = bx.U2 = bx.U3 = p.lattice_range;
         int R1 = bx.U1, R2 = bx.U1, R3 = bx.U1;
         if (!UNIFORM) {
-            float rvl[3] = {g_rvlen[n * 3 + 0], g_rvlen[n * 3 + 1], g_rvlen[n * 3 + 2]};
-            range_rule(a, p.cutoff, rvl, p.lattice_range, p.min_range, R1, R2, R3);
+            range_rule(a, p.cutoff, geo.rvl, p.lattice_range, p.min_range, R1, R2, R3);
             if (!col_on) R1 = R2 = R3 = 0;
             bx.U1 = __builtin_amdgcn_readfirstlane(wave_max_int(R1));
             bx.U2 = __builtin_amdgcn_readfirstlane(wave_max_int(R2));
@@ -147,40 +155,30 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         bx.inv_S3 = 1.0f / (float)bx.S3;
         const int T = bx.T;
 
+        ColumnBoxes cbox{0, 0, 0};
+        if (!UNIFORM) cbox = column_boxes(R1, R2, R3, bx, lane);
         // geometry of one translation: d^2 and the in-box bits of the 16 columns
         auto geometry = [&](int idx, bool valid, float &d2, int &colbits) {
             int n1, n2, n3;
             decode(bx, valid ? idx : 0, n1, n2, n3);
             d2 = dist2(cell, (float)n1, (float)n2, (float)n3);
-            colbits = 0;
-            if (valid) {
-                if (UNIFORM) {
-                    colbits = 0xFFFF;
-                } else {
-#pragma unroll
-                    for (int x = 0; x < 16; x++) {
-                        int r1 = __builtin_amdgcn_readlane(R1, x);
-                        int r2 = __builtin_amdgcn_readlane(R2, x);
-                        int r3 = __builtin_amdgcn_readlane(R3, x);
-                        if (abs(n1) <= r1 && abs(n2) <= r2 && abs(n3) <= r3) colbits |= (1 << x);
-                    }
-                }
-            }
-        };
-        // per-column minimum of d^2 over the column's own box
-        float mloc[UNIFORM ? 1 : 16];
-#pragma unroll
-        for (int x = 0; x < (UNIFORM ? 1 : 16); x++) mloc[x] = 1e10f;
-        auto track_min = [&](float d2, int colbits) {
             if (UNIFORM) {
-                if (colbits) mloc[0] = fminf(mloc[0], d2);
+                colbits = valid ? 0xFFFF : 0;
             } else {
-#pragma unroll
-                for (int x = 0; x < 16; x++)
-                    if ((colbits >> x) & 1) mloc[x] = fminf(mloc[x], d2);
+                colbits = column_bits(cbox, n1, n2, n3);     // all lanes take part in the lookup
+                if (!valid) colbits = 0;
             }
         };
-        // boxes of up to RING_CAP translations are evaluated once and kept in registers
+        // First pass over the box: the nearest image inside at least one column's box.  Boxes of up
+        // to RING_CAP translations are evaluated once and kept in registers.
+        float best = 1e10f;
+        int best_idx = 0;
+        auto track_min = [&](float d2, int colbits, int idx) {
+            if (colbits != 0 && d2 < best) {
+                best = d2;
+                best_idx = idx;
+            }
+        };
         constexpr int NCACHE = RING_CAP / WAVE;
         float d2c[NCACHE];
         int bitsc[UNIFORM ? 1 : NCACHE];
@@ -192,7 +190,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 if (ch * WAVE < T) {
                     int cb;
                     geometry(ch * WAVE + lane, ch * WAVE + lane < T, d2c[ch], cb);
-                    track_min(d2c[ch], cb);
+                    track_min(d2c[ch], cb, ch * WAVE + lane);
                     if (!UNIFORM) bitsc[ch] = cb;
                 }
             }
@@ -201,18 +199,38 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 float d2;
                 int cb;
                 geometry(c0 + lane, c0 + lane < T, d2, cb);
-                track_min(d2, cb);
+                track_min(d2, cb, c0 + lane);
             }
         }
-        float d2min;
-        if (UNIFORM) {
-            d2min = wave_min(mloc[0]);
-        } else {
-            d2min = 1e10f;
+        // Per-column minimum of d^2 over the column's own box: the overall minimum wherever the
+        // nearest image lies inside the column's box (nearly always); otherwise a pass that
+        // tracks the 16 columns separately.
+        float d2min = wave_min(best);
+        if (!UNIFORM) {
+            const unsigned long long holders = __ballot(best == d2min);
+            const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)holders) - 1);
+            const int idx_star = __builtin_amdgcn_readlane(best_idx, src);
+            int n1, n2, n3;
+            decode(bx, idx_star, n1, n2, n3);
+            const int inside = __builtin_amdgcn_readfirstlane(column_bits(cbox, n1, n2, n3));
+            const bool own_min = col_on && !((inside >> c) & 1);
+            if (__ballot(own_min) != 0ull) {
+                float mloc[16];
 #pragma unroll
-            for (int x = 0; x < 16; x++) {
-                float mx = wave_min(mloc[x]);
-                if (c == x) d2min = mx;
+                for (int x = 0; x < 16; x++) mloc[x] = 1e10f;
+                for (int c0 = 0; c0 < T; c0 += WAVE) {
+                    float d2;
+                    int cb;
+                    geometry(c0 + lane, c0 + lane < T, d2, cb);
+#pragma unroll
+                    for (int x = 0; x < 16; x++)
+                        if ((cb >> x) & 1) mloc[x] = fminf(mloc[x], d2);
+                }
+#pragma unroll
+                for (int x = 0; x < 16; x++) {
+                    const float mx = wave_min(mloc[x]);
+                    if (c == x) d2min = mx;
+                }
             }
         }
         // A translation out of reach of every bin whose weight is below 2^-40 of the leading
@@ -318,6 +336,10 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
             }
             wave_mem_sync();
         }
+        // the loads issued at the top of the round have landed: make them uniform before the
+        // stores of the epilogue so that nothing younger is waited for
+        const UnitGeom geo_next = unit_geom(gv_next, !UNIFORM);
+        const UnitIds ids_next2 = unit_ids(dv_next2);
         // column totals: the 4 lanes sharing c hold partial sums
         sum += __shfl_xor(sum, 16, WAVE);
         sum += __shfl_xor(sum, 32, WAVE);
@@ -425,10 +447,15 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 }
             }
         }
+        ids = ids_next;
+        geo = geo_next;
+        a_cur = a_next;
+        ids_next = ids_next2;
     }
 }
 
-// (i <= j) edges of every crystal's dense block and their reverses.
+// Unit descriptors: the (i <= j) edges of every crystal's dense block, their reverses,
+// the two atoms and the crystal.
 __global__ void edge_pairs_kernel(const int64_t *atom_start, const int64_t *edge_start,
                                   const int64_t *unit_start, int64_t B, int64_t E, int64_t *pairs)
 {
@@ -439,15 +466,20 @@ __global__ void edge_pairs_kernel(const int64_t *atom_start, const int64_t *edge
         int64_t mid = (lo + hi) >> 1;
         if (edge_start[mid] <= e) lo = mid; else hi = mid;
     }
-    const int64_t n = atom_start[lo + 1] - atom_start[lo];
+    const int64_t a0 = atom_start[lo];
+    const int64_t n = atom_start[lo + 1] - a0;
     const int64_t e0 = edge_start[lo];
     const int64_t local = e - e0;
     const int64_t il = local / n, jl = local - il * n;
     if (il > jl) return;
     // row il of the upper triangle starts after il*n - il*(il-1)/2 units
     const int64_t u = unit_start[lo] + il * n - (il * (il - 1)) / 2 + (jl - il);
-    pairs[2 * u] = e;
-    pairs[2 * u + 1] = e0 + jl * n + il;
+    int64_t *d = pairs + PAIR_FIELDS * u;
+    d[0] = e;
+    d[1] = e0 + jl * n + il;
+    d[2] = a0 + il;
+    d[3] = a0 + jl;
+    d[4] = lo;
 }
 
 }  // namespace

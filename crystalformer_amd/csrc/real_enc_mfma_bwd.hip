@@ -36,8 +36,6 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     const int c = lane & 15;
     const int H = p.H, K = p.K, D = p.D;
     const int64_t *__restrict__ g_pairs = p.pairs;
-    const int64_t *__restrict__ g_edges = p.edges;
-    const int64_t *__restrict__ g_batch = p.batch;
     const float *__restrict__ g_rpos = p.rpos;
     const float *__restrict__ g_tvecs = p.tvecs;
     const float *__restrict__ g_a = p.a_ik;
@@ -50,7 +48,6 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     int *ring_bits = reinterpret_cast<int *>(ring_s + BRING_SLOTS);
     float *Sbuf = lds + WPB * 3 * BRING_SLOTS;                          // [8 heads][2 dirs][8 units][SROW]
     float *PXbuf = Sbuf + WPB * 16 * SROW;                              // [8 units][16 cols]
-    int64_t *meta = reinterpret_cast<int64_t *>(PXbuf + WPB * 16);      // [8 units][2]
 
     float ck[NT];
 #pragma unroll
@@ -63,18 +60,28 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 
     const int64_t rounds_per_hg = (p.U + WPB - 1) / WPB;
     const int64_t rounds = rounds_per_hg * p.head_groups;
-    struct Desc { int64_t e_ij, e_ji, i, j, n; };
-    auto fetch = [&](int64_t rd_) {
-        Desc dsc;
-        const int hg_ = (int)(rd_ / rounds_per_hg);
-        int64_t u_ = (rd_ - (int64_t)hg_ * rounds_per_hg) * WPB + wave;
-        if (rd_ >= rounds || u_ >= p.U) u_ = 0;
-        dsc.e_ij = g_pairs[2 * u_];
-        dsc.e_ji = g_pairs[2 * u_ + 1];
-        dsc.i = g_edges[dsc.e_ij];
-        dsc.j = g_edges[p.E + dsc.e_ij];
-        dsc.n = g_batch[dsc.i];
-        return dsc;
+    auto unit_of = [&](int64_t rd_) -> int64_t {
+        const int64_t hg_ = rd_ / rounds_per_hg;
+        const int64_t u_ = (rd_ - hg_ * rounds_per_hg) * WPB + wave;
+        return (rd_ < rounds && u_ < p.U) ? u_ : 0;
+    };
+    // exponent and forward output of column c of a unit in the head group of round rd_
+    auto load_a = [&](const UnitIds &d, int64_t rd_) -> float {
+        const int h_ = min((int)(rd_ / rounds_per_hg) * 8 + (c & 7), H - 1);
+        return g_a[((c < 8) ? d.i : d.j) * H + h_];
+    };
+    auto load_z = [&](const UnitIds &d, int64_t rd_) -> float {
+        const int h_ = min((int)(rd_ / rounds_per_hg) * 8 + (c & 7), H - 1);
+        return g_z[((c < 8) ? d.e_ij : d.e_ji) * H + h_];
+    };
+    // edge of product column c of round rd_: direction c/8 of the unit of wave c%8
+    // (-1: no such unit, or the reverse of a self edge)
+    auto load_col_edge = [&](int64_t rd_) -> int64_t {
+        const int64_t hg_ = rd_ / rounds_per_hg;
+        const int64_t u_ = (rd_ - hg_ * rounds_per_hg) * WPB + (c & 7);
+        if (rd_ >= rounds || u_ >= p.U) return -1;
+        const int64_t e0 = g_pairs[u_ * PAIR_FIELDS], e1 = g_pairs[u_ * PAIR_FIELDS + 1];
+        return (c < 8) ? e0 : (e1 != e0 ? e1 : -1);
     };
     auto flush_gW = [&](int hg_) {
         // lane (q, j) holds gW[d = 4q + r][bin = 16t + j] of head hg_*8 + wave
@@ -90,13 +97,30 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 }
         }
     };
-    Desc next = fetch(blockIdx.x);
-    for (int64_t rd = blockIdx.x; rd < rounds; rd += gridDim.x) {
+    const int64_t stride = gridDim.x;
+    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x), lane));
+    float a_cur, z_cur;
+    UnitGeom geo;
+    UnitIds ids_next;
+    int64_t col_edge = load_col_edge(blockIdx.x);
+    {
+        const float gv0 = load_unit_geom(ids, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
+        a_cur = load_a(ids, blockIdx.x);
+        z_cur = load_z(ids, blockIdx.x);
+        const int64_t dv1 = load_unit_ids(g_pairs, unit_of(blockIdx.x + stride), lane);
+        geo = unit_geom(gv0, !UNIFORM);
+        ids_next = unit_ids(dv1);
+    }
+    for (int64_t rd = blockIdx.x; rd < rounds; rd += stride) {
         const int hg = (int)(rd / rounds_per_hg);
         const int64_t u = (rd - (int64_t)hg * rounds_per_hg) * WPB + wave;
         const bool unit_on = u < p.U;
-        const Desc cur = next;
-        next = fetch(rd + gridDim.x);
+        // loads for the coming rounds, consumed just before this round's exchange
+        const float gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
+        const float a_next = load_a(ids_next, rd + stride);
+        const float z_next = load_z(ids_next, rd + stride);
+        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride), lane);
+        const int64_t col_edge_next = load_col_edge(rd + stride);
         if (hg != wa_hg) {
             if (wa_hg >= 0) flush_gW(wa_hg);
             const int hw = hg * 8 + wave;
@@ -109,28 +133,25 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             for (int t = 0; t < NT; t++) gWacc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
             wa_hg = hg;
         }
-        const int64_t e_ij = cur.e_ij, e_ji = cur.e_ji, i = cur.i, j = cur.j, n = cur.n;
+        const int64_t e_ij = ids.e_ij, e_ji = ids.e_ji;
         Cell cell;
-        cell.rx = g_rpos[e_ij * 3 + 0];
-        cell.ry = g_rpos[e_ij * 3 + 1];
-        cell.rz = g_rpos[e_ij * 3 + 2];
+        cell.rx = geo.rx;
+        cell.ry = geo.ry;
+        cell.rz = geo.rz;
 #pragma unroll
-        for (int x = 0; x < 9; x++) cell.t[x] = g_tvecs[n * 9 + x];
+        for (int x = 0; x < 9; x++) cell.t[x] = geo.t[x];
 
         const int h = hg * 8 + (c & 7);
         const bool col_on = unit_on && h < H && (c < 8 || e_ji != e_ij);
-        const int64_t atom = (c < 8) ? i : j;
-        const int64_t e_col = (c < 8) ? e_ij : e_ji;
-        const float a = col_on ? g_a[atom * H + h] : -1.0f;
+        const float a = col_on ? a_cur : -1.0f;
         const float a2 = a * LOG2E;
-        const float z2 = col_on ? g_z[e_col * H + h] * LOG2E : 0.f;
+        const float z2 = col_on ? z_cur * LOG2E : 0.f;
 
         BoxDims bx;
         bx.U1 = bx.U2 = bx.U3 = p.lattice_range;
         int R1 = bx.U1, R2 = bx.U1, R3 = bx.U1;
         if (!UNIFORM) {
-            float rvl[3] = {g_rvlen[n * 3 + 0], g_rvlen[n * 3 + 1], g_rvlen[n * 3 + 2]};
-            range_rule(a, p.cutoff, rvl, p.lattice_range, p.min_range, R1, R2, R3);
+            range_rule(a, p.cutoff, geo.rvl, p.lattice_range, p.min_range, R1, R2, R3);
             if (!col_on) R1 = R2 = R3 = 0;
             bx.U1 = __builtin_amdgcn_readfirstlane(wave_max_int(R1));
             bx.U2 = __builtin_amdgcn_readfirstlane(wave_max_int(R2));
@@ -143,6 +164,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         bx.inv_plane = 1.0f / (float)bx.plane;
         bx.inv_S3 = 1.0f / (float)bx.S3;
         const int T = bx.T;
+        ColumnBoxes cbox{0, 0, 0};
+        if (!UNIFORM) cbox = column_boxes(R1, R2, R3, bx, lane);
 
         // p_t <= 2^-40 in every column when a2_weak d2 - z2_floor <= -40
         const float a2_weak = wave_max(col_on ? a2 : -3.0e38f);
@@ -161,18 +184,11 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 decode(bx, valid ? s0 + c0 + lane : 0, n1, n2, n3);
                 const float d2 = dist2(cell, (float)n1, (float)n2, (float)n3);
                 int bits = 0;
-                if (valid) {
-                    if (UNIFORM) {
-                        bits = 0xFFFF;
-                    } else {
-#pragma unroll
-                        for (int x = 0; x < 16; x++) {
-                            int r1 = __builtin_amdgcn_readlane(R1, x);
-                            int r2 = __builtin_amdgcn_readlane(R2, x);
-                            int r3 = __builtin_amdgcn_readlane(R3, x);
-                            if (abs(n1) <= r1 && abs(n2) <= r2 && abs(n3) <= r3) bits |= (1 << x);
-                        }
-                    }
+                if (UNIFORM) {
+                    bits = valid ? 0xFFFF : 0;
+                } else {
+                    bits = column_bits(cbox, n1, n2, n3);     // all lanes take part in the lookup
+                    if (!valid) bits = 0;
                 }
                 const int colbits = bits;
                 const float s = sqrt_hw(d2) * p.s_scale;
@@ -244,22 +260,45 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             }
             wave_mem_sync();
         }
+        // the loads issued at the top of the round have landed
+        const UnitGeom geo_next = unit_geom(gv_next, !UNIFORM);
+        const UnitIds ids_next2 = unit_ids(dv_next2);
         px += __shfl_xor(px, 16, WAVE);
         px += __shfl_xor(px, 32, WAVE);
 
         // ---- exchange: column (dir, head) of unit `wave` -> row ((head*2 + dir)*8 + wave)
         const int srow = ((c & 7) * 2 + (c >> 3)) * WPB + wave;
         if (q == 0) PXbuf[wave * 16 + c] = px;
-        if (lane == 0) {
-            meta[2 * wave + 0] = unit_on ? e_ij : -1;
-            meta[2 * wave + 1] = (unit_on && e_ji != e_ij) ? e_ji : -1;
-        }
         const int hw = hg * 8 + wave;
         const int jcol = c, unit_j = jcol & 7, dir_j = jcol >> 3;    // product column j = dir*8 + unit
         const float *src = Sbuf + ((wave * 2 + dir_j) * WPB + unit_j) * SROW;
         float dotS = 0.f, dotQ = 0.f;
+        // gradient operands of this wave's head for the 16 product columns, requested before
+        // the exchange so that they arrive while the columns are parked
+        const int64_t e_out = col_edge;
         float4_t gv4 = {0.f, 0.f, 0.f, 0.f};
-        int64_t e_out = -1;
+        float gz_out = 0.f;
+        float gvk[4] = {0.f, 0.f, 0.f, 0.f};
+        if (hw < H) {
+            if (e_out >= 0 && g_gv) {
+                const float *gp = g_gv + (e_out * H + hw) * D + 4 * q;
+                if (4 * q + 3 < D) {
+                    gv4 = *reinterpret_cast<const float4_t *>(gp);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 3; r++)
+                        if (4 * q + r < D) gv4[r] = gp[r];
+                }
+            }
+            if (e_out >= 0 && g_gz && q == 0) gz_out = g_gz[e_out * H + hw];
+            if (p.gW_part && g_gv) {
+#pragma unroll
+                for (int s4 = 0; s4 < 4; s4++) {
+                    const int64_t e_k = __shfl(col_edge, 4 * s4 + q, WAVE);      // column 4*s4 + q
+                    if (e_k >= 0 && c < D) gvk[s4] = g_gv[(e_k * H + hw) * D + c];
+                }
+            }
+        }
 #pragma unroll
         for (int pass = 0; pass < 2; pass++) {
             // pass 0 exchanges S (also feeds gW), pass 1 exchanges Q
@@ -274,15 +313,6 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                     }
             }
             __syncthreads();
-            if (pass == 0) {
-                e_out = meta[2 * unit_j + dir_j];
-                if (e_out >= 0 && hw < H && g_gv) {
-                    const float *gp = g_gv + (e_out * H + hw) * D + 4 * q;
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        if (4 * q + r < D) gv4[r] = gp[r];
-                }
-            }
             float4_t out = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int t4 = 0; t4 < NT; t4++) {
@@ -303,8 +333,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 dotQ = dot;
                 if (q == 0 && e_out >= 0 && hw < H) {
                     const float PX = PXbuf[unit_j * 16 + dir_j * 8 + wave];
-                    const float gz = g_gz ? g_gz[e_out * H + hw] : 0.f;
-                    p.ga_edge[e_out * H + hw] = PX * gz + (dotQ - PX * dotS);
+                    p.ga_edge[e_out * H + hw] = PX * gz_out + (dotQ - PX * dotS);
                 }
             }
             if (pass == 0 && p.gW_part) {
@@ -313,9 +342,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 #pragma unroll
                 for (int s4 = 0; s4 < 4; s4++) {
                     const int colk = 4 * s4 + q;                    // this lane's reduction index
-                    const int64_t e_k = meta[2 * (colk & 7) + (colk >> 3)];
-                    float av = 0.f;
-                    if (e_k >= 0 && hw < H && g_gv && c < D) av = g_gv[(e_k * H + hw) * D + c];
+                    const float av = gvk[s4];
                     const float *srck = Sbuf + ((wave * 2 + (colk >> 3)) * WPB + (colk & 7)) * SROW;
 #pragma unroll
                     for (int t = 0; t < NT; t++)
@@ -324,6 +351,12 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             }
             __syncthreads();
         }
+        ids = ids_next;
+        geo = geo_next;
+        a_cur = a_next;
+        z_cur = z_next;
+        ids_next = ids_next2;
+        col_edge = col_edge_next;
     }
     if (wa_hg >= 0) flush_gW(wa_hg);
 }

@@ -16,7 +16,7 @@ struct PairArgs {
     const float *tvecs;
     const int64_t *batch;
     const int64_t *edges;
-    const int64_t *pairs;   // (U,2): edge (i->j) with i <= j and its reverse
+    const int64_t *pairs;   // (U,5): edge (i->j) with i <= j, its reverse, atoms i and j, crystal
     const float *W;
     const float *rvlen;
     float *z;
@@ -81,7 +81,117 @@ __device__ __forceinline__ int wave_max_int(int v)
     return v;
 }
 
+// ---- per-column boxes --------------------------------------------------------
+// Under the adaptive rule the 16 columns of a unit have their own half-widths
+// (R1,R2,R3 in lanes 0..15).  Lane r of the tables holds, for |n| = r + 1 along one
+// axis, the set of columns whose box reaches that far; |n| = 0 is inside every box.
+struct ColumnBoxes { int m1, m2, m3; };
+
+__device__ __forceinline__ int axis_table(int R, int U, int lane)
+{
+    int m = 0;
+    for (int r = 1; r <= U; r++) {       // U is wave-uniform
+        const int mask = (int)(__ballot(R >= r) & 0xFFFFull);
+        m = (lane == r - 1) ? mask : m;
+    }
+    return m;
+}
+
+__device__ __forceinline__ ColumnBoxes column_boxes(int R1, int R2, int R3, const BoxDims &bx, int lane)
+{
+    ColumnBoxes cb;
+    cb.m1 = axis_table(R1, bx.U1, lane);
+    cb.m2 = axis_table(R2, bx.U2, lane);
+    cb.m3 = axis_table(R3, bx.U3, lane);
+    return cb;
+}
+
+// columns whose box contains translation (n1,n2,n3); |n| <= 64 on every axis
+__device__ __forceinline__ int column_bits(const ColumnBoxes &cb, int n1, int n2, int n3)
+{
+    const int a1 = abs(n1), a2 = abs(n2), a3 = abs(n3);
+    int b1 = __shfl(cb.m1, max(a1 - 1, 0), WAVE);
+    int b2 = __shfl(cb.m2, max(a2 - 1, 0), WAVE);
+    int b3 = __shfl(cb.m3, max(a3 - 1, 0), WAVE);
+    b1 = a1 == 0 ? 0xFFFF : b1;
+    b2 = a2 == 0 ? 0xFFFF : b2;
+    b3 = a3 == 0 ? 0xFFFF : b3;
+    return b1 & b2 & b3;
+}
+
 constexpr int WPB = 8;                   // wavefronts per work-group = units per round
+constexpr int PAIR_FIELDS = 5;           // words per unit descriptor: e_ij, e_ji, i, j, crystal
+
+// ---- unit descriptors --------------------------------------------------------
+// Everything a round needs about its unit is fetched with per-lane vector loads
+// one or two rounds ahead and turned into wave-uniform values with readlane just
+// before the epilogue of the round in flight: the dependent chain
+// descriptor -> (p_j - p_i, lattice, exponents) never sits in front of compute,
+// and the waits land where the loads are a whole round old.
+struct UnitIds { int64_t e_ij, e_ji, i, j, n; };
+struct UnitGeom { float rx, ry, rz, t[9], rvl[3]; };
+
+__device__ __forceinline__ int64_t readlane_i64(int64_t v, int l)
+{
+    const int lo = __builtin_amdgcn_readlane((int)(v & 0xffffffffll), l);
+    const int hi = __builtin_amdgcn_readlane((int)(v >> 32), l);
+    return ((int64_t)hi << 32) | (int64_t)(unsigned int)lo;
+}
+
+// pins a wave-uniform value in a scalar register at this point of the program
+__device__ __forceinline__ float pin_uniform(float v)
+{
+    int x = __float_as_int(v);
+    asm volatile("" : "+s"(x));
+    return __int_as_float(x);
+}
+__device__ __forceinline__ int64_t pin_uniform(int64_t v)
+{
+    asm volatile("" : "+s"(v));
+    return v;
+}
+
+// lanes 0..4 receive the five descriptor words of unit u
+__device__ __forceinline__ int64_t load_unit_ids(const int64_t *__restrict__ pairs, int64_t u, int lane)
+{
+    return pairs[u * PAIR_FIELDS + min(lane, PAIR_FIELDS - 1)];
+}
+
+__device__ __forceinline__ UnitIds unit_ids(int64_t dv)
+{
+    UnitIds d;
+    d.e_ij = pin_uniform(readlane_i64(dv, 0));
+    d.e_ji = pin_uniform(readlane_i64(dv, 1));
+    d.i = pin_uniform(readlane_i64(dv, 2));
+    d.j = pin_uniform(readlane_i64(dv, 3));
+    d.n = pin_uniform(readlane_i64(dv, 4));
+    return d;
+}
+
+// lanes 0..2: p_j - p_i of the edge, 3..11: lattice rows, 12..14: reciprocal lengths
+__device__ __forceinline__ float load_unit_geom(const UnitIds &d, int lane, const float *__restrict__ rpos,
+                                                const float *__restrict__ tvecs,
+                                                const float *__restrict__ rvlen)
+{
+    const int l = min(lane, rvlen ? 14 : 11);
+    const float *src = l < 3 ? rpos + d.e_ij * 3 + l
+                     : l < 12 ? tvecs + d.n * 9 + (l - 3)
+                              : rvlen + d.n * 3 + (l - 12);
+    return *src;
+}
+
+__device__ __forceinline__ UnitGeom unit_geom(float gv, bool with_rvlen)
+{
+    UnitGeom g;
+    g.rx = pin_uniform(readlane_f(gv, 0));
+    g.ry = pin_uniform(readlane_f(gv, 1));
+    g.rz = pin_uniform(readlane_f(gv, 2));
+#pragma unroll
+    for (int x = 0; x < 9; x++) g.t[x] = pin_uniform(readlane_f(gv, 3 + x));
+#pragma unroll
+    for (int x = 0; x < 3; x++) g.rvl[x] = with_rvlen ? pin_uniform(readlane_f(gv, 12 + x)) : 0.f;
+    return g;
+}
 
 // Bin handled by reduction step s (0..4*NT-1) and sub-lane kk (0..3) of the projection:
 // chosen so that a lane's 4 consecutive steps read 4 consecutive bins.

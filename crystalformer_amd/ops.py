@@ -138,7 +138,7 @@ def real_enc_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
                  rvlen_n: Optional[Tensor] = None, cutoff_radius: Optional[float] = None,
                  lattice_range: int = 2, minimum_range: int = 0,
                  pairs_u: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
-    """``pairs_u`` (U,2) from :func:`edge_pairs` selects the matrix-core kernel
+    """``pairs_u`` (U,5) from :func:`edge_pairs` selects the matrix-core kernel
     that evaluates both directions of an atom pair together."""
     dev = require_device(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, W_k, rvlen_n, pairs_u)
     pairs_u = _i64(pairs_u, "pairs_u")
@@ -359,9 +359,13 @@ def edge_index(sizes: Tensor, pos: Optional[Tensor] = None,
     return edges, rpos
 
 
+PAIR_FIELDS = 5   # words per unit descriptor: e_ij, e_ji, i, j, crystal
+
+
 def edge_pairs(sizes: Tensor, num_atoms: Optional[int] = None, num_edges: Optional[int] = None) -> Tensor:
-    """(U,2) int64: for every unordered atom pair of each crystal's dense edge
-    block the edge (i->j), i <= j, and its reverse (j->i).  U = (E + N)/2; pass
+    """(U,5) int64 unit descriptors: for every unordered atom pair of each crystal's
+    dense edge block the edge (i->j), i <= j, its reverse (j->i), the atoms i and j
+    and the crystal.  U = (E + N)/2; pass
     ``num_atoms`` and ``num_edges`` when known to avoid a host sync."""
     dev = require_device(sizes)
     sizes = _i64(sizes, "sizes")
@@ -373,7 +377,7 @@ def edge_pairs(sizes: Tensor, num_atoms: Optional[int] = None, num_edges: Option
         tail = torch.stack([atom_start[-1], edge_start[-1]]).tolist() if B > 0 else [0, 0]
         num_atoms, num_edges = int(tail[0]), int(tail[1])
     U = (num_edges + num_atoms) // 2
-    pairs = torch.empty((U, 2), dtype=torch.int64, device=dev)
+    pairs = torch.empty((U, PAIR_FIELDS), dtype=torch.int64, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.load().cf_edge_pairs(ptr(atom_start), ptr(edge_start), ptr(unit_start), B, num_edges,
                                        ptr(pairs), stream_handle(dev))

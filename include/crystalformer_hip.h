@@ -59,13 +59,14 @@ int cf_max_translation_range(void);
  *                  <0: adaptive box from sqrt(-0.5/a)*|cutoff| per (atom,head);
  *                  >0: adaptive box from that radius.  Non-zero needs rvlen_n.
  *   minimum_range  lower bound of every adaptive half-width (0 = none)
- *   pairs_u   nullable, (U,2): for every unordered pair of atoms of a crystal
- *             (self pairs included) the edge (i->j), i <= j, and its reverse
- *             (j->i), as written by cf_edge_pairs.  When given (and K > 0) the
- *             two directions of a pair are evaluated together on the matrix
- *             cores; every edge must appear in exactly one pair and its reverse
- *             must carry rpos = -rpos.  NULL selects the per-edge kernels,
- *             which accept any edge list.
+ *   pairs_u   nullable, (U,5) unit descriptors as written by cf_edge_pairs: for
+ *             every unordered pair of atoms of a crystal (self pairs included)
+ *             the edge (i->j), i <= j, its reverse (j->i), the atoms i and j and
+ *             the crystal.  When given (and K > 0) the two directions of a pair
+ *             are evaluated together on the matrix cores; every edge must
+ *             appear in exactly one descriptor and its reverse must carry
+ *             rpos = -rpos.  NULL selects the per-edge kernels, which accept
+ *             any edge list.
  * Outputs
  *   z_ek  (E,H)                       log sum_n exp(a d^2)
  *   v_ekd nullable if K==0; (E,H,K) when W_k is NULL, else (E,H,D)
@@ -97,7 +98,7 @@ int64_t cf_real_enc_bwd_workspace(int64_t N, int64_t H, int64_t E, int64_t K, in
  *   gz_ek     (E,H)  gradient of z
  *   gv_ekd    nullable; (E,H,K) when W_k is NULL else (E,H,D)
  *   workspace device scratch of cf_real_enc_bwd_workspace() bytes (256-byte aligned)
- *   pairs_u   nullable, (U,2) pair list as for cf_real_enc_fwd; with it (and a shared
+ *   pairs_u   nullable, (U,5) unit descriptors as for cf_real_enc_fwd; with it (and a shared
  *             W_k, K <= 64, D <= 16) the two directions of a pair are evaluated together
  *             on the matrix cores
  * Outputs
@@ -206,14 +207,15 @@ int cf_edge_index(const int64_t *atom_start_n, const int64_t *edge_start_n, int6
                   void *stream);
 
 /*
- * Pair list of the dense per-crystal edge blocks: for each crystal of n atoms
- * the n(n+1)/2 pairs (i <= j) in row-major order of the upper triangle.
+ * Unit descriptors of the dense per-crystal edge blocks: for each crystal of n
+ * atoms the n(n+1)/2 pairs (i <= j) in row-major order of the upper triangle,
+ * five words each: edge (i->j), edge (j->i), atom i, atom j, crystal.
  * No counterpart in the reference (its kernels treat the two directions of an
  * edge independently, models/kernels/real_enc_proj_fwd.cu:24-31).
  *   atom_start_n, edge_start_n, unit_start_n (B+1): leading-zero cumulative
  *   sums of sizes, sizes^2 and sizes*(sizes+1)/2
  * Output
- *   pairs_u (U,2) with U = unit_start_n[B] = (E + N) / 2
+ *   pairs_u (U,5) with U = unit_start_n[B] = (E + N) / 2
  */
 int cf_edge_pairs(const int64_t *atom_start_n, const int64_t *edge_start_n,
                   const int64_t *unit_start_n, int64_t B, int64_t E, int64_t *pairs_u,

@@ -78,6 +78,43 @@ def test_real_enc_pair_kernel_large_boxes_and_indexed_projection(dev):
         assert_close(v, v_ref, "v")
 
 
+@pytest.mark.parametrize("cutoff,mr", [(-3.5, 0), (-1.0, 0), (2.0, 0), (-3.5, 1)])
+def test_real_enc_pair_kernel_atoms_outside_the_home_cell(dev, cutoff, mr):
+    """Atoms displaced by whole lattice vectors: the nearest image of an edge is then a
+    translation n != 0 that small per-column boxes do not contain, so columns of one unit
+    have different minimum distances (and some boxes miss the neighbourhood entirely)."""
+    p = Problem([5, 2, 8, 1], H=8, K=64, D=16, seed=31)
+    g = torch.Generator().manual_seed(77)
+    shift = torch.randint(-2, 3, (p.N, 3), generator=g).float()
+    p.b.pos = p.b.pos + (shift[:, None, :] @ p.b.trans_vec[p.b.batch]).squeeze(1)
+    p.rpos = tp.relative_positions(p.b.pos, p.edges)
+    p.a = p.a * torch.linspace(0.3, 3.0, 8)[None, :]        # heads with very different boxes
+    z_ref, v_ref = enc_fwd_ref(p, 64, p.W, cutoff, 2, mr)
+    z, v = enc_fwd_gpu(dev, p, 64, p.W, cutoff, 2, mr, pairs=True)
+    ok = torch.isfinite(z_ref)
+    assert ok.float().mean() > 0.5
+    assert_close(torch.where(ok, z.cpu(), torch.zeros(())), torch.where(ok, z_ref, torch.zeros(())), "z")
+    okv = ok[:, :, None].expand_as(v_ref)
+    assert_close(torch.where(okv, v.cpu(), torch.zeros(())), torch.where(okv, v_ref, torch.zeros(())), "v")
+    # backward on the same problem
+    a, rpos, tv, bt, ed, W, rv, es = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.W, p.rvlen,
+                                            p.e_start)
+    gz, gv = p.randn(p.E, 8), p.randn(p.E, 8, 16)
+    gz = torch.where(ok, gz, torch.zeros(()))
+    gv = torch.where(okv, gv, torch.zeros(()))
+    pairs = ops.edge_pairs(p.b.sizes.to(dev))
+    ga, gW = ops.real_enc_bwd(a, rpos, tv, bt, ed, es, z, gz.to(dev), gv.to(dev), 64, p.dist_max, p.wscale, W, rv,
+                              cutoff, 2, mr, pairs_u=pairs)
+    ga_ref, gW_ref = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv, 64,
+                                     p.dist_max, p.wscale, p.W, p.rvlen, cutoff, 2, mr)
+    if bool(ok.all()):
+        # exp(a d^2 - z) with |a d^2| ~ |z| ~ 10^3 here: the difference of two such float32 numbers
+        # carries ~1e-4 absolute error whatever the summation order, so this (deliberately extreme)
+        # case is held to 1e-4 instead of 1e-5
+        assert_close(ga, ga_ref, "ga", rtol=1e-4)
+        assert_close(gW, gW_ref.reshape(gW.shape), "gW", rtol=1e-4)
+
+
 @pytest.mark.parametrize("cutoff,lr,mr", RULES[:3])
 @pytest.mark.parametrize("H,K,D", [(8, 64, 16), (4, 16, 8), (16, 32, 16), (1, 7, 12), (8, 64, 32)])
 def test_real_enc_bwd_pair_kernel(dev, H, K, D, cutoff, lr, mr):
@@ -119,14 +156,17 @@ def test_edge_pairs_bit_exact(dev):
         b = make_sized_batch(sizes, seed=45)
         pairs = ops.edge_pairs(b.sizes.to(dev)).cpu()
         edges = tp.get_edge_index(sizes)
-        ref, off, eoff = [], 0, 0
-        for n in sizes:
+        ref, aoff, eoff = [], 0, 0
+        for b_idx, n in enumerate(sizes):
             for i in range(n):
                 for j in range(i, n):
-                    ref.append((eoff + i * n + j, eoff + j * n + i))
+                    ref.append((eoff + i * n + j, eoff + j * n + i, aoff + i, aoff + j, b_idx))
             eoff += n * n
+            aoff += n
         assert pairs.dtype == torch.int64 and pairs.tolist() == [list(r) for r in ref]
         assert torch.equal(edges[0][pairs[:, 0]], edges[1][pairs[:, 1]])
+        assert torch.equal(edges[0][pairs[:, 0]], pairs[:, 2]) and torch.equal(edges[1][pairs[:, 0]], pairs[:, 3])
+        assert torch.equal(b.batch[pairs[:, 2]], pairs[:, 4])
 
 
 def test_real_enc_fwd_matches_torch_path_fixed_cube(dev):
