@@ -65,32 +65,65 @@ __device__ __forceinline__ float readlane_f(float v, int lane)
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
 
+// ---- wave64 reductions on the DPP data path (no LDS round trips) --------------
+// Four steps inside each row of 16 lanes (quad swaps, rotations by 4 and 8), then
+// row 0 -> 1 and 2 -> 3 (row_bcast:15) and rows 0..1 -> 2..3 (row_bcast:31): lane 63
+// holds the result, which is returned wave-uniform.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_i(int old, int v)
+{
+    return __builtin_amdgcn_update_dpp(old, v, CTRL, ROW_MASK, 0xF, false);
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f(float old, float v)
+{
+    return __int_as_float(dpp_i<CTRL, ROW_MASK>(__float_as_int(old), __float_as_int(v)));
+}
+constexpr int DPP_QUAD_1032 = 0xB1, DPP_QUAD_2301 = 0x4E, DPP_ROW_ROR4 = 0x124, DPP_ROW_ROR8 = 0x128,
+              DPP_ROW_BCAST15 = 0x142, DPP_ROW_BCAST31 = 0x143;
+
 __device__ __forceinline__ float wave_sum(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
-    return v;
+    v += dpp_f<DPP_QUAD_1032, 0xF>(0.f, v);
+    v += dpp_f<DPP_QUAD_2301, 0xF>(0.f, v);
+    v += dpp_f<DPP_ROW_ROR4, 0xF>(0.f, v);
+    v += dpp_f<DPP_ROW_ROR8, 0xF>(0.f, v);
+    v += dpp_f<DPP_ROW_BCAST15, 0xA>(0.f, v);
+    v += dpp_f<DPP_ROW_BCAST31, 0xC>(0.f, v);
+    return readlane_f(v, 63);
 }
 
 __device__ __forceinline__ float wave_min(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, WAVE));
-    return v;
+    v = fminf(v, dpp_f<DPP_QUAD_1032, 0xF>(v, v));
+    v = fminf(v, dpp_f<DPP_QUAD_2301, 0xF>(v, v));
+    v = fminf(v, dpp_f<DPP_ROW_ROR4, 0xF>(v, v));
+    v = fminf(v, dpp_f<DPP_ROW_ROR8, 0xF>(v, v));
+    v = fminf(v, dpp_f<DPP_ROW_BCAST15, 0xA>(v, v));
+    v = fminf(v, dpp_f<DPP_ROW_BCAST31, 0xC>(v, v));
+    return readlane_f(v, 63);
 }
 
 __device__ __forceinline__ float wave_max(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
-    return v;
+    v = fmaxf(v, dpp_f<DPP_QUAD_1032, 0xF>(v, v));
+    v = fmaxf(v, dpp_f<DPP_QUAD_2301, 0xF>(v, v));
+    v = fmaxf(v, dpp_f<DPP_ROW_ROR4, 0xF>(v, v));
+    v = fmaxf(v, dpp_f<DPP_ROW_ROR8, 0xF>(v, v));
+    v = fmaxf(v, dpp_f<DPP_ROW_BCAST15, 0xA>(v, v));
+    v = fmaxf(v, dpp_f<DPP_ROW_BCAST31, 0xC>(v, v));
+    return readlane_f(v, 63);
 }
 
 __device__ __forceinline__ int wave_max_i(int v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, WAVE));
-    return v;
+    v = max(v, dpp_i<DPP_QUAD_1032, 0xF>(v, v));
+    v = max(v, dpp_i<DPP_QUAD_2301, 0xF>(v, v));
+    v = max(v, dpp_i<DPP_ROW_ROR4, 0xF>(v, v));
+    v = max(v, dpp_i<DPP_ROW_ROR8, 0xF>(v, v));
+    v = max(v, dpp_i<DPP_ROW_BCAST15, 0xA>(v, v));
+    v = max(v, dpp_i<DPP_ROW_BCAST31, 0xC>(v, v));
+    return __builtin_amdgcn_readlane(v, 63);
 }
 
 // Orders this wave's earlier LDS/global writes before its later reads.

@@ -59,8 +59,10 @@ __global__ void edge_index_kernel(const int64_t *atom_start, const int64_t *edge
     const int64_t local = e - edge_start[lo];
     const int64_t il = local / n;
     const int64_t i = a0 + il, j = a0 + (local - il * n);
-    edges[e] = i;
-    edges[E + e] = j;
+    if (edges) {
+        edges[e] = i;
+        edges[E + e] = j;
+    }
     if (pos && rpos) {
         rpos[e * 3 + 0] = pos[j * 3 + 0] - pos[i * 3 + 0];
         rpos[e * 3 + 1] = pos[j * 3 + 1] - pos[i * 3 + 1];
@@ -100,8 +102,9 @@ extern "C" int cf_edge_index(const int64_t *atom_start_n, const int64_t *edge_st
 {
     CF_REQUIRE(B >= 0 && E >= 0, CF_ERR_INVALID_ARGUMENT, "cf_edge_index: negative size");
     if (E == 0) return CF_OK;
-    CF_REQUIRE(B > 0 && atom_start_n && edge_start_n && edge_ij_e, CF_ERR_INVALID_ARGUMENT,
+    CF_REQUIRE(B > 0 && atom_start_n && edge_start_n, CF_ERR_INVALID_ARGUMENT,
                "cf_edge_index: null pointer or no crystals");
+    CF_REQUIRE(edge_ij_e || (pos && rpos_ij_e), CF_ERR_INVALID_ARGUMENT, "cf_edge_index: no output requested");
     edge_index_kernel<<<(int)((E + 255) / 256), 256, 0, (hipStream_t)stream>>>(atom_start_n, edge_start_n, B, E,
                                                                               pos, edge_ij_e, rpos_ij_e);
     CF_CHECK_LAUNCH("cf_edge_index");

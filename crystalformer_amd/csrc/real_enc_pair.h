@@ -74,12 +74,7 @@ __device__ __forceinline__ void decode(const BoxDims &bx, int idx, int &n1, int 
     n3 = r3 - bx.U3;
 }
 
-__device__ __forceinline__ int wave_max_int(int v)
-{
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, WAVE));
-    return v;
-}
+__device__ __forceinline__ int wave_max_int(int v) { return wave_max_i(v); }
 
 // ---- per-column boxes --------------------------------------------------------
 // Under the adaptive rule the 16 columns of a unit have their own half-widths

@@ -154,13 +154,15 @@ class CrystalformerEncoderCUDA(Module):
                 onehot: Optional[Tensor] = None) -> Tensor:
         if src.size(-1) != self.d_model:
             raise RuntimeError("the feature number of src and tgt must be equal to d_model")
-        batch = batch - batch[0]
         P = self.lattice_params
         # geometry prologue of compute_lattice_distances_for_cuda, plus the lengths of the
         # reciprocal vectors (all a block needs of them), in two launches
-        sizes = _sizes_on_device(sizes, batch, trans.shape[0], pos.device)
+        if not torch.is_tensor(sizes) or sizes.device != pos.device or sizes.dtype != torch.long:
+            sizes = _sizes_on_device(sizes, batch, trans.shape[0], pos.device)
+        layout = ops.batch_layout(sizes, batch)       # index structure: built once per batch
+        batch, edges = layout.batch, layout.edges
         vcell, _, rvlen = ops.lattice_geometry(trans)
-        edges, pos_ij = ops.edge_index(sizes, pos.contiguous())
+        pos_ij = ops.relative_positions(layout, pos)
         dist2_min = kr_base = None
         output = src
         for layer in self.layers:

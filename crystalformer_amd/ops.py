@@ -69,7 +69,7 @@ class _timed:
 # and the CSR offsets are built once.  Entries keep their key tensors alive, so a
 # recycled address can never alias a stale entry.
 _index_cache: list = []
-_INDEX_CACHE_SIZE = 8
+_INDEX_CACHE_SIZE = 24
 
 
 def _cache_lookup(kind: str, *keys: Tensor):
@@ -408,6 +408,64 @@ def cached_crystal_offsets(batch_i: Tensor) -> Tuple[Tensor, Tensor]:
     if hit is not None:
         return hit
     return _cache_store(sig, (batch_i,), crystal_offsets(batch_i))
+
+
+class BatchLayout:
+    """Index structure of a batch of crystals with dense intra-crystal edges.
+    Depends on the crystal sizes only, so it is built once per ``sizes`` tensor and
+    reused by every forward over that batch (and baked into a captured graph)."""
+
+    __slots__ = ("sizes", "batch", "atom_start", "edge_start", "num_atoms", "num_edges", "edges",
+                 "e_start", "pairs")
+
+
+def batch_layout(sizes: Tensor, batch_i: Tensor) -> BatchLayout:
+    """Layout for ``sizes`` (B,) / ``batch_i`` (N,), cached on the identity and version
+    of both tensors.  ``layout.batch`` is ``batch_i`` renumbered from 0.  The derived
+    tensors are also entered in the index caches under the keys the operators use."""
+    sig, hit = _cache_lookup("layout", sizes, batch_i)
+    if hit is not None:
+        return hit
+    dev = require_device(sizes, batch_i)
+    sizes = _i64(sizes, "sizes")
+    lay = BatchLayout()
+    lay.sizes = sizes
+    lay.batch = (batch_i - batch_i[0]) if batch_i.numel() else batch_i
+    lay.atom_start = F.pad(sizes.cumsum(0), (1, 0))
+    lay.edge_start = F.pad((sizes * sizes).cumsum(0), (1, 0))
+    tail = torch.stack([lay.atom_start[-1], lay.edge_start[-1]]).tolist() if sizes.numel() else [0, 0]
+    lay.num_atoms, lay.num_edges = int(tail[0]), int(tail[1])
+    if lay.num_atoms != batch_i.numel():
+        raise _lib.CrystalformerHipError(
+            f"sizes sum to {lay.num_atoms} atoms but batch has {batch_i.numel()} entries")
+    lay.edges, _ = edge_index(sizes, None, lay.num_edges)
+    lay.e_start = edge_row_offsets(lay.edges, lay.num_atoms)
+    lay.pairs = edge_pairs(sizes, lay.num_atoms, lay.num_edges) if lay.num_edges else None
+    s_, _ = _cache_lookup("e_start", lay.edges)
+    _cache_store(s_, (lay.edges,), lay.e_start)
+    if lay.pairs is not None:
+        s_, _ = _cache_lookup("pairs", lay.batch, lay.edges)
+        _cache_store(s_, (lay.batch, lay.edges), lay.pairs)
+    s_, _ = _cache_lookup("offsets", lay.batch)
+    _cache_store(s_, (lay.batch,), (lay.atom_start, lay.edge_start))
+    s_, _ = _cache_lookup("mean_start", sizes)
+    _cache_store(s_, (sizes,), lay.atom_start)
+    return _cache_store(sig, (sizes, batch_i), lay)
+
+
+def relative_positions(layout: BatchLayout, pos: Tensor) -> Tensor:
+    """p_j - p_i for every edge of the layout, (E,3)
+    (models/indexed_latticeformer_encoder.py:214)."""
+    dev = require_device(pos)
+    pos = _f32(pos, "pos")
+    if pos.shape != (layout.num_atoms, 3):
+        raise _lib.CrystalformerHipError(f"pos must be ({layout.num_atoms},3), got {tuple(pos.shape)}")
+    rpos = torch.empty((layout.num_edges, 3), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_edge_index(ptr(layout.atom_start), ptr(layout.edge_start), layout.sizes.numel(),
+                                       layout.num_edges, ptr(pos), None, ptr(rpos), stream_handle(dev))
+    check(rc, "cf_edge_index")
+    return rpos
 
 
 def lattice_geometry(trans_n: Tensor) -> Tuple[Tensor, Tensor, Tensor]:

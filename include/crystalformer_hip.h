@@ -200,7 +200,8 @@ int cf_minimum_distance(const float *rpos_ij_e, const float *tvecs_n, const int6
  *   atom_start_n, edge_start_n (B+1): leading-zero cumulative sums of sizes
  *   and sizes^2;  pos (N,3) nullable (then rpos_ij_e is not written)
  * Outputs
- *   edge_ij_e (2,E); rpos_ij_e nullable (E,3)
+ *   edge_ij_e (2,E), nullable when only the relative positions of a known
+ *   layout are wanted; rpos_ij_e nullable (E,3)
  */
 int cf_edge_index(const int64_t *atom_start_n, const int64_t *edge_start_n, int64_t B,
                   int64_t E, const float *pos, int64_t *edge_ij_e, float *rpos_ij_e,

@@ -429,3 +429,22 @@ def test_gauss_exponents_autograd(dev):
     assert_close(a, a_ref.detach(), "a")
     assert_close(qd.grad, qr.grad, "gq")
     assert_close(wd.grad, wr.grad, "gw")
+
+
+def test_batch_layout_bit_exact_and_cached(dev):
+    sizes = [3, 1, 4, 1, 5]
+    b = make_sized_batch(sizes, seed=3)
+    s_dev, bt_dev = b.sizes.to(dev), (b.batch + 7).to(dev)        # batch ids need not start at 0
+    lay = ops.batch_layout(s_dev, bt_dev)
+    edges = tp.get_edge_index(sizes)
+    assert torch.equal(lay.edges.cpu(), edges)
+    assert torch.equal(lay.batch.cpu(), b.batch)
+    assert torch.equal(lay.e_start.cpu(), tp.edge_row_offsets(edges, b.pos.shape[0]))
+    assert (lay.num_atoms, lay.num_edges) == (14, 52)
+    assert ops.batch_layout(s_dev, bt_dev) is lay                  # same tensors: cached
+    rpos = ops.relative_positions(lay, b.pos.to(dev))
+    assert torch.equal(rpos.cpu(), tp.relative_positions(b.pos, edges))
+    other = ops.batch_layout(torch.tensor([2, 2], device=dev), torch.tensor([0, 0, 1, 1], device=dev))
+    assert other is not lay and other.num_edges == 8
+    with pytest.raises(lib.CrystalformerHipError):
+        ops.batch_layout(torch.tensor([2, 2], device=dev), torch.tensor([0, 0, 1], device=dev))
