@@ -115,6 +115,25 @@ __device__ __forceinline__ float wave_max(float v)
     return readlane_f(v, 63);
 }
 
+// Maximum over each row of 16 lanes, left in every lane of the row.
+__device__ __forceinline__ float row16_max(float v)
+{
+    v = fmaxf(v, dpp_f<DPP_QUAD_1032, 0xF>(v, v));
+    v = fmaxf(v, dpp_f<DPP_QUAD_2301, 0xF>(v, v));
+    v = fmaxf(v, dpp_f<DPP_ROW_ROR4, 0xF>(v, v));
+    v = fmaxf(v, dpp_f<DPP_ROW_ROR8, 0xF>(v, v));
+    return v;
+}
+
+__device__ __forceinline__ float row16_min(float v)
+{
+    v = fminf(v, dpp_f<DPP_QUAD_1032, 0xF>(v, v));
+    v = fminf(v, dpp_f<DPP_QUAD_2301, 0xF>(v, v));
+    v = fminf(v, dpp_f<DPP_ROW_ROR4, 0xF>(v, v));
+    v = fminf(v, dpp_f<DPP_ROW_ROR8, 0xF>(v, v));
+    return v;
+}
+
 __device__ __forceinline__ int wave_max_i(int v)
 {
     v = max(v, dpp_i<DPP_QUAD_1032, 0xF>(v, v));

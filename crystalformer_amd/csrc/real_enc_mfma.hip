@@ -183,11 +183,14 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         float d2c[NCACHE];
         int bitsc[UNIFORM ? 1 : NCACHE];
         const bool cached = T <= RING_CAP;
+        // chunks of 64 translations in the box; kept opaque so that the chunk guards below stay
+        // real (wave-uniform) branches instead of being folded into lane predicates
+        const int nchunk = __builtin_amdgcn_readfirstlane((T + WAVE - 1) / WAVE);
         if (cached) {
 #pragma unroll
             for (int ch = 0; ch < NCACHE; ch++) {
                 d2c[ch] = 0.f;
-                if (ch * WAVE < T) {
+                if (ch < nchunk) {
                     int cb;
                     geometry(ch * WAVE + lane, ch * WAVE + lane < T, d2c[ch], cb);
                     track_min(d2c[ch], cb, ch * WAVE + lane);
@@ -237,8 +240,9 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         // term in EVERY column cannot change an fp32 sum and is dropped.  For all columns
         // a2_c (d2 - d2min_c) <= a2_weak (d2 - d2min_far) with the weakest decay and the
         // largest per-column minimum.
-        const float a2_weak = wave_max(col_on ? a2 : -3.0e38f);
-        const float d2min_far = wave_max(col_on ? d2min : 0.f);
+        // (every row of 16 lanes holds the 16 columns, so a reduction over a row is complete)
+        const float a2_weak = row16_max(col_on ? a2 : -3.0e38f);
+        const float d2min_far = UNIFORM ? d2min : row16_max(col_on ? d2min : 0.f);
 
         float4_t acc[NT];
 #pragma unroll
@@ -279,7 +283,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
             if (cached) {
 #pragma unroll
                 for (int ch = 0; ch < NCACHE; ch++)
-                    if (ch * WAVE < T) stage(d2c[ch], UNIFORM ? (ch * WAVE + lane < T ? 0xFFFF : 0) : bitsc[UNIFORM ? 0 : ch],
+                    if (ch < nchunk) stage(d2c[ch], UNIFORM ? (ch * WAVE + lane < T ? 0xFFFF : 0) : bitsc[UNIFORM ? 0 : ch],
                                              ch * WAVE + lane < T);
             } else {
                 for (int c0 = 0; c0 < cnt; c0 += WAVE) {

@@ -168,8 +168,9 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         if (!UNIFORM) cbox = column_boxes(R1, R2, R3, bx, lane);
 
         // p_t <= 2^-40 in every column when a2_weak d2 - z2_floor <= -40
-        const float a2_weak = wave_max(col_on ? a2 : -3.0e38f);
-        const float z2_floor = wave_min(col_on ? z2 : 3.0e38f);
+        // (every row of 16 lanes holds the 16 columns, so a reduction over a row is complete)
+        const float a2_weak = row16_max(col_on ? a2 : -3.0e38f);
+        const float z2_floor = row16_min(col_on ? z2 : 3.0e38f);
 
         float4_t accS[NT], accQ[NT];
 #pragma unroll
