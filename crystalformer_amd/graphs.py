@@ -54,3 +54,77 @@ class GraphedForward:
             self.static.trans_vec.copy_(batch.trans_vec)
         self.graph.replay()
         return self.output
+
+
+class GraphedTrainStep:
+    """One whole training step -- forward, L1 loss, backward, gradient-norm clip,
+    AdamW update and learning-rate schedule -- captured into a HIP graph and
+    replayed with a single submission.
+
+    Optimiser settings are those of :func:`crystalformer_amd.training.make_optimizer`;
+    the schedule lr0 * sqrt(decay / (decay + t)) is evaluated on the device from a
+    step counter that lives in the graph, so no host value is baked into it.
+    ``batch`` fixes the layout; later calls may pass other positions, lattices,
+    species and targets with identical ``sizes``.
+    """
+
+    def __init__(self, model: torch.nn.Module, batch: CrystalBatch, lr: float = 5e-4, sch_decay: float = 4000.0,
+                 clip_norm: float = 1.0, warmup: int = 3, capture: bool = True):
+        from .training import make_optimizer
+        if not batch.pos.is_cuda or batch.y is None:
+            raise ValueError("GraphedTrainStep needs a batch with targets on the GPU")
+        dev = batch.pos.device
+        self.model = model
+        self.static = CrystalBatch(batch.x.clone(), batch.pos.clone(), batch.batch.clone(),
+                                   batch.trans_vec.clone(), batch.sizes.clone(), batch.y.clone())
+        self.clip_norm = clip_norm
+        self.lr0, self.decay = lr, sch_decay
+        self.opt, _ = make_optimizer(model, lr=lr, capturable=True)
+        self.lr_t = torch.tensor(lr, dtype=torch.float32, device=dev)
+        for group in self.opt.param_groups:
+            group["lr"] = self.lr_t                       # one device scalar shared by all groups
+        self.step_t = torch.zeros((), dtype=torch.float32, device=dev)
+        self.params = [p for p in model.parameters() if p.requires_grad]
+        model.train()
+        stream = torch.cuda.Stream()                      # default priority
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            for _ in range(max(warmup, 1)):               # primes caches, optimiser state and workspaces
+                self.opt.zero_grad(set_to_none=True)
+                self._step()
+        torch.cuda.current_stream().wait_stream(stream)
+        torch.cuda.synchronize()
+        self.graph = None
+        self.opt.zero_grad(set_to_none=True)
+        if capture:                                       # capture=False: same step, launched eagerly
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.loss = self._step()
+            torch.cuda.synchronize()
+
+    def _step(self) -> torch.Tensor:
+        import torch.nn.functional as F
+        self.lr_t.copy_(self.lr0 * torch.sqrt(self.decay / (self.decay + self.step_t)))
+        out = self.model(self.static)
+        loss = F.l1_loss(out[:, 0], self.static.y, reduction="none").mean()
+        loss.backward()
+        if self.clip_norm > 0:
+            torch.nn.utils.clip_grad_norm_(self.params, self.clip_norm, foreach=True)
+        self.opt.step()
+        self.step_t += 1.0
+        return loss.detach()
+
+    def __call__(self, batch: Optional[CrystalBatch] = None) -> torch.Tensor:
+        if batch is not None and batch is not self.static:
+            if batch.pos.shape != self.static.pos.shape or batch.sizes.shape != self.static.sizes.shape:
+                raise ValueError("batch layout differs from the captured one")
+            self.static.x.copy_(batch.x)
+            self.static.pos.copy_(batch.pos)
+            self.static.trans_vec.copy_(batch.trans_vec)
+            self.static.y.copy_(batch.y)
+        if self.graph is None:
+            self.opt.zero_grad(set_to_none=True)
+            self.loss = self._step()
+        else:
+            self.graph.replay()
+        return self.loss

@@ -14,7 +14,8 @@ from torch.optim import lr_scheduler
 
 
 def make_optimizer(model: nn.Module, lr: float = 5e-4, betas=(0.9, 0.98), weight_decay: float = 1e-5,
-                   sch_decay: float = 4000.0) -> Tuple[optim.Optimizer, lr_scheduler.LambdaLR]:
+                   sch_decay: float = 4000.0,
+                   capturable: bool = False) -> Tuple[optim.Optimizer, lr_scheduler.LambdaLR]:
     nodecay, decay = [], []
     for m in model.modules():
         if isinstance(m, (nn.BatchNorm1d, nn.LayerNorm, nn.SyncBatchNorm)):
@@ -25,7 +26,7 @@ def make_optimizer(model: nn.Module, lr: float = 5e-4, betas=(0.9, 0.98), weight
     assert sum(p.numel() for p in nodecay + decay) == sum(p.numel() for p in model.parameters())
     groups = [{"params": nodecay}, {"params": decay, "weight_decay": weight_decay}] if weight_decay > 0 \
         else [{"params": list(model.parameters())}]
-    opt = optim.AdamW(groups, lr=lr, betas=betas, weight_decay=0.0 if weight_decay > 0 else 0.0)
+    opt = optim.AdamW(groups, lr=lr, betas=betas, weight_decay=0.0, capturable=capturable)
     sch = lr_scheduler.LambdaLR(opt, lambda t: (sch_decay / (sch_decay + t)) ** 0.5)
     return opt, sch
 
