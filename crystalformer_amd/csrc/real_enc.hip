@@ -862,7 +862,7 @@ extern "C" int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const 
                (long long)((E + N) / 2), (long long)U);
     p.z = z_ek;
     p.v = v_ekd;
-    if (pairs_u && K > 0) {
+    if (pairs_u) {
         rc = launch_real_enc_fwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, N, H, E, K, D,
                                        p.bin_step, p.s_scale, p.W, W_num, rvlen_n, p.cutoff, lattice_range,
                                        minimum_range, z_ek, v_ekd, (hipStream_t)stream);

@@ -499,7 +499,7 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
                               int64_t W_num, const float *rvlen, float cutoff, int lattice_range,
                               int min_range, float *z, float *v, hipStream_t st)
 {
-    if (K < 1 || K > 128) return CF_ERR_UNSUPPORTED;
+    if (K < 0 || K > 128) return CF_ERR_UNSUPPORTED;
     if (W && (D < 1 || D > 64)) return CF_ERR_UNSUPPORTED;
     PairArgs p{};
     p.a_ik = a_ik; p.rpos = rpos; p.tvecs = tvecs; p.batch = batch; p.edges = edges; p.pairs = pairs;
@@ -511,6 +511,11 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     p.bin_step = bin_step; p.s_scale = s_scale;
     p.inv_bin_step = 1.0f / bin_step;
     p.window = sqrtf(40.0f) / bin_step;                 // exp2(-(bin_step*x)^2) < 2^-40 beyond it
+    if (K == 0) {
+        // bias only: no bins, so no translation is ever "near"; all of them feed the column sums
+        p.bin_step = p.s_scale = p.inv_bin_step = 0.f;
+        p.window = -1.0e30f;
+    }
     const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
     const bool uniform = cutoff == 0.0f;
     int mode = PROJ_NONE;

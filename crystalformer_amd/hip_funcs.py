@@ -86,7 +86,7 @@ def compile_kernels(lattice_range: int, head_num: int, key_head_dim: int, value_
 
 
 def _pairs(batch_i: Tensor, edge_ij_e: Tensor, tvecs_n: Tensor, K: int) -> Optional[Tensor]:
-    if K <= 0 or not KernelManager.DENSE_EDGE_BLOCKS or edge_ij_e.shape[1] == 0:
+    if not KernelManager.DENSE_EDGE_BLOCKS or edge_ij_e.shape[1] == 0:
         return None
     return ops.cached_edge_pairs(batch_i, edge_ij_e, tvecs_n.shape[0])
 
