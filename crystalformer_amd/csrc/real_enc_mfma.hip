@@ -66,6 +66,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
     int *ring_bits = reinterpret_cast<int *>(ring_s + RING_SLOTS);
     float *Sbuf = lds + WPB * 3 * RING_SLOTS;                        // [WPB][16][SROW]
     int64_t *meta = reinterpret_cast<int64_t *>(Sbuf + WPB * 16 * SROW);   // [WPB][2]
+    float *invbuf = reinterpret_cast<float *>(meta + WPB * 2);             // [WPB][16]
 
     // Gaussian argument of bin 16m + c at distance 0
     float ck[NT];
@@ -76,40 +77,42 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
     float Wa[PROJ == PROJ_SHARED ? DT : 1][PROJ == PROJ_SHARED ? 4 * NT : 1];
     int wa_hg = -1;
 
-    const int64_t rounds_per_hg = (p.U + WPB - 1) / WPB;
-    const int64_t rounds = rounds_per_hg * p.head_groups;
+    const int rounds_per_hg = (int)((p.U + WPB - 1) / WPB);
+    const int rounds = rounds_per_hg * p.head_groups;
     // unit of round rd_ for this wave (0 when the round or the unit does not exist: loads stay valid)
-    auto unit_of = [&](int64_t rd_) -> int64_t {
-        const int64_t hg_ = rd_ / rounds_per_hg;
-        const int64_t u_ = (rd_ - hg_ * rounds_per_hg) * WPB + wave;
+    auto unit_of = [&](int rd_, const RoundPos &rp) -> int64_t {
+        const int64_t u_ = (int64_t)rp.r * WPB + wave;
         return (rd_ < rounds && u_ < p.U) ? u_ : 0;
     };
-    // exponent of column c of a unit in the head group of round rd_
-    auto load_a = [&](const UnitIds &d, int64_t rd_) -> float {
-        const int h_ = min((int)(rd_ / rounds_per_hg) * 8 + (c & 7), H - 1);
+    // exponent of column c of a unit in the head group of a round
+    auto load_a = [&](const UnitIds &d, const RoundPos &rp) -> float {
+        const int h_ = min(rp.hg * 8 + (c & 7), H - 1);
         return g_a[((c < 8) ? d.i : d.j) * H + h_];
     };
-    const int64_t stride = gridDim.x;
+    const int stride = gridDim.x;
+    RoundPos pos = round_pos(blockIdx.x, rounds_per_hg, p.head_groups);
+    RoundPos pos_next = round_pos(blockIdx.x + stride, rounds_per_hg, p.head_groups);
     // fill the descriptor pipeline: current round complete, next round's ids known
-    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x), lane));
+    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x, pos), lane));
     float a_cur;
     UnitGeom geo;
     UnitIds ids_next;
     {
         const float gv0 = load_unit_geom(ids, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
-        a_cur = load_a(ids, blockIdx.x);
-        const int64_t dv1 = load_unit_ids(g_pairs, unit_of(blockIdx.x + stride), lane);
+        a_cur = load_a(ids, pos);
+        const int64_t dv1 = load_unit_ids(g_pairs, unit_of(blockIdx.x + stride, pos_next), lane);
         geo = unit_geom(gv0, !UNIFORM);
         ids_next = unit_ids(dv1);
     }
-    for (int64_t rd = blockIdx.x; rd < rounds; rd += stride) {
-        const int hg = (int)(rd / rounds_per_hg);
-        const int64_t u = (rd - (int64_t)hg * rounds_per_hg) * WPB + wave;
+    for (int rd = blockIdx.x; rd < rounds; rd += stride) {
+        const int hg = pos.hg;
+        const int64_t u = (int64_t)pos.r * WPB + wave;
         const bool unit_on = u < p.U;
+        const RoundPos pos_next2 = round_pos(rd + 2 * stride, rounds_per_hg, p.head_groups);
         // loads for the coming rounds, consumed just before this round's epilogue
         const float gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
-        const float a_next = load_a(ids_next, rd + stride);
-        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride), lane);
+        const float a_next = load_a(ids_next, pos_next);
+        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane);
         if (PROJ == PROJ_SHARED && hg != wa_hg) {
             const int hw = hg * 8 + wave;
 #pragma unroll
@@ -255,6 +258,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
             // of the ring, so that the second kind never enters the Gaussian loop.
             int near_cnt = 0, far_cnt = 0;
             auto stage = [&](float d2, int colbits, bool valid) {
+                asm volatile("" : "+v"(d2));      // keeps this chunk's arithmetic behind its guard
                 const float s = sqrt_hw(d2) * p.s_scale;
                 const float xb = s * p.inv_bin_step - 1.0f;          // fractional bin coordinate
                 int bits = colbits;
@@ -364,12 +368,14 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 }
             }
         } else if (PROJ == PROJ_SHARED) {
-            // park the normalised column (zero for inactive columns), then project per head
+            // park the column sums (inactive columns hold zeros: their weights are masked) and the
+            // reciprocal of the column totals, then project per head
             float *col = Sbuf + (wave * 16 + c) * SROW;
 #pragma unroll
             for (int m = 0; m < NT; m++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) col[16 * m + 4 * q + r] = col_on ? acc[m][r] * inv : 0.f;
+                for (int r = 0; r < 4; r++) col[16 * m + 4 * q + r] = acc[m][r];
+            if (q == 0) invbuf[wave * 16 + c] = inv;
             if (lane == 0) {
                 meta[2 * wave + 0] = unit_on ? e_ij : -1;
                 meta[2 * wave + 1] = (unit_on && e_ji != e_ij) ? e_ji : -1;
@@ -394,8 +400,11 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                         for (int dt = 0; dt < DT; dt++)
                             out[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(Wa[dt][4 * t4 + r], sb[r], out[dt], 0, 0, 0);
                 }
-                // lane (q, j) holds components 16dt + 4q + r of column j
+                // lane (q, j) holds components 16dt + 4q + r of column j, still to be normalised
                 const int64_t e_out = meta[2 * unit_j + dir_j];
+                const float inv_j = invbuf[unit_j * 16 + dir_j * 8 + wave];
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++) out[dt] *= inv_j;
                 if (e_out >= 0 && hw < H) {
 #pragma unroll
                     for (int dt = 0; dt < DT; dt++) {
@@ -455,6 +464,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         geo = geo_next;
         a_cur = a_next;
         ids_next = ids_next2;
+        pos = pos_next;
+        pos_next = pos_next2;
     }
 }
 
@@ -523,8 +534,10 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     if (mode == PROJ_SHARED && D > 32) return CF_ERR_UNSUPPORTED;
     const int DT = (mode == PROJ_SHARED && D > 16) ? 2 : 1;
     size_t lds = sizeof(float) * (size_t)WPB * 3 * RING_SLOTS;
-    if (mode == PROJ_SHARED) lds += sizeof(float) * (size_t)WPB * 16 * (16 * NT + 1) + sizeof(int64_t) * WPB * 2 + 8;
+    if (mode == PROJ_SHARED)
+        lds += sizeof(float) * (size_t)WPB * 16 * (16 * NT + 1) + sizeof(int64_t) * WPB * 2 + sizeof(float) * WPB * 16 + 8;
     const int64_t rounds = ((U + WPB - 1) / WPB) * p.head_groups;
+    if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // round positions are 32-bit in the kernel
     int64_t blocks = rounds;
     int64_t cap = (int64_t)device_cu_count() * 2;      // 16 waves per CU
     if (blocks > cap) blocks = cap;

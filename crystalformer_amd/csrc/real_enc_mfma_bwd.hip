@@ -58,27 +58,25 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     float4_t gWacc[NT];
     int wa_hg = -1;
 
-    const int64_t rounds_per_hg = (p.U + WPB - 1) / WPB;
-    const int64_t rounds = rounds_per_hg * p.head_groups;
-    auto unit_of = [&](int64_t rd_) -> int64_t {
-        const int64_t hg_ = rd_ / rounds_per_hg;
-        const int64_t u_ = (rd_ - hg_ * rounds_per_hg) * WPB + wave;
+    const int rounds_per_hg = (int)((p.U + WPB - 1) / WPB);
+    const int rounds = rounds_per_hg * p.head_groups;
+    auto unit_of = [&](int rd_, const RoundPos &rp) -> int64_t {
+        const int64_t u_ = (int64_t)rp.r * WPB + wave;
         return (rd_ < rounds && u_ < p.U) ? u_ : 0;
     };
-    // exponent and forward output of column c of a unit in the head group of round rd_
-    auto load_a = [&](const UnitIds &d, int64_t rd_) -> float {
-        const int h_ = min((int)(rd_ / rounds_per_hg) * 8 + (c & 7), H - 1);
+    // exponent and forward output of column c of a unit in the head group of a round
+    auto load_a = [&](const UnitIds &d, const RoundPos &rp) -> float {
+        const int h_ = min(rp.hg * 8 + (c & 7), H - 1);
         return g_a[((c < 8) ? d.i : d.j) * H + h_];
     };
-    auto load_z = [&](const UnitIds &d, int64_t rd_) -> float {
-        const int h_ = min((int)(rd_ / rounds_per_hg) * 8 + (c & 7), H - 1);
+    auto load_z = [&](const UnitIds &d, const RoundPos &rp) -> float {
+        const int h_ = min(rp.hg * 8 + (c & 7), H - 1);
         return g_z[((c < 8) ? d.e_ij : d.e_ji) * H + h_];
     };
     // edge of product column c of round rd_: direction c/8 of the unit of wave c%8
     // (-1: no such unit, or the reverse of a self edge)
-    auto load_col_edge = [&](int64_t rd_) -> int64_t {
-        const int64_t hg_ = rd_ / rounds_per_hg;
-        const int64_t u_ = (rd_ - hg_ * rounds_per_hg) * WPB + (c & 7);
+    auto load_col_edge = [&](int rd_, const RoundPos &rp) -> int64_t {
+        const int64_t u_ = (int64_t)rp.r * WPB + (c & 7);
         if (rd_ >= rounds || u_ >= p.U) return -1;
         const int64_t e0 = g_pairs[u_ * PAIR_FIELDS], e1 = g_pairs[u_ * PAIR_FIELDS + 1];
         return (c < 8) ? e0 : (e1 != e0 ? e1 : -1);
@@ -97,30 +95,33 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 }
         }
     };
-    const int64_t stride = gridDim.x;
-    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x), lane));
+    const int stride = gridDim.x;
+    RoundPos pos = round_pos(blockIdx.x, rounds_per_hg, p.head_groups);
+    RoundPos pos_next = round_pos(blockIdx.x + stride, rounds_per_hg, p.head_groups);
+    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x, pos), lane));
     float a_cur, z_cur;
     UnitGeom geo;
     UnitIds ids_next;
-    int64_t col_edge = load_col_edge(blockIdx.x);
+    int64_t col_edge = load_col_edge(blockIdx.x, pos);
     {
         const float gv0 = load_unit_geom(ids, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
-        a_cur = load_a(ids, blockIdx.x);
-        z_cur = load_z(ids, blockIdx.x);
-        const int64_t dv1 = load_unit_ids(g_pairs, unit_of(blockIdx.x + stride), lane);
+        a_cur = load_a(ids, pos);
+        z_cur = load_z(ids, pos);
+        const int64_t dv1 = load_unit_ids(g_pairs, unit_of(blockIdx.x + stride, pos_next), lane);
         geo = unit_geom(gv0, !UNIFORM);
         ids_next = unit_ids(dv1);
     }
-    for (int64_t rd = blockIdx.x; rd < rounds; rd += stride) {
-        const int hg = (int)(rd / rounds_per_hg);
-        const int64_t u = (rd - (int64_t)hg * rounds_per_hg) * WPB + wave;
+    for (int rd = blockIdx.x; rd < rounds; rd += stride) {
+        const int hg = pos.hg;
+        const int64_t u = (int64_t)pos.r * WPB + wave;
         const bool unit_on = u < p.U;
+        const RoundPos pos_next2 = round_pos(rd + 2 * stride, rounds_per_hg, p.head_groups);
         // loads for the coming rounds, consumed just before this round's exchange
         const float gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
-        const float a_next = load_a(ids_next, rd + stride);
-        const float z_next = load_z(ids_next, rd + stride);
-        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride), lane);
-        const int64_t col_edge_next = load_col_edge(rd + stride);
+        const float a_next = load_a(ids_next, pos_next);
+        const float z_next = load_z(ids_next, pos_next);
+        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane);
+        const int64_t col_edge_next = load_col_edge(rd + stride, pos_next);
         if (hg != wa_hg) {
             if (wa_hg >= 0) flush_gW(wa_hg);
             const int hw = hg * 8 + wave;
@@ -358,6 +359,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         z_cur = z_next;
         ids_next = ids_next2;
         col_edge = col_edge_next;
+        pos = pos_next;
+        pos_next = pos_next2;
     }
     if (wa_hg >= 0) flush_gW(wa_hg);
 }
@@ -415,6 +418,7 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
     const bool uniform = cutoff == 0.0f;
     const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)WPB * 16 * (16 * NT + 1) + WPB * 16) +
                        sizeof(int64_t) * WPB * 2 + 8;
+    if (((U + WPB - 1) / WPB) * ((H + 7) / 8) >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // 32-bit round positions
     const int blocks = real_enc_bwd_pairs_blocks(U, H);
 #define CF_BPAIR(NTV)                                                                              \
     do {                                                                                           \

@@ -117,6 +117,23 @@ __device__ __forceinline__ int column_bits(const ColumnBoxes &cb, int n1, int n2
 constexpr int WPB = 8;                   // wavefronts per work-group = units per round
 constexpr int PAIR_FIELDS = 5;           // words per unit descriptor: e_ij, e_ji, i, j, crystal
 
+// Position of a round: head group and round index inside it.  32-bit; the launchers
+// refuse work with 2^30 rounds or more.  One head group (H <= 8) needs no division.
+struct RoundPos { int hg, r; };
+
+__device__ __forceinline__ RoundPos round_pos(int rd, int rounds_per_hg, int head_groups)
+{
+    RoundPos x;
+    if (head_groups == 1) {
+        x.hg = 0;
+        x.r = rd;
+    } else {
+        x.hg = rd / rounds_per_hg;
+        x.r = rd - x.hg * rounds_per_hg;
+    }
+    return x;
+}
+
 // ---- unit descriptors --------------------------------------------------------
 // Everything a round needs about its unit is fetched with per-lane vector loads
 // one or two rounds ahead and turned into wave-uniform values with readlane just
