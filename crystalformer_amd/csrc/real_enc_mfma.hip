@@ -319,11 +319,16 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                     sn = ring_s[slot];
                     bitsn = ring_bits[slot];
                     float w = exp2_hw(a2 * (d2t - d2min));
-                    w = (col_on && ((bits >> c) & 1)) ? w : 0.f;
+                    // (fixed cube: every staged translation is inside every column's box, and the
+                    // padding records carry d2 = +inf, i.e. weight 0)
+                    w = (col_on && (UNIFORM || ((bits >> c) & 1))) ? w : 0.f;
                     sum += w;
+                    // tiles within reach of any of the group's 4 translations (one record per q)
+                    const int reach = __builtin_amdgcn_readlane(bits, 0) | __builtin_amdgcn_readlane(bits, 16) |
+                                      __builtin_amdgcn_readlane(bits, 32) | __builtin_amdgcn_readlane(bits, 48);
 #pragma unroll
                     for (int m = 0; m < NT; m++) {
-                        if (__ballot((bits & (0x10000 << m)) != 0) != 0ull) {     // wave-uniform
+                        if (reach & (0x10000 << m)) {                             // wave-uniform
                             float b = ck[m] - st;
                             float gm = exp2_hw(-(b * b));
                             acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, w, acc[m], 0, 0, 0);

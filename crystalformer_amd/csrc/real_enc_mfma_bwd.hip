@@ -240,9 +240,12 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                     const float w = on ? exp2_hw(a2 * d2t - z2) : 0.f;
                     const float wd = on ? w * d2t : 0.f;
                     px += wd;
+                    // tiles within reach of any of the group's 4 translations (one record per q)
+                    const int reach = __builtin_amdgcn_readlane(bits, 0) | __builtin_amdgcn_readlane(bits, 16) |
+                                      __builtin_amdgcn_readlane(bits, 32) | __builtin_amdgcn_readlane(bits, 48);
 #pragma unroll
                     for (int m = 0; m < NT; m++) {
-                        if (__ballot((bits & (0x10000 << m)) != 0) != 0ull) {
+                        if (reach & (0x10000 << m)) {
                             float b = ck[m] - st;
                             float gm = exp2_hw(-(b * b));
                             accS[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, w, accS[m], 0, 0, 0);
@@ -310,8 +313,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 for (int m = 0; m < NT; m++)
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
-                        const float val = pass == 0 ? accS[m][r] : accQ[m][r];
-                        col[16 * m + 4 * q + r] = col_on ? val : 0.f;
+                        // (inactive columns hold zeros: their weights are masked in the loop)
+                        col[16 * m + 4 * q + r] = pass == 0 ? accS[m][r] : accQ[m][r];
                     }
             }
             __syncthreads();
