@@ -20,6 +20,7 @@ from torch.nn import Module, Parameter
 from torch.nn.init import constant_, normal_, xavier_uniform_
 
 from . import global_config as config
+from . import ops
 from .hip_funcs import (FusedDotProductAttentionCUDA, GaussianExponentsHIP, RealPeriodicEncodingFuncCUDA,
                         RealPeriodicEncodingWithProjFuncCUDA)
 from .params import LatticeformerParams
@@ -70,6 +71,12 @@ def gaussian_exponents(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, ga
                 gauss_scale.copy_(torch.stack([scale, shift]))
     rho = make_positive_func(params.positive_func)(alpha, params.gauss_lb_real)
     return rho * (-0.5 * params.scale_real ** -2)
+
+
+def inference_only(*tensors: Optional[Tensor]) -> bool:
+    """True when no gradient can be asked of an op on these tensors: the fused
+    row-block linear kernels (no autograd) may then replace F.linear."""
+    return not torch.is_grad_enabled() or not any(t is not None and t.requires_grad for t in tensors)
 
 
 def fused_exponents_spec(params: LatticeformerParams):
@@ -197,7 +204,9 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                 edges: Tensor, points: Tensor, dist2_min: Optional[Tensor], tvecs: Tensor,
                 kr_base: Optional[Tensor] = None, rvecs: Optional[Tensor] = None,
                 vcell: Optional[Tensor] = None, onehot: Optional[Tensor] = None,
-                need_weights: bool = True) -> Tuple[Tensor, Optional[Tensor]]:
+                need_weights: bool = True, residual: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
+        """Same arguments as the reference module; ``residual`` (an extension, default None)
+        is added to the output projection, in its epilogue on the inference path."""
         P = self.params
         H = self.num_heads
         n = query.shape[0]
@@ -205,9 +214,21 @@ class CrystalformerMultiheadAttentionCUDA(Module):
         b_q = b_k = b_v = None
         if self.in_proj_bias is not None:
             b_q, b_k, b_v = self.in_proj_bias.split([kd, kd, vd])
-        q = F.linear(query, self.q_proj_weight, b_q).contiguous().view(n, H, kd // H)
-        k = F.linear(key, self.k_proj_weight, b_k).contiguous().view(key.shape[0], H, kd // H)
-        v = F.linear(value, self.v_proj_weight, b_v).contiguous().view(value.shape[0], H, vd // H)
+        fused_linear = (query is key and key is value and kd == vd
+                        and inference_only(query, self.q_proj_weight, self.k_proj_weight, self.v_proj_weight,
+                                           self.in_proj_bias, self.out_proj.weight, self.out_proj.bias, residual)
+                        and ops.linear_rows_supported(query, self.q_proj_weight, self.k_proj_weight,
+                                                      self.v_proj_weight)
+                        and vd % 16 == 0)
+        if fused_linear:
+            # the three projections in one launch
+            q, k, v = ops.linear_rows(query, (self.q_proj_weight, self.k_proj_weight, self.v_proj_weight),
+                                      self.in_proj_bias)
+            q, k, v = q.view(n, H, kd // H), k.view(n, H, kd // H), v.view(n, H, vd // H)
+        else:
+            q = F.linear(query, self.q_proj_weight, b_q).contiguous().view(n, H, kd // H)
+            k = F.linear(key, self.k_proj_weight, b_k).contiguous().view(key.shape[0], H, kd // H)
+            v = F.linear(value, self.v_proj_weight, b_v).contiguous().view(value.shape[0], H, vd // H)
 
         bias = values = qs = None
         if P.domain == "real":
@@ -251,7 +272,12 @@ class CrystalformerMultiheadAttentionCUDA(Module):
         else:
             attn = loop_attention(qs, k, v, batch_q, edges, bias, values)
         attn = attn.contiguous().view(n, vd)
-        attn = F.linear(attn, self.out_proj.weight, self.out_proj.bias)
+        if fused_linear:
+            attn, = ops.linear_rows(attn, (self.out_proj.weight,), self.out_proj.bias, residual=residual)
+        else:
+            attn = F.linear(attn, self.out_proj.weight, self.out_proj.bias)
+            if residual is not None:
+                attn = residual + attn
         if need_weights:
             raise NotImplementedError("need_weights=True: attention weights are not returned by the fused path")
         return attn, values

@@ -112,4 +112,28 @@ class Latticeformer(nn.Module):
         x = self.encoder(x, data.pos, data.batch, data.trans_vec, data.sizes, data.x)
         x = self.proj_before_pooling(x)
         x = self.pooling_layer(x, data.batch, data.sizes)
-        return self.mlp(x)
+        return self._head(x)
+
+    def _head(self, x):
+        """The regression head; on the inference path each Linear (+ ReLU) of a head without
+        norm layers is one row-block launch instead of a library GEMM plus elementwise launches."""
+        from . import ops
+        from .attention import inference_only
+        mods = list(self.mlp)
+        plain = all(isinstance(m, (nn.Linear, nn.ReLU, nn.Identity)) for m in mods)
+        if not (plain and x.is_cuda and inference_only(x, *self.mlp.parameters())):
+            return self.mlp(x)
+        i = 0
+        while i < len(mods):
+            m = mods[i]
+            if isinstance(m, nn.Linear) and ops.linear_rows_supported(x, m.weight):
+                j = i + 1
+                while j < len(mods) and isinstance(mods[j], nn.Identity):
+                    j += 1
+                relu = j < len(mods) and isinstance(mods[j], nn.ReLU)
+                x, = ops.linear_rows(x, (m.weight,), m.bias, relu=relu)
+                i = j + 1 if relu else j
+            else:
+                x = m(x)
+                i += 1
+        return x

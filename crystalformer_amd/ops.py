@@ -527,3 +527,39 @@ def gauss_exponents(q_ihd: Tensor, w_hd: Tensor, gauss_scale: Optional[Tensor], 
                                     ptr(alpha_n), ptr(a), ptr(qs), stream_handle(dev))
     check(rc, "cf_gauss_exponents")
     return a, qs, alpha_n, (ws[-4:-2] if normalize else None)
+
+
+def linear_rows_supported(x: Tensor, *weights: Tensor) -> bool:
+    """True when :func:`linear_rows` serves these operands (float32 on the GPU, input
+    width a multiple of 16, equal weight shapes)."""
+    if not x.is_cuda or x.dtype != torch.float32 or x.dim() != 2 or x.shape[1] % 16 != 0:
+        return False
+    return all(w.is_cuda and w.dtype == torch.float32 and w.dim() == 2 and w.shape == weights[0].shape
+               and w.shape[1] == x.shape[1] for w in weights) and 1 <= len(weights) <= 3
+
+
+def linear_rows(x: Tensor, weights, bias: Optional[Tensor] = None, residual: Optional[Tensor] = None,
+                relu: bool = False):
+    """``act(x @ w.T + b) (+ residual)`` for up to three equally shaped weights in one
+    launch; returns a tuple of outputs, one per weight.  No autograd."""
+    weights = [_f32(w, "weight") for w in weights]
+    dev = require_device(x, *weights, bias, residual)
+    x = _f32(x, "x")
+    bias = _f32(bias, "bias")
+    residual = _f32(residual, "residual")
+    N, K = x.shape
+    C = weights[0].shape[0]
+    if any(w.shape != (C, K) for w in weights):
+        raise _lib.CrystalformerHipError("linear_rows: weights must all be (C, K) with K = x.shape[1]")
+    if bias is not None and bias.numel() != len(weights) * C:
+        raise _lib.CrystalformerHipError("linear_rows: bias must have one entry per output column")
+    if residual is not None and (len(weights) != 1 or residual.shape != (N, C)):
+        raise _lib.CrystalformerHipError("linear_rows: residual must be (N, C) with a single weight")
+    ys = [torch.empty((N, C), dtype=torch.float32, device=dev) for _ in weights]
+    pw = [ptr(w) for w in weights] + [None] * (3 - len(weights))
+    py = [ptr(y) for y in ys] + [None] * (3 - len(weights))
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_linear_rows(ptr(x), N, K, pw[0], pw[1], pw[2], len(weights), C, ptr(bias),
+                                        ptr(residual), int(bool(relu)), py[0], py[1], py[2], stream_handle(dev))
+    check(rc, "cf_linear_rows")
+    return tuple(ys)

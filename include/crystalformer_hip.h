@@ -260,6 +260,23 @@ int cf_gauss_exponents(const float *q_ihd, const float *w_hd, float *gauss_scale
                        int64_t workspace_bytes, float *alpha_n, float *a_ih, float *q_scaled,
                        void *stream);
 
+/*
+ * Row-block linear layer(s): y_w = act(x W_w^T + b_w) (+ residual), w < n_weights <= 3,
+ * for the small dense layers around the attention: the query/key/value
+ * projections in one launch (models/indexed_lattice_multi_head_attention_cuda.py:865-867,
+ * three F.linear calls), the output projection with its residual and the two
+ * feed-forward layers with ReLU / residual fused
+ * (models/indexed_latticeformer_encoder.py:806-826, F.linear + activation + add).
+ * fp32 on the matrix cores; inference path (no autograd).
+ *   x (N,K), K a multiple of 16;  w0..w2 each (C,K) row-major;  bias (n_weights*C) nullable
+ *   residual (N,C) nullable, only with n_weights == 1;  relu != 0 applies max(.,0) last
+ * Outputs
+ *   y0..y2 each (N,C)
+ */
+int cf_linear_rows(const float *x, int64_t N, int64_t K, const float *w0, const float *w1,
+                   const float *w2, int n_weights, int64_t C, const float *bias,
+                   const float *residual, int relu, float *y0, float *y1, float *y2, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -451,3 +451,23 @@ def test_batch_layout_bit_exact_and_cached(dev):
     assert other is not lay and other.num_edges == 8
     with pytest.raises(lib.CrystalformerHipError):
         ops.batch_layout(torch.tensor([2, 2], device=dev), torch.tensor([0, 0, 1], device=dev))
+
+
+@pytest.mark.parametrize("N,K,C,nw", [(1774, 128, 128, 3), (1774, 128, 512, 1), (1774, 512, 128, 1), (5, 16, 7, 2),
+                                      (33, 48, 100, 1), (64, 64, 64, 3)])
+def test_linear_rows(dev, N, K, C, nw):
+    g = torch.Generator().manual_seed(N + C)
+    x = torch.randn(N, K, generator=g)
+    ws = [torch.randn(C, K, generator=g) * K ** -0.5 for _ in range(nw)]
+    bias = torch.randn(nw * C, generator=g)
+    ys = ops.linear_rows(x.to(dev), [w.to(dev) for w in ws], bias.to(dev))
+    for i, (w, y) in enumerate(zip(ws, ys)):
+        ref = (x.double() @ w.double().T + bias[i * C:(i + 1) * C].double()).float()
+        assert_close(y, ref, f"y{i}", rtol=2e-6)
+    if nw == 1:
+        res = torch.randn(N, C, generator=g)
+        y, = ops.linear_rows(x.to(dev), [ws[0].to(dev)], None, residual=res.to(dev), relu=True)
+        ref = torch.relu(x.double() @ ws[0].double().T + res.double()).float()
+        assert_close(y, ref, "relu(x w^T + r)", rtol=2e-6)
+    with pytest.raises(lib.CrystalformerHipError):
+        ops.linear_rows(torch.randn(4, 10).to(dev), [torch.randn(3, 10).to(dev)])
