@@ -22,90 +22,103 @@ struct LinArgs {
     int K, C, nw, relu;
 };
 
-constexpr int LIN_ROWS = 16;   // rows per work-group
-constexpr int LIN_COLS = 32;   // columns per work-group (two 16 x 16 accumulator tiles)
-constexpr int LIN_WAVES = 4;   // wavefronts per work-group, splitting the reduction dimension
+constexpr int LIN_KC = 32;         // reduction chunk staged in LDS
+constexpr int LIN_LD = LIN_KC + 4; // LDS row stride (floats): 16-byte aligned, staggers the banks
 
-// A work-group owns 16 rows x 32 columns; its 4 wavefronts take the 16-wide k-steps
-// round robin (few dependent loads per wavefront: these layers are latency, not
-// throughput) and wavefront 0 adds the partial tiles from LDS and runs the epilogue.
-// Lane (q, c) = (lane / 16, lane % 16) loads 16 bytes of row c of X and of rows c, c + 16
-// of W at k = 16 s + 4 q: four MFMA steps per load, step r reducing over
-// k = 16 s + 4 q' + r (q' = 0..3) in both operands.
-__global__ __launch_bounds__(64 * LIN_WAVES) void linear_rows_kernel(LinArgs p)
+// LDS-tiled: a work-group of 4 wavefronts (WR x WC) owns TM rows x TN columns; every 32-wide
+// chunk of the reduction is staged once in LDS (X tile and W tile, 16-byte global loads held
+// in registers while the previous chunk is multiplied) and read back as MFMA operands:
+// lane (q, c) = (lane / 16, lane % 16) reads 16 bytes of row c of a 16-row tile at
+// k = 16 s + 4 q, four MFMA steps per read, step r reducing over k = 16 s + 4 q' + r.
+template <int TM, int TN, int WR, int WC>
+__global__ __launch_bounds__(256) void linear_rows_kernel(LinArgs p)
 {
-    __shared__ float part[LIN_WAVES - 1][8][WAVE];
+    constexpr int MT = TM / (16 * WR), NT = TN / (16 * WC);     // 16 x 16 tiles per wavefront
+    constexpr int XL = TM / 32, WL = TN / 32;                   // 16-byte loads per thread and chunk
+    __shared__ __align__(16) float xs[TM * LIN_LD];
+    __shared__ __align__(16) float ws[TN * LIN_LD];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int q = lane >> 4, c = lane & 15;
-    const int64_t row0 = (int64_t)blockIdx.x * LIN_ROWS;
-    const int col0 = blockIdx.y * LIN_COLS;                         // column over all weights
+    const int wr = wave / WC, wc = wave - wr * WC;
+    const int64_t row0 = (int64_t)blockIdx.x * TM;
+    const int col0 = blockIdx.y * TN;                           // column over all weights
     const int total_cols = p.nw * p.C;
-    const int64_t arow = min(row0 + c, p.N - 1);
-    const float *xa = p.x + arow * p.K + 4 * q;
-    const float *wb[2];
+    // staging role: thread -> (row t/8 (+32 u), 16-byte piece t%8) of a tile
+    const int srow = threadIdx.x >> 3, spiece = threadIdx.x & 7;
+    const float *xg[XL];
+    const float *wg[WL];
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
-        const int col = min(col0 + 16 * t + c, total_cols - 1);
+    for (int u = 0; u < XL; u++) xg[u] = p.x + min(row0 + srow + 32 * u, p.N - 1) * p.K + 4 * spiece;
+#pragma unroll
+    for (int u = 0; u < WL; u++) {
+        const int col = min(col0 + srow + 32 * u, total_cols - 1);
         const int wi = col / p.C;
-        wb[t] = p.w[wi] + (int64_t)(col - wi * p.C) * p.K + 4 * q;
+        wg[u] = p.w[wi] + (int64_t)(col - wi * p.C) * p.K + 4 * spiece;
     }
-    float4_t acc[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
-    auto step = [&](const float4_t &a, const float4_t &b0, const float4_t &b1) {
+    float4_t acc[MT][NT];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[r], b0[r], acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[r], b1[r], acc[1], 0, 0, 0);
-        }
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) acc[mt][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    float4_t xr[XL], wrg[WL];
+    auto fetch = [&](int k0) {
+        const bool in = k0 + 4 * spiece < p.K;                  // K is a multiple of 4
+#pragma unroll
+        for (int u = 0; u < XL; u++) xr[u] = in ? *reinterpret_cast<const float4_t *>(xg[u] + k0) : zero4;
+#pragma unroll
+        for (int u = 0; u < WL; u++) wrg[u] = in ? *reinterpret_cast<const float4_t *>(wg[u] + k0) : zero4;
     };
-    const int stride = 16 * LIN_WAVES;
-    int k0 = 16 * wave;
-    for (; k0 + 3 * stride < p.K; k0 += 4 * stride) {     // 12 loads in flight, then 32 MFMAs
-        float4_t a[4], b0[4], b1[4];
+    fetch(0);
+    for (int k0 = 0; k0 < p.K; k0 += LIN_KC) {
+        __syncthreads();                                        // previous chunk fully consumed
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            a[u] = *reinterpret_cast<const float4_t *>(xa + k0 + stride * u);
-            b0[u] = *reinterpret_cast<const float4_t *>(wb[0] + k0 + stride * u);
-            b1[u] = *reinterpret_cast<const float4_t *>(wb[1] + k0 + stride * u);
+        for (int u = 0; u < XL; u++)
+            *reinterpret_cast<float4_t *>(xs + (srow + 32 * u) * LIN_LD + 4 * spiece) = xr[u];
+#pragma unroll
+        for (int u = 0; u < WL; u++)
+            *reinterpret_cast<float4_t *>(ws + (srow + 32 * u) * LIN_LD + 4 * spiece) = wrg[u];
+        __syncthreads();
+        if (k0 + LIN_KC < p.K) fetch(k0 + LIN_KC);              // in flight during the MFMAs below
+#pragma unroll
+        for (int ss = 0; ss < LIN_KC / 16; ss++) {
+            float4_t a[MT], b[NT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+                a[mt] = *reinterpret_cast<const float4_t *>(xs + ((wr * MT + mt) * 16 + c) * LIN_LD + 16 * ss + 4 * q);
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+                b[nt] = *reinterpret_cast<const float4_t *>(ws + ((wc * NT + nt) * 16 + c) * LIN_LD + 16 * ss + 4 * q);
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[mt][r], b[nt][r], acc[mt][nt], 0, 0, 0);
         }
-#pragma unroll
-        for (int u = 0; u < 4; u++) step(a[u], b0[u], b1[u]);
     }
-    for (; k0 < p.K; k0 += stride)
-        step(*reinterpret_cast<const float4_t *>(xa + k0), *reinterpret_cast<const float4_t *>(wb[0] + k0),
-             *reinterpret_cast<const float4_t *>(wb[1] + k0));
-    if (wave > 0) {
+    // lane (q, c) of tile (mt, nt) holds rows .. + 4 q + r, column .. + c
 #pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) part[wave - 1][4 * t + r][lane] = acc[t][r];
-    }
-    __syncthreads();
-    if (wave > 0) return;
-#pragma unroll
-    for (int w = 0; w < LIN_WAVES - 1; w++)
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) acc[t][r] += part[w][4 * t + r][lane];
-    // lane (q, c) holds rows row0 + 4 q + r, column col0 + 16 t + c
-#pragma unroll
-    for (int t = 0; t < 2; t++) {
-        const int col = col0 + 16 * t + c;
+    for (int nt = 0; nt < NT; nt++) {
+        const int col = col0 + (wc * NT + nt) * 16 + c;
         if (col >= total_cols) continue;
         const int wi = col / p.C;
         const int lc = col - wi * p.C;
         const float bv = p.bias ? p.bias[col] : 0.f;
         float *y = p.y[wi];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int64_t row = row0 + 4 * q + r;
-            if (row >= p.N) continue;
-            float v = acc[t][r] + bv;
-            if (p.res) v += p.res[row * p.C + lc];
-            if (p.relu) v = fmaxf(v, 0.f);
-            y[row * p.C + lc] = v;
-        }
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int64_t row = row0 + (wr * MT + mt) * 16 + 4 * q + r;
+                if (row >= p.N) continue;
+                float v = acc[mt][nt][r] + bv;
+                if (p.res) v += p.res[row * p.C + lc];
+                if (p.relu) v = fmaxf(v, 0.f);
+                y[row * p.C + lc] = v;
+            }
     }
 }
 
@@ -136,10 +149,16 @@ extern "C" int cf_linear_rows(const float *x, int64_t N, int64_t K, const float 
     }
     p.bias = bias; p.res = residual;
     p.N = N; p.K = (int)K; p.C = (int)C; p.nw = n_weights; p.relu = relu;
-    const int64_t gx = (N + LIN_ROWS - 1) / LIN_ROWS;
-    const int64_t gy = ((int64_t)n_weights * C + LIN_COLS - 1) / LIN_COLS;
+    // wide outputs: 64 x 64 tiles (2 x 2 wavefronts); narrow ones: 64 x 32 (4 x 1), more work-groups
+    const int64_t total_cols = (int64_t)n_weights * C;
+    const bool wide = total_cols >= 256;
+    const int64_t gx = (N + 63) / 64;
+    const int64_t gy = (total_cols + (wide ? 63 : 31)) / (wide ? 64 : 32);
     CF_REQUIRE(gx < (1ll << 31) && gy < 65536, CF_ERR_UNSUPPORTED, "cf_linear_rows: too large");
-    linear_rows_kernel<<<dim3((unsigned)gx, (unsigned)gy), 64 * LIN_WAVES, 0, (hipStream_t)stream>>>(p);
+    if (wide)
+        linear_rows_kernel<64, 64, 2, 2><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
+    else
+        linear_rows_kernel<64, 32, 4, 1><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
     CF_CHECK_LAUNCH("cf_linear_rows");
     return CF_OK;
 }
