@@ -81,7 +81,7 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
     bwd_ms = avg("real_enc_bwd")
     roofline = {
         "kernel": "real_enc_bwd_pair_kernel + reductions (periodic encoding backward)",
-        "bound": "valu", "achieved": round(flop_bwd / (bwd_ms * 1e-3) / 1e12, 3) if bwd_ms > 0 else 0.0,
+        "bound": "mfma", "achieved": round(flop_bwd / (bwd_ms * 1e-3) / 1e12, 3) if bwd_ms > 0 else 0.0,
         "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
         "frac": round(flop_bwd / (bwd_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4) if bwd_ms > 0 else 0.0,
         "traffic": None, "avg_launch_ms": bwd_ms,
@@ -262,7 +262,7 @@ def main() -> int:
     achieved_tflops = flop_launch / (enc_avg_ms * 1e-3) / 1e12 if enc_avg_ms > 0 else 0.0
     roofline = {
         "kernel": "real_enc_fwd_pair_kernel (periodic encoding forward, projection fused)",
-        "bound": "valu",
+        "bound": "mfma",
         "achieved": round(achieved_tflops, 3),
         "peak": PEAK_FP32_TFLOPS,
         "unit": "TFLOP/s",
