@@ -154,13 +154,22 @@ __device__ __forceinline__ void wave_mem_sync()
 }
 
 // Translation half-width along one axis: ceil((cutoff+0.01f)*rvl / (2*pi)),
-// float product, double quotient.
+// float product, double quotient.  The double division only runs where it can
+// matter: a float quotient is within 1.3e-7 relative of the exact one, so its
+// ceiling is already the answer unless it lies that close to an integer.
 __device__ __forceinline__ int range_axis(float cutoff, float rvl, int minimum_range)
 {
-    float num = (cutoff + 0.01f) * rvl;
-    double q = ceil((double)num / (2.0 * (double)PI_F));
-    int r = (q >= 0.0 && q <= (double)MAX_RANGE) ? (int)q : (q > (double)MAX_RANGE ? MAX_RANGE : 0);
-    if (q != q) r = MAX_RANGE;  // NaN exponent: bounded loop, result is NaN anyway
+    const float num = (cutoff + 0.01f) * rvl;
+    const float qf = num * (float)(1.0 / (2.0 * (double)PI_F));
+    int r;
+    if (fabsf(qf - rintf(qf)) > 1.0e-6f * fabsf(qf) && fabsf(qf) < 1.0e6f) {
+        const float c = ceilf(qf);
+        r = c <= 0.f ? 0 : (c > (float)MAX_RANGE ? MAX_RANGE : (int)c);
+    } else {
+        const double q = ceil((double)num / (2.0 * (double)PI_F));
+        r = (q >= 0.0 && q <= (double)MAX_RANGE) ? (int)q : (q > (double)MAX_RANGE ? MAX_RANGE : 0);
+        if (q != q) r = MAX_RANGE;  // NaN exponent: bounded loop, result is NaN anyway
+    }
     return max(r, minimum_range);
 }
 

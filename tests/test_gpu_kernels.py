@@ -240,6 +240,33 @@ def test_translation_ranges_bit_exact(dev, cutoff, lr, mr):
     assert got.dtype == torch.int32 and torch.equal(got, ref)
 
 
+def test_translation_ranges_at_integer_quotients(dev):
+    """Half-widths where (cutoff + 0.01) * |b| / 2 pi sits on, or within a few float ulps of, an
+    integer: the ceiling must come from the double quotient there (the kernel only takes its float
+    shortcut away from integers)."""
+    two_pi = 2.0 * float(torch.tensor(3.141592654, dtype=torch.float32))
+    cutoff = 3.0
+    ks_int = torch.arange(1, 41, dtype=torch.float64)
+    base = (ks_int * two_pi / (float(torch.tensor(cutoff, dtype=torch.float32)) + float(torch.tensor(0.01, dtype=torch.float32)))).float()
+    variants = [base]
+    for _ in range(3):
+        variants.append(torch.nextafter(variants[-1], torch.full_like(base, 1e9)))
+    lo = base
+    for _ in range(3):
+        lo = torch.nextafter(lo, torch.zeros_like(base))
+        variants.append(lo)
+    rv = torch.stack(variants).reshape(-1)                      # 280 reciprocal lengths
+    B = rv.numel()
+    rvlen = torch.stack([rv, rv.flip(0), rv.roll(7)], dim=1).contiguous()
+    batch = torch.arange(B)
+    a = -torch.rand(B, 8, generator=torch.Generator().manual_seed(2)) - 0.1
+    for mr in (0, 2):
+        got = ops.translation_ranges(a.to(dev), rvlen.to(dev), batch.to(dev), cutoff, 2, mr).cpu()
+        ref = ks.translation_ranges(a, rvlen, batch, cutoff, 2, mr)
+        assert torch.equal(got, ref)
+    assert int(ref.max()) >= 40 and len(set(ref[:, 0, 0].tolist())) > 30
+
+
 def test_empty_and_single_atom_inputs(dev):
     # no crystals at all
     z, v = ops.real_enc_fwd(torch.zeros(0, 8, device=dev), torch.zeros(0, 3, device=dev),
