@@ -28,7 +28,7 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
                               const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
                               int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
                               int64_t W_num, const float *rvlen, float cutoff, int lattice_range,
-                              int min_range, float *z, float *v, hipStream_t st);
+                              int min_range, unsigned int *sched, float *z, float *v, hipStream_t st);
 
 // real_enc_mfma_bwd.hip
 int real_enc_bwd_pairs_blocks(int64_t U, int64_t H);

@@ -847,7 +847,8 @@ extern "C" int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const 
                                int64_t E, int64_t B, int64_t K, int64_t D, double dist_max,
                                double wscale, const float *W_k, int64_t W_num, const float *rvlen_n,
                                double cutoff_radius, int lattice_range, int minimum_range,
-                               const int64_t *pairs_u, int64_t U, float *z_ek, float *v_ekd, void *stream)
+                               const int64_t *pairs_u, int64_t U, int32_t *sched_2, float *z_ek, float *v_ekd,
+                               void *stream)
 {
     EncArgs p;
     int rc = fill_args(p, "cf_real_enc_fwd", a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, N, H, E, B, K,
@@ -865,7 +866,8 @@ extern "C" int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const 
     if (pairs_u) {
         rc = launch_real_enc_fwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, N, H, E, K, D,
                                        p.bin_step, p.s_scale, p.W, W_num, rvlen_n, p.cutoff, lattice_range,
-                                       minimum_range, z_ek, v_ekd, (hipStream_t)stream);
+                                       minimum_range, reinterpret_cast<unsigned int *>(sched_2), z_ek, v_ekd,
+                                       (hipStream_t)stream);
         if (rc == CF_OK) {
             CF_CHECK_LAUNCH("cf_real_enc_fwd (pairs)");
             return CF_OK;

@@ -21,6 +21,7 @@ struct PairArgs {
     const float *rvlen;
     float *z;
     float *v;
+    unsigned int *sched;    // forward only, nullable: {next ticket, finished work-groups}, both 0 at launch
     // backward only
     const float *z_in;      // (E,H) forward output
     const float *gz;        // (E,H), nullable

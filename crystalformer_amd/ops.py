@@ -133,6 +133,25 @@ def crystal_offsets(batch_i: Tensor, num_slots: Optional[int] = None) -> Tuple[T
     return atom_start, edge_start
 
 
+# Scheduling words of the pair-evaluated forward (two zeroed int32 the work-groups draw their
+# rounds from; the kernel leaves them zeroed).  Launches that may overlap need words of their
+# own: eager launches on one stream run in order and share one pair per (device, stream); under
+# stream capture every launch gets a fresh zero-filled pair, because graphs captured on one
+# stream can later be replayed side by side.
+DYNAMIC_ROUNDS = True
+_sched_words: dict = {}
+
+
+def _scheduling_words(dev: torch.device) -> Tensor:
+    if torch.cuda.is_current_stream_capturing():
+        return torch.zeros(2, dtype=torch.int32, device=dev)
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    words = _sched_words.get(key)
+    if words is None:
+        words = _sched_words[key] = torch.zeros(2, dtype=torch.int32, device=dev)
+    return words
+
+
 def real_enc_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor,
                  K: int, dist_max: float, wscale: float, W_k: Optional[Tensor] = None,
                  rvlen_n: Optional[Tensor] = None, cutoff_radius: Optional[float] = None,
@@ -167,7 +186,9 @@ def real_enc_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
             ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), N, H, E, B, K, D,
             float(dist_max), float(wscale), ptr(W_k if K > 0 else None), W_num,
             ptr(rvlen_n), cutoff, int(lattice_range), int(minimum_range), ptr(pairs_u),
-            0 if pairs_u is None else pairs_u.shape[0], ptr(z), ptr(v), stream_handle(dev))
+            0 if pairs_u is None else pairs_u.shape[0],
+            ptr(_scheduling_words(dev) if (pairs_u is not None and DYNAMIC_ROUNDS) else None),
+            ptr(z), ptr(v), stream_handle(dev))
     check(rc, "cf_real_enc_fwd")
     return z, v
 

@@ -67,6 +67,12 @@ int cf_max_translation_range(void);
  *             appear in exactly one descriptor and its reverse must carry
  *             rpos = -rpos.  NULL selects the per-edge kernels, which accept
  *             any edge list.
+ *   sched_2   nullable, with pairs_u only: two int32 words holding 0.  With them the
+ *             work-groups draw their rounds of units from a shared counter (they finish
+ *             together whatever the units cost); without, rounds are dealt out in a fixed
+ *             stride.  Results are identical bit for bit either way.  The words are 0 again
+ *             when the launch completes and may serve the next launch on the same stream;
+ *             launches that can overlap in time need words of their own.
  * Outputs
  *   z_ek  (E,H)                       log sum_n exp(a d^2)
  *   v_ekd nullable if K==0; (E,H,K) when W_k is NULL, else (E,H,D)
@@ -76,7 +82,7 @@ int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvec
                     int64_t N, int64_t H, int64_t E, int64_t B, int64_t K, int64_t D,
                     double dist_max, double wscale, const float *W_k, int64_t W_num,
                     const float *rvlen_n, double cutoff_radius, int lattice_range,
-                    int minimum_range, const int64_t *pairs_u, int64_t U,
+                    int minimum_range, const int64_t *pairs_u, int64_t U, int32_t *sched_2,
                     float *z_ek, float *v_ekd, void *stream);
 
 /*

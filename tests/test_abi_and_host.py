@@ -40,19 +40,19 @@ def test_argument_validation_needs_no_device():
     null = ctypes.c_void_p(0)
     # unsupported head count
     rc = L.cf_real_enc_fwd(null, null, null, null, null, 0, 3, 0, 0, 0, 0, 1.0, 1.0, null, 0, null, 0.0, 2, 0,
-                           null, 0, null, null, null)
+                           null, 0, null, null, null, null)
     assert rc == -2 and b"head count" in L.cf_last_error()
     # K outside range
     rc = L.cf_real_enc_fwd(null, null, null, null, null, 0, 8, 0, 0, 500, 16, 1.0, 1.0, null, 0, null, 0.0, 2, 0,
-                           null, 0, null, null, null)
+                           null, 0, null, null, null, null)
     assert rc == -2 and b"K=" in L.cf_last_error()
     # adaptive cut-off without reciprocal lengths
     rc = L.cf_real_enc_fwd(null, null, null, null, null, 0, 8, 0, 0, 0, 0, 1.0, 1.0, null, 0, null, -3.5, 2, 0,
-                           null, 0, null, null, null)
+                           null, 0, null, null, null, null)
     assert rc == -1 and b"rvlen" in L.cf_last_error()
     # null pointers with work to do
     rc = L.cf_real_enc_fwd(null, null, null, null, null, 4, 8, 16, 1, 0, 0, 1.0, 1.0, null, 0, null, 0.0, 2, 0,
-                           null, 0, null, null, null)
+                           null, 0, null, null, null, null)
     assert rc == -1
     rc = L.cf_fused_dpa_fwd(null, null, null, null, null, null, null, 4, 8, 16, 16, 16, null, null, null)
     assert rc == -1
@@ -62,11 +62,11 @@ def test_argument_validation_needs_no_device():
     assert rc == -1
     # empty problems are fine and launch nothing
     assert L.cf_real_enc_fwd(null, null, null, null, null, 0, 8, 0, 0, 64, 16, 14.0, 1.0, null, 1, null, 0.0, 2,
-                             0, null, 0, null, null, null) == 0
+                             0, null, 0, null, null, null, null) == 0
     # a pair list must have (E + N) / 2 entries
     one = ctypes.c_void_p(8)
     rc = L.cf_real_enc_fwd(one, one, one, one, one, 4, 8, 16, 1, 64, 16, 14.0, 1.0, one, 1, null, 0.0, 2, 0,
-                           one, 7, one, one, null)
+                           one, 7, null, one, one, null)
     assert rc == -1 and b"pair list" in L.cf_last_error()
     assert L.cf_irregular_mean_fwd(null, null, 0, 128, null, null) == 0
     assert L.cf_edge_index(null, null, 0, 0, null, null, null, null) == 0
