@@ -498,3 +498,29 @@ def test_linear_rows(dev, N, K, C, nw):
         assert_close(y, ref, "relu(x w^T + r)", rtol=2e-6)
     with pytest.raises(lib.CrystalformerHipError):
         ops.linear_rows(torch.randn(4, 10).to(dev), [torch.randn(3, 10).to(dev)])
+
+
+def test_real_enc_fwd_ticket_rounds_are_bit_identical(dev):
+    """Enough units for the shared-counter scheduling to engage (>= 16 rounds per work-group):
+    same bits as the fixed stride, scheduling words handed back zeroed, launch after launch."""
+    p = Problem([256, 256], H=8, K=16, D=8, seed=41)
+    a, rpos, tv, bt, ed, W, rv = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.W, p.rvlen)
+    pairs = ops.edge_pairs(p.b.sizes.to(dev))
+    assert (pairs.shape[0] + 7) // 8 >= 16 * 512
+    for cutoff in (0.0, -3.5):
+        ops.DYNAMIC_ROUNDS = False
+        try:
+            z0, v0 = ops.real_enc_fwd(a, rpos, tv, bt, ed, 16, p.dist_max, 1.0, W, rv, cutoff, 1, 0, pairs_u=pairs)
+        finally:
+            ops.DYNAMIC_ROUNDS = True
+        for _ in range(3):
+            z1, v1 = ops.real_enc_fwd(a, rpos, tv, bt, ed, 16, p.dist_max, 1.0, W, rv, cutoff, 1, 0, pairs_u=pairs)
+            assert torch.equal(z0, z1) and torch.equal(v0, v1)
+            words = ops._scheduling_words(dev)
+            assert words.tolist() == [0, 0]
+    # a sample of edges against the oracle
+    sel = torch.arange(0, p.E, 997)
+    sub_z, sub_v = ks.real_enc_fwd(p.a, p.rpos[sel], p.b.trans_vec, p.b.batch,
+                                   p.edges[:, sel], 16, p.dist_max, 1.0, p.W, p.rvlen, -3.5, 1, 0)
+    assert_close(z1.cpu()[sel], sub_z, "z sample")
+    assert_close(v1.cpu()[sel], sub_v, "v sample")
