@@ -500,13 +500,14 @@ def test_linear_rows(dev, N, K, C, nw):
         ops.linear_rows(torch.randn(4, 10).to(dev), [torch.randn(3, 10).to(dev)])
 
 
-def test_real_enc_fwd_ticket_rounds_are_bit_identical(dev):
+@pytest.mark.parametrize("sizes,H", [([256, 256], 8), ([200, 200], 16)])
+def test_real_enc_fwd_ticket_rounds_are_bit_identical(dev, sizes, H):
     """Enough units for the shared-counter scheduling to engage (>= 16 rounds per work-group):
     same bits as the fixed stride, scheduling words handed back zeroed, launch after launch."""
-    p = Problem([256, 256], H=8, K=16, D=8, seed=41)
+    p = Problem(sizes, H=H, K=16, D=8, seed=41)
     a, rpos, tv, bt, ed, W, rv = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.W, p.rvlen)
     pairs = ops.edge_pairs(p.b.sizes.to(dev))
-    assert (pairs.shape[0] + 7) // 8 >= 16 * 512
+    assert ((pairs.shape[0] + 7) // 8) * ((H + 7) // 8) >= 16 * 512
     for cutoff in (0.0, -3.5):
         ops.DYNAMIC_ROUNDS = False
         try:
