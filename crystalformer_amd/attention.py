@@ -21,6 +21,7 @@ from torch.nn.init import constant_, normal_, xavier_uniform_
 
 from . import global_config as config
 from . import ops
+from .hip_funcs import linear as linear_hip
 from .hip_funcs import (FusedDotProductAttentionCUDA, GaussianExponentsHIP, RealPeriodicEncodingFuncCUDA,
                         RealPeriodicEncodingWithProjFuncCUDA)
 from .params import LatticeformerParams
@@ -226,9 +227,9 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                                       self.in_proj_bias)
             q, k, v = q.view(n, H, kd // H), k.view(n, H, kd // H), v.view(n, H, vd // H)
         else:
-            q = F.linear(query, self.q_proj_weight, b_q).contiguous().view(n, H, kd // H)
-            k = F.linear(key, self.k_proj_weight, b_k).contiguous().view(key.shape[0], H, kd // H)
-            v = F.linear(value, self.v_proj_weight, b_v).contiguous().view(value.shape[0], H, vd // H)
+            q = linear_hip(query, self.q_proj_weight, b_q).contiguous().view(n, H, kd // H)
+            k = linear_hip(key, self.k_proj_weight, b_k).contiguous().view(key.shape[0], H, kd // H)
+            v = linear_hip(value, self.v_proj_weight, b_v).contiguous().view(value.shape[0], H, vd // H)
 
         bias = values = qs = None
         if P.domain == "real":
@@ -275,7 +276,7 @@ class CrystalformerMultiheadAttentionCUDA(Module):
         if fused_linear:
             attn, = ops.linear_rows(attn, (self.out_proj.weight,), self.out_proj.bias, residual=residual)
         else:
-            attn = F.linear(attn, self.out_proj.weight, self.out_proj.bias)
+            attn = linear_hip(attn, self.out_proj.weight, self.out_proj.bias)
             if residual is not None:
                 attn = residual + attn
         if need_weights:

@@ -368,21 +368,32 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     if (wa_hg >= 0) flush_gW(wa_hg);
 }
 
-// gW[x] = sum over work-groups of part[b][x], fixed order.
-__global__ void gw_blocks_reduce_kernel(const float *part, int blocks, int64_t HDK, float *gW)
+// gW[x] = sum over work-groups of part[b][x], fixed order.  A work-group of 256 threads takes
+// 32 consecutive elements; 8 groups of threads each sum every 8th block (two running sums),
+// and the 8 partial results are added in order through LDS.
+__global__ __launch_bounds__(256) void gw_blocks_reduce_kernel(const float *part, int blocks, int64_t HDK,
+                                                               float *gW)
 {
-    int64_t x = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (x >= HDK) return;
-    float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
-    int b = 0;
-    for (; b + 4 <= blocks; b += 4) {
-        acc0 += part[(int64_t)b * HDK + x];
-        acc1 += part[(int64_t)(b + 1) * HDK + x];
-        acc2 += part[(int64_t)(b + 2) * HDK + x];
-        acc3 += part[(int64_t)(b + 3) * HDK + x];
+    __shared__ float red[8][32];
+    const int ex = threadIdx.x & 31, pt = threadIdx.x >> 5;
+    const int64_t x = (int64_t)blockIdx.x * 32 + ex;
+    float acc0 = 0.f, acc1 = 0.f;
+    if (x < HDK) {
+        int b = pt;
+        for (; b + 8 < blocks; b += 16) {
+            acc0 += part[(int64_t)b * HDK + x];
+            acc1 += part[(int64_t)(b + 8) * HDK + x];
+        }
+        if (b < blocks) acc0 += part[(int64_t)b * HDK + x];
     }
-    for (; b < blocks; b++) acc0 += part[(int64_t)b * HDK + x];
-    gW[x] = (acc0 + acc1) + (acc2 + acc3);
+    red[pt][ex] = acc0 + acc1;
+    __syncthreads();
+    if (pt == 0 && x < HDK) {
+        float total = red[0][ex];
+#pragma unroll
+        for (int g = 1; g < 8; g++) total += red[g][ex];
+        gW[x] = total;
+    }
 }
 
 }  // namespace
@@ -436,7 +447,7 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
 #undef CF_BPAIR
     if (gW_part && gW) {
         const int64_t HDK = H * D * K;
-        gw_blocks_reduce_kernel<<<(int)((HDK + 255) / 256), 256, 0, st>>>(gW_part, blocks, HDK, gW);
+        gw_blocks_reduce_kernel<<<(int)((HDK + 31) / 32), 256, 0, st>>>(gW_part, blocks, HDK, gW);
     }
     return CF_OK;
 }

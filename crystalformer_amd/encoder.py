@@ -21,6 +21,7 @@ from torch.nn.init import constant_, xavier_uniform_
 from . import ops
 from .attention import CrystalformerMultiheadAttentionCUDA
 from .hip_funcs import compile_kernels
+from .hip_funcs import linear as linear_hip
 from .params import LatticeformerParams
 
 
@@ -146,7 +147,8 @@ class CrystalformerEncoderLayerCUDA(Module):
         return self.dropout1(x)
 
     def _ff_block(self, x: Tensor) -> Tensor:
-        return self.dropout2(self.linear2(self.dropout(self.activation(self.linear1(x)))))
+        h = self.activation(linear_hip(x, self.linear1.weight, self.linear1.bias))
+        return self.dropout2(linear_hip(self.dropout(h), self.linear2.weight, self.linear2.bias))
 
 
 class CrystalformerEncoderCUDA(Module):

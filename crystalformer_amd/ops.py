@@ -584,3 +584,17 @@ def linear_rows(x: Tensor, weights, bias: Optional[Tensor] = None, residual: Opt
                                         ptr(residual), int(bool(relu)), py[0], py[1], py[2], stream_handle(dev))
     check(rc, "cf_linear_rows")
     return tuple(ys)
+
+
+def column_sum(g: Tensor) -> Tensor:
+    """Sum over the rows of a (N,C) float32 matrix, fixed order, one launch."""
+    dev = require_device(g)
+    g = _f32(g, "g")
+    if g.dim() != 2:
+        raise _lib.CrystalformerHipError("column_sum: g must be (N,C)")
+    N, C = g.shape
+    out = torch.empty(C, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().cf_column_sum(ptr(g), N, C, ptr(out), stream_handle(dev))
+    check(rc, "cf_column_sum")
+    return out

@@ -283,6 +283,13 @@ int cf_linear_rows(const float *x, int64_t N, int64_t K, const float *w0, const 
                    const float *w2, int n_weights, int64_t C, const float *bias,
                    const float *residual, int relu, float *y0, float *y1, float *y2, void *stream);
 
+/*
+ * Column sums of a row-major (N,C) matrix, out (C): the bias gradient of the linear layers
+ * (what autograd computes for the F.linear calls cited at cf_linear_rows), in a fixed
+ * order, one launch, no scratch.
+ */
+int cf_column_sum(const float *g, int64_t N, int64_t C, float *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -525,3 +525,29 @@ def test_real_enc_fwd_ticket_rounds_are_bit_identical(dev, sizes, H):
                                    p.edges[:, sel], 16, p.dist_max, 1.0, p.W, p.rvlen, -3.5, 1, 0)
     assert_close(z1.cpu()[sel], sub_z, "z sample")
     assert_close(v1.cpu()[sel], sub_v, "v sample")
+
+
+@pytest.mark.parametrize("N,C", [(1774, 128), (1774, 512), (5, 3), (100, 384), (0, 7)])
+def test_column_sum(dev, N, C):
+    g = torch.randn(N, C, generator=torch.Generator().manual_seed(N + C))
+    out = ops.column_sum(g.to(dev))
+    ref = g.double().sum(0).float()
+    if N == 0:
+        assert torch.equal(out.cpu(), torch.zeros(C))
+    else:
+        assert_close(out, ref, "column sums", rtol=2e-6)
+
+
+def test_linear_function_gradients(dev):
+    from crystalformer_amd.hip_funcs import linear
+    g = torch.Generator().manual_seed(12)
+    x, w, b = torch.randn(70, 32, generator=g), torch.randn(48, 32, generator=g), torch.randn(48, generator=g)
+    go = torch.randn(70, 48, generator=g)
+    xr, wr, br = (t.clone().requires_grad_() for t in (x, w, b))
+    torch.nn.functional.linear(xr, wr, br).backward(go)
+    xd, wd, bd = (t.to(dev).requires_grad_() for t in (x, w, b))
+    y = linear(xd, wd, bd)
+    y.backward(go.to(dev))
+    assert_close(y.detach(), torch.nn.functional.linear(x, w, b), "y")
+    for name, got, ref in (("gx", xd.grad, xr.grad), ("gw", wd.grad, wr.grad), ("gb", bd.grad, br.grad)):
+        assert_close(got, ref, name, rtol=5e-6)
