@@ -123,28 +123,28 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(LinArgs p)
 }
 
 // Column sums of a row-major (N, C) matrix (the bias gradient of a linear layer): 16 columns x
-// 16 row groups per work-group, each thread adds every 16th row into 4 running sums, the 16
-// partial sums of a column are then added in order.  No atomics, no zero-filled scratch.
-__global__ __launch_bounds__(256) void column_sum_kernel(const float *g, int64_t N, int C, float *out)
+// 64 row groups per work-group of 1024 threads, each thread adds every 64th row into 4 running
+// sums, the 64 partial sums of a column are then added in order.  No atomics, no scratch.
+__global__ __launch_bounds__(1024) void column_sum_kernel(const float *g, int64_t N, int C, float *out)
 {
-    __shared__ float red[16][17];
+    __shared__ float red[64][17];
     const int cx = threadIdx.x & 15, rg = threadIdx.x >> 4;
     const int col = blockIdx.x * 16 + cx;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (col < C) {
         int64_t n = rg;
-        for (; n + 48 < N; n += 64) {
+        for (; n + 192 < N; n += 256) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) acc[u] += g[(n + 16 * u) * C + col];
+            for (int u = 0; u < 4; u++) acc[u] += g[(n + 64 * u) * C + col];
         }
-        for (; n < N; n += 16) acc[0] += g[n * C + col];
+        for (; n < N; n += 64) acc[0] += g[n * C + col];
     }
     red[rg][cx] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
     __syncthreads();
     if (rg == 0 && col < C) {
         float total = red[0][cx];
-#pragma unroll
-        for (int r = 1; r < 16; r++) total += red[r][cx];
+#pragma unroll 8
+        for (int r = 1; r < 64; r++) total += red[r][cx];
         out[col] = total;
     }
 }
@@ -194,7 +194,7 @@ extern "C" int cf_column_sum(const float *g, int64_t N, int64_t C, float *out, v
 {
     CF_REQUIRE(N >= 0 && C >= 1 && C < (1ll << 30), CF_ERR_INVALID_ARGUMENT, "cf_column_sum: bad sizes");
     CF_REQUIRE(out && (N == 0 || g), CF_ERR_INVALID_ARGUMENT, "cf_column_sum: null pointer");
-    column_sum_kernel<<<(int)((C + 15) / 16), 256, 0, (hipStream_t)stream>>>(g, N, (int)C, out);
+    column_sum_kernel<<<(int)((C + 15) / 16), 1024, 0, (hipStream_t)stream>>>(g, N, (int)C, out);
     CF_CHECK_LAUNCH("cf_column_sum");
     return CF_OK;
 }
