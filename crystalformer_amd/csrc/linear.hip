@@ -149,6 +149,61 @@ __global__ __launch_bounds__(1024) void column_sum_kernel(const float *g, int64_
     }
 }
 
+// Weight gradient of a linear layer, gW (C, K) = g^T x with g (N, C), x (N, K): a short, wide
+// product with a long reduction over the rows.  The rows are cut into slices; a work-group of
+// 4 wavefronts (2 x 2) computes the 32 x 32 block (c0.., k0..) of one slice, operands straight
+// from global memory (lane (q, c) reads g[n + q][c0 + c] and x[n + q][k0 + c], 4 rows per MFMA),
+// and writes it to part[slice]; a second kernel adds the slices in order.
+constexpr int WG_SLICE_STEPS = 8;      // MFMA steps (of 4 rows) whose loads are issued together
+
+__global__ __launch_bounds__(256) void weight_grad_slices_kernel(const float *g, const float *x, int64_t N,
+                                                                 int C, int K, int rows_per_slice, float *part)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int q = lane >> 4, c = lane & 15;
+    const int c0 = blockIdx.x * 32 + 16 * (wave >> 1);
+    const int k0 = blockIdx.y * 32 + 16 * (wave & 1);
+    const int64_t n_begin = (int64_t)blockIdx.z * rows_per_slice;
+    const int64_t n_end = min(N, n_begin + rows_per_slice);
+    const int gc = min(c0 + c, C - 1), xk = min(k0 + c, K - 1);
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t n0 = n_begin; n0 < n_end; n0 += 4 * WG_SLICE_STEPS) {
+        float a[WG_SLICE_STEPS], b[WG_SLICE_STEPS];
+#pragma unroll
+        for (int t = 0; t < WG_SLICE_STEPS; t++) {
+            const int64_t n = n0 + 4 * t + q;
+            const bool in = n < n_end;
+            a[t] = in ? g[n * C + gc] : 0.f;
+            b[t] = in ? x[n * K + xk] : 0.f;
+        }
+#pragma unroll
+        for (int t = 0; t < WG_SLICE_STEPS; t++)
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t], b[t], acc, 0, 0, 0);
+    }
+    // lane (q, c) holds gW[c0 + 4 q + r][k0 + c]
+    float *dst = part + (int64_t)blockIdx.z * C * K;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int cc = c0 + 4 * q + r, kk = k0 + c;
+        if (cc < C && kk < K) dst[(int64_t)cc * K + kk] = acc[r];
+    }
+}
+
+__global__ __launch_bounds__(256) void add_slices_kernel(const float *part, int slices, int64_t total, float *out)
+{
+    const int64_t x = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (x >= total) return;
+    float a0 = 0.f, a1 = 0.f;
+    int s = 0;
+    for (; s + 1 < slices; s += 2) {
+        a0 += part[(int64_t)s * total + x];
+        a1 += part[(int64_t)(s + 1) * total + x];
+    }
+    if (s < slices) a0 += part[(int64_t)s * total + x];
+    out[x] = a0 + a1;
+}
+
 }  // namespace
 
 extern "C" int cf_linear_rows(const float *x, int64_t N, int64_t K, const float *w0, const float *w1,
@@ -196,5 +251,36 @@ extern "C" int cf_column_sum(const float *g, int64_t N, int64_t C, float *out, v
     CF_REQUIRE(out && (N == 0 || g), CF_ERR_INVALID_ARGUMENT, "cf_column_sum: null pointer");
     column_sum_kernel<<<(int)((C + 15) / 16), 1024, 0, (hipStream_t)stream>>>(g, N, (int)C, out);
     CF_CHECK_LAUNCH("cf_column_sum");
+    return CF_OK;
+}
+
+static int weight_grad_slices(int64_t N) { return N >= 512 ? 16 : (N >= 64 ? 4 : 1); }
+
+extern "C" int64_t cf_linear_weight_grad_workspace(int64_t N, int64_t C, int64_t K)
+{
+    if (N < 0 || C < 1 || K < 1) return -1;
+    return (int64_t)weight_grad_slices(N) * C * K * (int64_t)sizeof(float);
+}
+
+extern "C" int cf_linear_weight_grad(const float *g, const float *x, int64_t N, int64_t C, int64_t K,
+                                     void *workspace, int64_t workspace_bytes, float *gW, void *stream)
+{
+    CF_REQUIRE(N >= 0 && C >= 1 && K >= 1 && C < (1 << 20) && K < (1 << 20), CF_ERR_INVALID_ARGUMENT,
+               "cf_linear_weight_grad: bad sizes");
+    CF_REQUIRE(gW && (N == 0 || (g && x)), CF_ERR_INVALID_ARGUMENT, "cf_linear_weight_grad: null pointer");
+    const int slices = weight_grad_slices(N);
+    CF_REQUIRE(workspace && workspace_bytes >= cf_linear_weight_grad_workspace(N, C, K), CF_ERR_INVALID_ARGUMENT,
+               "cf_linear_weight_grad: workspace of %lld bytes needed",
+               (long long)cf_linear_weight_grad_workspace(N, C, K));
+    hipStream_t st = (hipStream_t)stream;
+    const int rows = (int)(((N + slices - 1) / slices + 3) / 4 * 4);
+    dim3 grid((unsigned)((C + 31) / 32), (unsigned)((K + 31) / 32), (unsigned)slices);
+    CF_REQUIRE(grid.y < 65536, CF_ERR_UNSUPPORTED, "cf_linear_weight_grad: too wide");
+    weight_grad_slices_kernel<<<grid, 256, 0, st>>>(g, x, N, (int)C, (int)K, rows < 4 ? 4 : rows,
+                                                    (float *)workspace);
+    CF_CHECK_LAUNCH("cf_linear_weight_grad: slices");
+    const int64_t total = C * K;
+    add_slices_kernel<<<(int)((total + 255) / 256), 256, 0, st>>>((const float *)workspace, slices, total, gW);
+    CF_CHECK_LAUNCH("cf_linear_weight_grad: sum");
     return CF_OK;
 }

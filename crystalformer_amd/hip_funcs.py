@@ -288,7 +288,7 @@ class LinearRowsHIP(torch.autograd.Function):
         x, weight = ctx.saved_tensors
         g = g.contiguous()
         gx = g @ weight if ctx.needs_input_grad[0] else None
-        gw = g.t() @ x if ctx.needs_input_grad[1] else None
+        gw = ops.linear_weight_grad(g, x.contiguous()) if ctx.needs_input_grad[1] else None
         gb = ops.column_sum(g) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
         return gx, gw, gb
 

@@ -598,3 +598,21 @@ def column_sum(g: Tensor) -> Tensor:
         rc = _lib.load().cf_column_sum(ptr(g), N, C, ptr(out), stream_handle(dev))
     check(rc, "cf_column_sum")
     return out
+
+
+def linear_weight_grad(g: Tensor, x: Tensor) -> Tensor:
+    """``g.T @ x`` for g (N,C), x (N,K): the weight gradient of a linear layer, fixed order."""
+    dev = require_device(g, x)
+    g, x = _f32(g, "g"), _f32(x, "x")
+    if g.dim() != 2 or x.dim() != 2 or g.shape[0] != x.shape[0]:
+        raise _lib.CrystalformerHipError("linear_weight_grad: g (N,C) and x (N,K) expected")
+    N, C = g.shape
+    K = x.shape[1]
+    lib = _lib.load()
+    ws_bytes = int(lib.cf_linear_weight_grad_workspace(N, C, K))
+    ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=dev)
+    out = torch.empty((C, K), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.cf_linear_weight_grad(ptr(g), ptr(x), N, C, K, ptr(ws), ws_bytes, ptr(out), stream_handle(dev))
+    check(rc, "cf_linear_weight_grad")
+    return out

@@ -290,6 +290,16 @@ int cf_linear_rows(const float *x, int64_t N, int64_t K, const float *w0, const 
  */
 int cf_column_sum(const float *g, int64_t N, int64_t C, float *out, void *stream);
 
+/*
+ * Weight gradient of a linear layer, gW (C,K) = g^T x for g (N,C), x (N,K) (what autograd
+ * computes for the F.linear calls cited at cf_linear_rows): rows cut into slices summed in a
+ * fixed order, fp32 on the matrix cores.
+ *   workspace: cf_linear_weight_grad_workspace(N,C,K) bytes
+ */
+int64_t cf_linear_weight_grad_workspace(int64_t N, int64_t C, int64_t K);
+int cf_linear_weight_grad(const float *g, const float *x, int64_t N, int64_t C, int64_t K,
+                          void *workspace, int64_t workspace_bytes, float *gW, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

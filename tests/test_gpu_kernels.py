@@ -551,3 +551,12 @@ def test_linear_function_gradients(dev):
     assert_close(y.detach(), torch.nn.functional.linear(x, w, b), "y")
     for name, got, ref in (("gx", xd.grad, xr.grad), ("gw", wd.grad, wr.grad), ("gb", bd.grad, br.grad)):
         assert_close(got, ref, name, rtol=5e-6)
+
+
+@pytest.mark.parametrize("N,C,K", [(1774, 128, 128), (1774, 512, 128), (1774, 128, 512), (70, 48, 32), (3, 5, 7),
+                                   (600, 33, 100)])
+def test_linear_weight_grad(dev, N, C, K):
+    gen = torch.Generator().manual_seed(N + C + K)
+    g, x = torch.randn(N, C, generator=gen), torch.randn(N, K, generator=gen)
+    out = ops.linear_weight_grad(g.to(dev), x.to(dev))
+    assert_close(out, (g.double().T @ x.double()).float(), "gW", rtol=3e-6)
