@@ -281,6 +281,15 @@ def main() -> int:
         "flop_per_eval": flop_per_eval(H, K),
         "fused_dpa_fwd_avg_ms": round(sum(dpa_ms) / max(len(dpa_ms), 1), 4),
     }
+    # the attention kernel is the memory-bound one: algorithmic bytes per edge 4 H (Dv + 2)
+    # (b_ij and a_ij read, prob written) + the q/k/v/out rows once per atom
+    dpa_avg_ms = sum(dpa_ms) / max(len(dpa_ms), 1)
+    if dpa_avg_ms > 0:
+        dpa_bytes = float(E) * H * (D + 2) * 4 + float(N) * H * D * 4 * 4
+        roofline["fused_dpa_fwd"] = {"bound": "hbm", "achieved": round(dpa_bytes / (dpa_avg_ms * 1e-3) / 1e9, 1),
+                                     "peak": 8000.0, "unit": "GB/s",
+                                     "frac": round(dpa_bytes / (dpa_avg_ms * 1e-3) / 1e9 / 8000.0, 4),
+                                     "avg_launch_ms": round(dpa_avg_ms, 4)}
     traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(traffic_file):
         try:
