@@ -15,6 +15,7 @@ from typing import Optional
 
 import torch
 
+from . import ops
 from .synthetic import CrystalBatch
 
 
@@ -43,6 +44,8 @@ class GraphedForward:
         torch.cuda.synchronize()
         with torch.no_grad(), torch.cuda.graph(self.graph):
             self.output = model(self.static)
+        # the graph holds raw addresses of the cached index tensors of this layout
+        self._keepalive = ops.index_cache_snapshot()
         torch.cuda.synchronize()
 
     def __call__(self, batch: Optional[CrystalBatch] = None) -> torch.Tensor:
@@ -100,6 +103,7 @@ class GraphedTrainStep:
             self.graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(self.graph):
                 self.loss = self._step()
+            self._keepalive = ops.index_cache_snapshot()
             torch.cuda.synchronize()
 
     def _step(self) -> torch.Tensor:

@@ -80,6 +80,13 @@ def _cache_lookup(kind: str, *keys: Tensor):
     return sig, None
 
 
+def index_cache_snapshot() -> list:
+    """The current cache entries (key tensors and derived tensors).  A captured graph bakes in
+    the addresses of the derived tensors it found here; whoever owns the graph keeps this list,
+    so that eviction from the cache can never free them."""
+    return list(_index_cache)
+
+
 def _cache_store(sig, keys, value):
     _index_cache.insert(0, (sig, keys, value))
     del _index_cache[_INDEX_CACHE_SIZE:]

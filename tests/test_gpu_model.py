@@ -317,3 +317,27 @@ def test_graphed_training_step_matches_eager(dev):
         moved = float((pp - state0[name]).double().norm())
         diff = float((pg - pp).double().norm())
         assert diff <= 0.05 * moved + 1e-7, (name, moved, diff)
+
+
+def test_graph_survives_index_cache_eviction(dev):
+    """A captured forward bakes in the addresses of the cached index tensors of its layout; it
+    must keep them alive itself when many other layouts push them out of the cache."""
+    from crystalformer_amd import ops
+    from crystalformer_amd.graphs import GraphedForward
+    cfg, model = build_model("cfg1_simplified_b32", num_layers=1, value_pe_dist_real=16)
+    model.to(dev).eval()
+    b = make_config_batch("cfg1_simplified_b32").to(dev)
+    with torch.no_grad():
+        y_eager = model(b).clone()
+    graphed = GraphedForward(model, b)
+    held = [t.data_ptr() for t in (ops.batch_layout(graphed.static.sizes, graphed.static.batch).edges,)]
+    for k in range(40):                                   # far more layouts than the cache holds
+        sizes = torch.tensor([1 + (k % 5), 2 + (k % 3)], device=dev)
+        batch = torch.repeat_interleave(torch.arange(2, device=dev), sizes)
+        ops.batch_layout(sizes, batch)
+    junk = [torch.full((1 << 16,), -7, dtype=torch.int64, device=dev) for _ in range(64)]   # reuse freed blocks
+    assert all(entry[0][0] != "layout" or entry[1][0] is not graphed.static.sizes
+               for entry in ops.index_cache_snapshot())   # really evicted
+    y = graphed().clone()
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_eager) and held and junk
