@@ -132,7 +132,7 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="cfg2_default_b128")
     ap.add_argument("--rule", choices=["A", "B"], default="A",
