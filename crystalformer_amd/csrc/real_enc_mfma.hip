@@ -128,13 +128,28 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd_next2, pos_next2), lane);
         if (PROJ == PROJ_SHARED && hg != wa_hg) {
             const int hw = hg * 8 + wave;
+            if (hw < H && K == 16 * NT && D == 16 * DT) {
+                // full tiles: one base address per lane, 16-byte loads at fixed offsets
+                // (proj_bin(s, q) = 16 (s / 4) + 4 q + s % 4)
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++)
+                for (int dt = 0; dt < DT; dt++) {
+                    const float *wrow = p.W + ((int64_t)hw * D + 16 * dt + c) * K + 4 * q;
 #pragma unroll
-                for (int s = 0; s < 4 * NT; s++) {
-                    const int d = 16 * dt + c, k = proj_bin(s, q);
-                    Wa[dt][s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
+                    for (int t4 = 0; t4 < NT; t4++) {
+                        const float4_t w4 = *reinterpret_cast<const float4_t *>(wrow + 16 * t4);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) Wa[dt][4 * t4 + r] = w4[r];
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int s = 0; s < 4 * NT; s++) {
+                        const int d = 16 * dt + c, k = proj_bin(s, q);
+                        Wa[dt][s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
+                    }
+            }
             wa_hg = hg;
         }
         const int64_t e_ij = ids.e_ij, e_ji = ids.e_ji, i = ids.i, j = ids.j;

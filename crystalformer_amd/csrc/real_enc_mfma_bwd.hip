@@ -125,10 +125,21 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         if (hg != wa_hg) {
             if (wa_hg >= 0) flush_gW(wa_hg);
             const int hw = hg * 8 + wave;
+            if (hw < H && K == 16 * NT && D == 16) {
+                // full tiles: one base address per lane, 16-byte loads at fixed offsets
+                const float *wrow = p.W + ((int64_t)hw * D + c) * K + 4 * q;
 #pragma unroll
-            for (int s = 0; s < 4 * NT; s++) {
-                const int d = c, k = proj_bin(s, q);
-                Wa[s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
+                for (int t4 = 0; t4 < NT; t4++) {
+                    const float4_t w4 = *reinterpret_cast<const float4_t *>(wrow + 16 * t4);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) Wa[4 * t4 + r] = w4[r];
+                }
+            } else {
+#pragma unroll
+                for (int s = 0; s < 4 * NT; s++) {
+                    const int d = c, k = proj_bin(s, q);
+                    Wa[s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
+                }
             }
 #pragma unroll
             for (int t = 0; t < NT; t++) gWacc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
