@@ -53,8 +53,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 #pragma unroll
     for (int m = 0; m < NT; m++) ck[m] = p.bin_step * (float)(16 * m + c + 1);
 
-    // this wave's head: projection operands and the running block of gW
-    float Wa[4 * NT];
+    // this wave's head: the running block of gW (the projection operands are fetched per round,
+    // just before they are used: 16 registers less across the accumulation)
     float4_t gWacc[NT];
     int wa_hg = -1;
 
@@ -124,23 +124,6 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         const int64_t col_edge_next = load_col_edge(rd + stride, pos_next);
         if (hg != wa_hg) {
             if (wa_hg >= 0) flush_gW(wa_hg);
-            const int hw = hg * 8 + wave;
-            if (hw < H && K == 16 * NT && D == 16) {
-                // full tiles: one base address per lane, 16-byte loads at fixed offsets
-                const float *wrow = p.W + ((int64_t)hw * D + c) * K + 4 * q;
-#pragma unroll
-                for (int t4 = 0; t4 < NT; t4++) {
-                    const float4_t w4 = *reinterpret_cast<const float4_t *>(wrow + 16 * t4);
-#pragma unroll
-                    for (int r = 0; r < 4; r++) Wa[4 * t4 + r] = w4[r];
-                }
-            } else {
-#pragma unroll
-                for (int s = 0; s < 4 * NT; s++) {
-                    const int d = c, k = proj_bin(s, q);
-                    Wa[s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
-                }
-            }
 #pragma unroll
             for (int t = 0; t < NT; t++) gWacc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
             wa_hg = hg;
@@ -289,6 +272,25 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         const int jcol = c, unit_j = jcol & 7, dir_j = jcol >> 3;    // product column j = dir*8 + unit
         const float *src = Sbuf + ((wave * 2 + dir_j) * WPB + unit_j) * SROW;
         float dotS = 0.f, dotQ = 0.f;
+        // projection operands of this wave's head (W stays in cache across rounds)
+        float Wa[4 * NT];
+        if (hw < H && K == 16 * NT && D == 16) {
+            // full tiles: one base address per lane, 16-byte loads at fixed offsets
+            // (proj_bin(s, q) = 16 (s / 4) + 4 q + s % 4)
+            const float *wrow = p.W + ((int64_t)hw * D + c) * K + 4 * q;
+#pragma unroll
+            for (int t4 = 0; t4 < NT; t4++) {
+                const float4_t w4 = *reinterpret_cast<const float4_t *>(wrow + 16 * t4);
+#pragma unroll
+                for (int r = 0; r < 4; r++) Wa[4 * t4 + r] = w4[r];
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4 * NT; s++) {
+                const int d = c, k = proj_bin(s, q);
+                Wa[s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
+            }
+        }
         // gradient operands of this wave's head for the 16 product columns, requested before
         // the exchange so that they arrive while the columns are parked
         const int64_t e_out = col_edge;
