@@ -53,9 +53,10 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 #pragma unroll
     for (int m = 0; m < NT; m++) ck[m] = p.bin_step * (float)(16 * m + c + 1);
 
-    // this wave's head: the running block of gW (the projection operands are fetched per round,
-    // just before they are used: 16 registers less across the accumulation)
-    float4_t gWacc[NT];
+    // this wave's head: the running block of gW lives in LDS between rounds (one 16-byte slot per
+    // lane and tile, touched by its own lane only), the projection operands are fetched per round
+    // just before they are used: 32 registers less across the accumulation
+    float4_t *gw_slot = reinterpret_cast<float4_t *>(PXbuf + WPB * 16) + (wave * NT) * WAVE + lane;
     int wa_hg = -1;
 
     const int rounds_per_hg = (int)((p.U + WPB - 1) / WPB);
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int d = 4 * q + r, k = 16 * t + c;
-                    if (d < D && k < K) dst[d * K + k] = gWacc[t][r];
+                    if (d < D && k < K) dst[d * K + k] = gw_slot[t * WAVE][r];
                 }
         }
     };
@@ -125,7 +126,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         if (hg != wa_hg) {
             if (wa_hg >= 0) flush_gW(wa_hg);
 #pragma unroll
-            for (int t = 0; t < NT; t++) gWacc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+            for (int t = 0; t < NT; t++) gw_slot[t * WAVE] = float4_t{0.f, 0.f, 0.f, 0.f};
             wa_hg = hg;
         }
         const int64_t e_ij = ids.e_ij, e_ji = ids.e_ji;
@@ -357,6 +358,9 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             if (pass == 0 && p.gW_part) {
                 // gW_h[d][bin] += sum over the 16 columns of gv[col][d] * S[bin][col]
                 // A[i = d][k = col], B[k = col][j = bin]; column 4*s4 + kk
+                float4_t gWacc[NT];
+#pragma unroll
+                for (int t = 0; t < NT; t++) gWacc[t] = gw_slot[t * WAVE];
 #pragma unroll
                 for (int s4 = 0; s4 < 4; s4++) {
                     const int colk = 4 * s4 + q;                    // this lane's reduction index
@@ -366,6 +370,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                     for (int t = 0; t < NT; t++)
                         gWacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, srck[16 * t + c], gWacc[t], 0, 0, 0);
                 }
+#pragma unroll
+                for (int t = 0; t < NT; t++) gw_slot[t * WAVE] = gWacc[t];
             }
             __syncthreads();
         }
@@ -443,8 +449,8 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
     p.window = sqrtf(40.0f) / bin_step;
     const int NT = K <= 16 ? 1 : K <= 32 ? 2 : 4;
     const bool uniform = cutoff == 0.0f;
-    const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)WPB * 16 * (16 * NT + 1) + WPB * 16) +
-                       sizeof(int64_t) * WPB * 2 + 8;
+    const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)WPB * 16 * (16 * NT + 1) + WPB * 16 +
+                                        (size_t)WPB * NT * WAVE * 4) + 16;
     if (((U + WPB - 1) / WPB) * ((H + 7) / 8) >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // 32-bit round positions
     const int blocks = real_enc_bwd_pairs_blocks(U, H);
 #define CF_BPAIR(NTV)                                                                              \
