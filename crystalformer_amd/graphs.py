@@ -107,6 +107,15 @@ class GraphedTrainStep:
             torch.cuda.synchronize()
 
     def _step(self) -> torch.Tensor:
+        from . import hip_funcs
+        previous = hip_funcs.USE_LINEAR_FUNCTION
+        hip_funcs.USE_LINEAR_FUNCTION = True
+        try:
+            return self._step_body()
+        finally:
+            hip_funcs.USE_LINEAR_FUNCTION = previous
+
+    def _step_body(self) -> torch.Tensor:
         import torch.nn.functional as F
         self.lr_t.copy_(self.lr0 * torch.sqrt(self.decay / (self.decay + self.step_t)))
         out = self.model(self.static)

@@ -293,10 +293,16 @@ class LinearRowsHIP(torch.autograd.Function):
         return gx, gw, gb
 
 
+# Set by the graphed training step (around capture and around its eager twin); plain eager
+# training keeps the stock op, whose autograd runs without Python in the loop.
+USE_LINEAR_FUNCTION = False
+
+
 def linear(x: Tensor, weight: Tensor, bias: Optional[Tensor]) -> Tensor:
-    """F.linear; on the GPU with gradients enabled, through :class:`LinearRowsHIP`."""
-    if x.is_cuda and x.dim() == 2 and x.dtype == torch.float32 and torch.is_grad_enabled() and \
-            (x.requires_grad or weight.requires_grad):
+    """F.linear; inside a graphed training step through :class:`LinearRowsHIP` (fewer and
+    memset-free nodes)."""
+    if USE_LINEAR_FUNCTION and x.is_cuda and x.dim() == 2 and x.dtype == torch.float32 and \
+            torch.is_grad_enabled() and (x.requires_grad or weight.requires_grad):
         return LinearRowsHIP.apply(x, weight, bias)
     return torch.nn.functional.linear(x, weight, bias)
 

@@ -539,7 +539,8 @@ def test_column_sum(dev, N, C):
 
 
 def test_linear_function_gradients(dev):
-    from crystalformer_amd.hip_funcs import linear
+    from crystalformer_amd.hip_funcs import LinearRowsHIP
+    linear = LinearRowsHIP.apply
     g = torch.Generator().manual_seed(12)
     x, w, b = torch.randn(70, 32, generator=g), torch.randn(48, 32, generator=g), torch.randn(48, generator=g)
     go = torch.randn(70, 48, generator=g)
