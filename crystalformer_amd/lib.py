@@ -105,6 +105,25 @@ def ptr(t: Optional[torch.Tensor]) -> int:
     return 0 if t is None else t.data_ptr()
 
 
+class _NoGuard:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device: torch.device):
+    """Context that makes ``device`` current for a launch; free when it already is (the
+    common case: switching the device context costs microseconds per call)."""
+    if torch.cuda.current_device() == device.index:
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
 def stream_handle(device: torch.device) -> int:
     """hipStream_t of torch's current stream on ``device``."""
     return torch.cuda.current_stream(device).cuda_stream

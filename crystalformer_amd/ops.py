@@ -11,7 +11,7 @@ import torch.nn.functional as F
 from torch import Tensor
 
 from . import lib as _lib
-from .lib import check, ptr, require_device, stream_handle
+from .lib import check, device_guard, ptr, require_device, stream_handle
 
 
 # Optional kernel timing: when a list is installed, every encoding / attention
@@ -188,7 +188,7 @@ def real_enc_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
     if _eval_counter is not None:
         _eval_counter.append(count_translation_evals(a_ik, rvlen_n, batch_i, edge_ij_e, cutoff,
                                                      int(lattice_range), int(minimum_range)))
-    with torch.cuda.device(dev), _timed("real_enc_fwd", E=E, H=H, K=K, D=D, proj=W_k is not None):
+    with device_guard(dev), _timed("real_enc_fwd", E=E, H=H, K=K, D=D, proj=W_k is not None):
         rc = _lib.load().cf_real_enc_fwd(
             ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), N, H, E, B, K, D,
             float(dist_max), float(wscale), ptr(W_k if K > 0 else None), W_num,
@@ -234,7 +234,7 @@ def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
     L = _lib.load()
     ws_bytes = int(L.cf_real_enc_bwd_workspace(N, H, E, K, D, W_num, 1 if want_gW else 0))
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev), _timed("real_enc_bwd", E=E, H=H, K=K, D=D, proj=W_k is not None):
+    with device_guard(dev), _timed("real_enc_bwd", E=E, H=H, K=K, D=D, proj=W_k is not None):
         rc = L.cf_real_enc_bwd(
             ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i),
             ptr(z_ek), ptr(gz_ek), ptr(gv_ekd if K > 0 else None), N, H, E, B, K, D, float(dist_max),
@@ -251,7 +251,7 @@ def translation_ranges(a_ik: Tensor, rvlen_n: Optional[Tensor], batch_i: Tensor,
     a_ik, rvlen_n, batch_i = _f32(a_ik, "a_ik"), _f32(rvlen_n, "rvlen_n"), _i64(batch_i, "batch_i")
     N, H = a_ik.shape
     out = torch.empty((N, H, 3), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_translation_ranges(ptr(a_ik), ptr(rvlen_n), ptr(batch_i), N, H,
                                                float(cutoff_radius), int(lattice_range),
                                                int(minimum_range), ptr(out), stream_handle(dev))
@@ -281,7 +281,7 @@ def fused_dpa_fwd(que: Tensor, key: Tensor, val: Tensor, aij_eh: Optional[Tensor
         raise _lib.CrystalformerHipError("fused_dpa_fwd: e_start_i must be (N+1,)")
     prob = torch.empty((E, H), dtype=torch.float32, device=dev)
     out = torch.empty((N, H, Dv), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev), _timed("fused_dpa_fwd", E=E, H=H, Dk=Dk, Dv=Dv, bij=bij_ehd is not None):
+    with device_guard(dev), _timed("fused_dpa_fwd", E=E, H=H, Dk=Dk, Dv=Dv, bij=bij_ehd is not None):
         rc = _lib.load().cf_fused_dpa_fwd(ptr(que), ptr(key), ptr(val), ptr(aij_eh), ptr(bij_ehd),
                                           ptr(edge_ij_e), ptr(e_start_i), N, H, E, Dk, Dv, ptr(prob),
                                           ptr(out), stream_handle(dev))
@@ -307,7 +307,7 @@ def fused_dpa_bwd(que: Tensor, key: Tensor, val: Tensor, bij_ehd: Optional[Tenso
     gq, gk, gv = torch.empty_like(que), torch.empty_like(key), torch.empty_like(val)
     ga = torch.empty((E, H), dtype=torch.float32, device=dev)
     gb = torch.empty((E, H, Dv), dtype=torch.float32, device=dev) if bij_ehd is not None else None
-    with torch.cuda.device(dev), _timed("fused_dpa_bwd", E=E, H=H, Dk=Dk, Dv=Dv, bij=bij_ehd is not None):
+    with device_guard(dev), _timed("fused_dpa_bwd", E=E, H=H, Dk=Dk, Dv=Dv, bij=bij_ehd is not None):
         rc = _lib.load().cf_fused_dpa_bwd(
             ptr(que), ptr(key), ptr(val), ptr(bij_ehd), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i),
             ptr(atom_start_n), ptr(edge_start_n), N, H, E, B, Dk, Dv, ptr(prob_eh), ptr(out), ptr(gout),
@@ -323,7 +323,7 @@ def irregular_mean_fwd(x_ik: Tensor, start_n: Tensor) -> Tensor:
     B = start_n.numel() - 1
     D = x_ik.numel() // N if N > 0 else 0
     out = torch.empty((B,) + tuple(x_ik.shape[1:]), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_irregular_mean_fwd(ptr(x_ik), ptr(start_n), B, D, ptr(out), stream_handle(dev))
     check(rc, "cf_irregular_mean_fwd")
     return out
@@ -335,7 +335,7 @@ def irregular_mean_bwd(go_nk: Tensor, batch_i: Tensor, start_n: Tensor) -> Tenso
     N = batch_i.numel()
     D = go_nk.numel() // go_nk.shape[0] if go_nk.shape[0] > 0 else 0
     gx = torch.empty((N,) + tuple(go_nk.shape[1:]), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_irregular_mean_bwd(ptr(go_nk), ptr(batch_i), ptr(start_n), N, D, ptr(gx),
                                                stream_handle(dev))
     check(rc, "cf_irregular_mean_bwd")
@@ -351,7 +351,7 @@ def minimum_distance(rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_i
     batch_i, edge_ij_e = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e")
     E = edge_ij_e.shape[1]
     out = torch.empty((E,), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_minimum_distance(ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), E,
                                              ptr(rvlen_n), float(cutoff_radius), int(lattice_range),
                                              int(minimum_range), ptr(out), stream_handle(dev))
@@ -380,7 +380,7 @@ def edge_index(sizes: Tensor, pos: Optional[Tensor] = None,
     E = int(num_edges)
     edges = torch.empty((2, E), dtype=torch.int64, device=dev)
     rpos = torch.empty((E, 3), dtype=torch.float32, device=dev) if pos is not None else None
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_edge_index(ptr(atom_start), ptr(edge_start), B, E, ptr(pos), ptr(edges),
                                        ptr(rpos), stream_handle(dev))
     check(rc, "cf_edge_index")
@@ -406,7 +406,7 @@ def edge_pairs(sizes: Tensor, num_atoms: Optional[int] = None, num_edges: Option
         num_atoms, num_edges = int(tail[0]), int(tail[1])
     U = (num_edges + num_atoms) // 2
     pairs = torch.empty((U, PAIR_FIELDS), dtype=torch.int64, device=dev)
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_edge_pairs(ptr(atom_start), ptr(edge_start), ptr(unit_start), B, num_edges,
                                        ptr(pairs), stream_handle(dev))
     check(rc, "cf_edge_pairs")
@@ -489,7 +489,7 @@ def relative_positions(layout: BatchLayout, pos: Tensor) -> Tensor:
     if pos.shape != (layout.num_atoms, 3):
         raise _lib.CrystalformerHipError(f"pos must be ({layout.num_atoms},3), got {tuple(pos.shape)}")
     rpos = torch.empty((layout.num_edges, 3), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_edge_index(ptr(layout.atom_start), ptr(layout.edge_start), layout.sizes.numel(),
                                        layout.num_edges, ptr(pos), None, ptr(rpos), stream_handle(dev))
     check(rc, "cf_edge_index")
@@ -507,7 +507,7 @@ def lattice_geometry(trans_n: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
     vcell = torch.empty(B, dtype=torch.float32, device=dev)
     recip = torch.empty((B, 3, 3), dtype=torch.float32, device=dev)
     rvlen = torch.empty((B, 3), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_lattice_geometry(ptr(trans_n), B, ptr(vcell), ptr(recip), ptr(rvlen),
                                              stream_handle(dev))
     check(rc, "cf_lattice_geometry")
@@ -547,7 +547,7 @@ def gauss_exponents(q_ihd: Tensor, w_hd: Tensor, gauss_scale: Optional[Tensor], 
     alpha_n = torch.empty((N, H), dtype=torch.float32, device=dev) if want_alpha else None
     ws_bytes = int(lib.cf_gauss_exponents_workspace(N, H)) if normalize else 0
     ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=dev) if normalize else None
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = lib.cf_gauss_exponents(ptr(q_ihd), ptr(w_hd), ptr(gauss_scale) if normalize else None, N, H, D,
                                     int(bool(normalize)), int(bool(update_stats)),
                                     POSITIVE_FUNCS[positive_func], float(beta), float(lower_bound), float(coef),
@@ -586,7 +586,7 @@ def linear_rows(x: Tensor, weights, bias: Optional[Tensor] = None, residual: Opt
     ys = [torch.empty((N, C), dtype=torch.float32, device=dev) for _ in weights]
     pw = [ptr(w) for w in weights] + [None] * (3 - len(weights))
     py = [ptr(y) for y in ys] + [None] * (3 - len(weights))
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_linear_rows(ptr(x), N, K, pw[0], pw[1], pw[2], len(weights), C, ptr(bias),
                                         ptr(residual), int(bool(relu)), py[0], py[1], py[2], stream_handle(dev))
     check(rc, "cf_linear_rows")
@@ -601,7 +601,7 @@ def column_sum(g: Tensor) -> Tensor:
         raise _lib.CrystalformerHipError("column_sum: g must be (N,C)")
     N, C = g.shape
     out = torch.empty(C, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = _lib.load().cf_column_sum(ptr(g), N, C, ptr(out), stream_handle(dev))
     check(rc, "cf_column_sum")
     return out
@@ -619,7 +619,7 @@ def linear_weight_grad(g: Tensor, x: Tensor) -> Tensor:
     ws_bytes = int(lib.cf_linear_weight_grad_workspace(N, C, K))
     ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=dev)
     out = torch.empty((C, K), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with device_guard(dev):
         rc = lib.cf_linear_weight_grad(ptr(g), ptr(x), N, C, K, ptr(ws), ws_bytes, ptr(out), stream_handle(dev))
     check(rc, "cf_linear_weight_grad")
     return out
