@@ -77,7 +77,15 @@ def gaussian_exponents(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, ga
 def inference_only(*tensors: Optional[Tensor]) -> bool:
     """True when no gradient can be asked of an op on these tensors: the fused
     row-block linear kernels (no autograd) may then replace F.linear."""
-    return not torch.is_grad_enabled() or not any(t is not None and t.requires_grad for t in tensors)
+    if not torch.is_grad_enabled():
+        return True
+    for t in tensors:
+        if callable(t):                               # lazily listed tensors (e.g. module.parameters)
+            if any(u.requires_grad for u in t()):
+                return False
+        elif t is not None and t.requires_grad:
+            return False
+    return True
 
 
 def fused_exponents_spec(params: LatticeformerParams):

@@ -136,7 +136,7 @@ class CrystalformerEncoderLayerCUDA(Module):
         no_drop = not self.training or all(isinstance(d, Identity) for d in (self.dropout, self.dropout1,
                                                                             self.dropout2))
         return (plain and no_drop and self.activation is F.relu
-                and inference_only(x, *self.parameters())
+                and inference_only(x, self.parameters)
                 and ops.linear_rows_supported(x, self.linear1.weight)
                 and ops.linear_rows_supported(x, self.self_attn.out_proj.weight)
                 and self.linear2.weight.is_cuda and self.linear2.weight.shape[1] % 16 == 0)

@@ -121,7 +121,7 @@ class Latticeformer(nn.Module):
         from .attention import inference_only
         mods = list(self.mlp)
         plain = all(isinstance(m, (nn.Linear, nn.ReLU, nn.Identity)) for m in mods)
-        if not (plain and x.is_cuda and inference_only(x, *self.mlp.parameters())):
+        if not (plain and x.is_cuda and inference_only(x, self.mlp.parameters)):
             return self.mlp(x)
         i = 0
         while i < len(mods):

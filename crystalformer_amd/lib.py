@@ -124,8 +124,13 @@ def device_guard(device: torch.device):
     return torch.cuda.device(device)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_handle(device: torch.device) -> int:
     """hipStream_t of torch's current stream on ``device``."""
+    if _raw_stream is not None:                       # same value, a tenth of the cost
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
 
 

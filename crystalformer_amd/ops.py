@@ -152,7 +152,7 @@ _sched_words: dict = {}
 def _scheduling_words(dev: torch.device) -> Tensor:
     if torch.cuda.is_current_stream_capturing():
         return torch.zeros(2, dtype=torch.int32, device=dev)
-    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    key = (dev.index, stream_handle(dev))
     words = _sched_words.get(key)
     if words is None:
         words = _sched_words[key] = torch.zeros(2, dtype=torch.int32, device=dev)
