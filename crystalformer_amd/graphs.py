@@ -73,7 +73,7 @@ class GraphedTrainStep:
 
     def __init__(self, model: torch.nn.Module, batch: CrystalBatch, lr: float = 5e-4, sch_decay: float = 4000.0,
                  clip_norm: float = 1.0, warmup: int = 3, capture: bool = True):
-        from .training import make_optimizer
+        from .training import FusedAdamW
         if not batch.pos.is_cuda or batch.y is None:
             raise ValueError("GraphedTrainStep needs a batch with targets on the GPU")
         dev = batch.pos.device
@@ -82,12 +82,8 @@ class GraphedTrainStep:
                                    batch.trans_vec.clone(), batch.sizes.clone(), batch.y.clone())
         self.clip_norm = clip_norm
         self.lr0, self.decay = lr, sch_decay
-        self.opt, _ = make_optimizer(model, lr=lr, capturable=True)
-        self.lr_t = torch.tensor(lr, dtype=torch.float32, device=dev)
-        for group in self.opt.param_groups:
-            group["lr"] = self.lr_t                       # one device scalar shared by all groups
-        self.step_t = torch.zeros((), dtype=torch.float32, device=dev)
-        self.params = [p for p in model.parameters() if p.requires_grad]
+        # clip + AdamW + schedule as one device-side update; its step counter lives on the device
+        self.opt = FusedAdamW(model, lr=lr, sch_decay=sch_decay, clip_norm=clip_norm)
         model.train()
         stream = torch.cuda.Stream()                      # default priority
         stream.wait_stream(torch.cuda.current_stream())
@@ -117,14 +113,10 @@ class GraphedTrainStep:
 
     def _step_body(self) -> torch.Tensor:
         import torch.nn.functional as F
-        self.lr_t.copy_(self.lr0 * torch.sqrt(self.decay / (self.decay + self.step_t)))
         out = self.model(self.static)
         loss = F.l1_loss(out[:, 0], self.static.y, reduction="none").mean()
         loss.backward()
-        if self.clip_norm > 0:
-            torch.nn.utils.clip_grad_norm_(self.params, self.clip_norm, foreach=True)
         self.opt.step()
-        self.step_t += 1.0
         return loss.detach()
 
     def __call__(self, batch: Optional[CrystalBatch] = None) -> torch.Tensor:

@@ -623,3 +623,51 @@ def linear_weight_grad(g: Tensor, x: Tensor) -> Tensor:
         rc = lib.cf_linear_weight_grad(ptr(g), ptr(x), N, C, K, ptr(ws), ws_bytes, ptr(out), stream_handle(dev))
     check(rc, "cf_linear_weight_grad")
     return out
+
+
+class AdamWPlan:
+    """Host-side tables for :func:`adamw_step`: the pointer arrays of the parameters and
+    moments (fixed for the life of the optimiser), element counts, decay factors and the
+    chunk-sum workspace."""
+
+    def __init__(self, params, exp_avg, exp_avg_sq, weight_decay):
+        import ctypes
+        dev = require_device(*params)
+        n = len(params)
+        for t in list(params) + list(exp_avg) + list(exp_avg_sq):
+            if t.dtype != torch.float32 or not t.is_contiguous() or t.device != dev:
+                raise _lib.CrystalformerHipError("adamw_step: contiguous float32 tensors on one GPU expected")
+        self.device, self.n = dev, n
+        self.keep = (list(params), list(exp_avg), list(exp_avg_sq))
+        self.p = (ctypes.c_void_p * n)(*[t.data_ptr() for t in params])
+        self.m = (ctypes.c_void_p * n)(*[t.data_ptr() for t in exp_avg])
+        self.v = (ctypes.c_void_p * n)(*[t.data_ptr() for t in exp_avg_sq])
+        self.numel = (ctypes.c_int64 * n)(*[t.numel() for t in params])
+        self.wd = (ctypes.c_float * n)(*[float(w) for w in weight_decay])
+        self.GradArray = ctypes.c_void_p * n
+        self.ws_bytes = int(_lib.load().cf_adamw_step_workspace(n, self.numel))
+        if self.ws_bytes < 0:
+            raise _lib.CrystalformerHipError("adamw_step: bad tensor sizes")
+        self.ws = torch.empty(max(self.ws_bytes // 4, 1), dtype=torch.float32, device=dev)
+
+
+def adamw_step(plan: AdamWPlan, grads, lr0: float, sch_decay: float, beta1: float, beta2: float, eps: float,
+               clip_norm: float, state: Tensor) -> None:
+    """In place: clip the gradients' global norm, AdamW-update the plan's parameters and
+    moments, advance ``state`` (3 floats on the device: updates taken, gradient norm, lr)."""
+    dev = plan.device
+    if len(grads) != plan.n:
+        raise _lib.CrystalformerHipError("adamw_step: one gradient per parameter expected")
+    for g, p in zip(grads, plan.keep[0]):
+        if g is None:
+            raise _lib.CrystalformerHipError("adamw_step: a parameter has no gradient")
+        if g.dtype != torch.float32 or not g.is_contiguous() or g.device != dev or g.numel() != p.numel():
+            raise _lib.CrystalformerHipError("adamw_step: gradients must be contiguous float32 of the parameter's size")
+    if state.dtype != torch.float32 or state.numel() != 3 or state.device != dev:
+        raise _lib.CrystalformerHipError("adamw_step: state is 3 floats on the device")
+    g_arr = plan.GradArray(*[g.data_ptr() for g in grads])
+    with device_guard(dev):
+        rc = _lib.load().cf_adamw_step(plan.n, plan.p, g_arr, plan.m, plan.v, plan.numel, plan.wd, lr0, sch_decay,
+                                       beta1, beta2, eps, clip_norm, ptr(state), ptr(plan.ws), plan.ws_bytes,
+                                       stream_handle(dev))
+    check(rc, "cf_adamw_step")

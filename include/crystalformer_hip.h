@@ -300,6 +300,28 @@ int64_t cf_linear_weight_grad_workspace(int64_t N, int64_t C, int64_t K);
 int cf_linear_weight_grad(const float *g, const float *x, int64_t N, int64_t C, int64_t K,
                           void *workspace, int64_t workspace_bytes, float *gW, void *stream);
 
+/*
+ * One optimiser update of a training step over n_tensors parameter tensors: global
+ * gradient-norm clip (nn.utils.clip_grad_norm_, models/regression.py:122), AdamW
+ * (optim.AdamW, models/regression.py:254; decoupled weight decay per tensor, betas, eps)
+ * and the schedule lr0 * sqrt(sch_decay / (sch_decay + t)) of models/regression.py:269
+ * (sch_decay <= 0: constant lr0), in 2 * ceil(n_tensors / 24) launches.
+ *   params, grads, exp_avg, exp_avg_sq: HOST arrays of n_tensors device pointers (read at
+ *       call time and passed to the kernels by value; the device memory they name is read
+ *       and written when the kernels run)
+ *   numel, weight_decay: HOST arrays of n_tensors element counts / decay factors
+ *   clip_norm <= 0: no clipping
+ *   state_3: DEVICE, [0] updates taken so far, counted in fp32 (exact below 2^24; zero it
+ *       once; every call adds one before using it), [1] gradient norm of this call,
+ *       [2] learning rate of this call
+ *   workspace: cf_adamw_step_workspace(n_tensors, numel) bytes (DEVICE)
+ */
+int64_t cf_adamw_step_workspace(int n_tensors, const int64_t *numel);
+int cf_adamw_step(int n_tensors, float *const *params, const float *const *grads, float *const *exp_avg,
+                  float *const *exp_avg_sq, const int64_t *numel, const float *weight_decay, float lr0,
+                  float sch_decay, float beta1, float beta2, float eps, float clip_norm, float *state_3,
+                  void *workspace, int64_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -561,3 +561,47 @@ def test_linear_weight_grad(dev, N, C, K):
     g, x = torch.randn(N, C, generator=gen), torch.randn(N, K, generator=gen)
     out = ops.linear_weight_grad(g.to(dev), x.to(dev))
     assert_close(out, (g.double().T @ x.double()).float(), "gW", rtol=3e-6)
+
+
+@pytest.mark.parametrize("clip", [1.0, 0.0, 1e4])
+def test_fused_adamw_follows_torch(dev, clip):
+    """clip + AdamW + inverse square-root schedule in one device-side update against
+    torch.nn.utils.clip_grad_norm_ + torch.optim.AdamW + LambdaLR (the reference's training
+    step, models/regression.py:106-135, :254-269) on 30 tensors of ragged sizes (more than
+    one kernel-argument group, chunks with tails, a single-element tensor)."""
+    from crystalformer_amd.training import FusedAdamW, make_optimizer
+    gen = torch.Generator().manual_seed(11)
+    sizes = [1, 7, 128, 2048, 2049, 5000, 128 * 128, 512 * 128] + [100 + 37 * k for k in range(22)]
+
+    class Bag(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            for k, n in enumerate(sizes):                 # odd ones named bias: no weight decay
+                name = f"bias_{k}" if k % 2 else f"weight_{k}"
+                self.register_parameter(name, torch.nn.Parameter(torch.randn(n, generator=gen)))
+
+    ref, mine = Bag().to(dev), Bag().to(dev)
+    mine.load_state_dict(ref.state_dict())
+    opt, sch = make_optimizer(ref, lr=5e-4, weight_decay=1e-2, sch_decay=3.0)
+    fused = FusedAdamW(mine, lr=5e-4, weight_decay=1e-2, sch_decay=3.0, clip_norm=clip)
+    for step in range(6):
+        scale = 10.0 ** (step - 3)                        # clip active on some steps only
+        grads = [torch.randn(n, generator=gen) * scale for n in sizes]
+        for p, q, g in zip(ref.parameters(), mine.parameters(), grads):
+            p.grad, q.grad = g.to(dev), g.to(dev).clone()
+        total = float(torch.linalg.vector_norm(torch.cat(grads).double()))
+        if clip > 0:
+            torch.nn.utils.clip_grad_norm_(ref.parameters(), clip)
+        lr_ref = sch.get_last_lr()[0]
+        opt.step()
+        sch.step()
+        fused.step()
+        st = fused.state.cpu()
+        assert float(st[0]) == step + 1
+        assert abs(float(st[1]) - total) <= 1e-5 * total
+        assert abs(float(st[2]) - lr_ref) <= 1e-6 * lr_ref
+        for (name, p), q in zip(ref.named_parameters(), mine.parameters()):
+            assert_close(q.detach(), p.detach(), f"{name} step {step}", rtol=2e-6)
+    with pytest.raises(Exception):
+        next(iter(mine.parameters())).grad = None
+        fused.step()
