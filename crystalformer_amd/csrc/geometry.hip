@@ -201,7 +201,140 @@ __global__ __launch_bounds__(GE_THREADS) void gauss_exponents_final_kernel(Gauss
     p.a[t] = positive_map(x, p.func, p.beta, p.lb) * p.coef;
 }
 
+// ---- Gaussian exponents, backward --------------------------------------------
+struct GaussBwdArgs {
+    const float *ga, *gqs, *q, *w, *alpha_n, *used_scale;
+    int64_t N, H, D, total;
+    int func;
+    float beta, lb, coef, q_scale;
+    float *part;       // (blocks, H, D) partial weight gradients
+    int blocks;
+    float *gq, *gw;
+};
+
+__device__ __forceinline__ float positive_map_slope(float x, int func, float beta, float lb)
+{
+    if (func == 0) {            // elu
+        const float t = x * (beta / (1.0f - lb));
+        return (t > 0.f ? 1.0f : expf(t)) * beta;
+    }
+    if (func == 1) return (x > 0.f ? 1.0f : (x < 0.f ? -1.0f : 0.f)) * (1.0f - lb);   // abs
+    return expf(x * (beta / (1.0f - lb))) * beta;                                      // exp
+}
+
+// One thread per (atom, head): g_alpha = ga * rho'(alpha_n) * coef * scale;
+// gq = g_alpha w_head + gqs * q_scale; the block leaves sum_atoms g_alpha q per (head, d),
+// 16 columns of d at a time through LDS, atoms added in ascending order.
+__global__ __launch_bounds__(GE_THREADS) void gauss_exponents_bwd_kernel(GaussBwdArgs p)
+{
+    __shared__ float prod[GE_THREADS][17];
+    const int64_t first = (int64_t)blockIdx.x * GE_THREADS;
+    const int64_t t = first + threadIdx.x;
+    const bool live = t < p.total;
+    const int64_t h = live ? t % p.H : 0;
+    float g_alpha = 0.f;
+    if (live && p.ga) {
+        g_alpha = p.ga[t] * positive_map_slope(p.alpha_n[t], p.func, p.beta, p.lb) * p.coef;
+        if (p.used_scale) g_alpha *= p.used_scale[0];
+    }
+    const float *qr = p.q + (live ? t : 0) * p.D;
+    const float *wr = p.w + h * p.D;
+    for (int64_t d0 = 0; d0 < p.D; d0 += 16) {
+        const int nd = (int)min((int64_t)16, p.D - d0);
+        for (int d = 0; d < nd; d++) {
+            const float qv = live ? qr[d0 + d] : 0.f;
+            prod[threadIdx.x][d] = g_alpha * qv;
+            if (live && p.gq) {
+                float g = g_alpha * wr[d0 + d];
+                if (p.gqs) g += p.gqs[t * p.D + d0 + d] * p.q_scale;
+                p.gq[t * p.D + d0 + d] = g;
+            }
+        }
+        __syncthreads();
+        if (p.part) {
+            for (int64_t j = threadIdx.x; j < p.H * 16; j += GE_THREADS) {
+                const int64_t hh = j >> 4;
+                const int d = (int)(j & 15);
+                if (d < nd) {
+                    // first thread of this block whose head is hh
+                    int tid = (int)((hh - first % p.H + p.H) % p.H);
+                    float s = 0.f;
+                    for (; tid < GE_THREADS; tid += (int)p.H) s += prod[tid][d];
+                    p.part[((int64_t)blockIdx.x * p.H + hh) * p.D + d0 + d] = s;
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void gauss_exponents_bwd_reduce_kernel(const float *part, int blocks, int64_t hd,
+                                                                        float *gw)
+{
+    const int64_t x = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (x >= hd) return;
+    float s0 = 0.f, s1 = 0.f;
+    int b = 0;
+    for (; b + 1 < blocks; b += 2) {
+        s0 += part[(int64_t)b * hd + x];
+        s1 += part[(int64_t)(b + 1) * hd + x];
+    }
+    if (b < blocks) s0 += part[(int64_t)b * hd + x];
+    gw[x] = s0 + s1;
+}
+
 }  // namespace
+
+extern "C" int64_t cf_gauss_exponents_bwd_workspace(int64_t N, int64_t H, int64_t D)
+{
+    if (N < 0 || H < 1 || D < 1) return -1;
+    const int64_t blocks = (N * H + GE_THREADS - 1) / GE_THREADS;
+    return (blocks > 0 ? blocks : 1) * H * D * (int64_t)sizeof(float);
+}
+
+extern "C" int cf_gauss_exponents_bwd(const float *ga, const float *gqs, const float *q, const float *w,
+                                      const float *alpha_n, const float *used_scale, int64_t N, int64_t H,
+                                      int64_t D, int positive_func, float beta, float lower_bound, float coef,
+                                      float q_scale, void *workspace, int64_t workspace_bytes, float *gq,
+                                      float *gw, void *stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    CF_REQUIRE(N >= 0 && H >= 1 && D >= 1 && H <= 4096, CF_ERR_INVALID_ARGUMENT,
+               "cf_gauss_exponents_bwd: bad sizes N=%lld H=%lld D=%lld", (long long)N, (long long)H, (long long)D);
+    CF_REQUIRE(positive_func >= 0 && positive_func <= 2, CF_ERR_UNSUPPORTED,
+               "cf_gauss_exponents_bwd: positive map %d not served (0 elu, 1 abs, 2 exp)", positive_func);
+    CF_REQUIRE(lower_bound < 1.0f, CF_ERR_INVALID_ARGUMENT, "cf_gauss_exponents_bwd: lower bound must be < 1");
+    CF_REQUIRE(gq || gw, CF_ERR_INVALID_ARGUMENT, "cf_gauss_exponents_bwd: no output requested");
+    if (N == 0) {
+        if (gw) {                                  // no atoms: zero gradient (the sum over zero blocks)
+            gauss_exponents_bwd_reduce_kernel<<<(int)((H * D + 255) / 256), 256, 0, stream>>>(nullptr, 0, H * D, gw);
+            CF_CHECK_LAUNCH("cf_gauss_exponents_bwd: zero");
+        }
+        return CF_OK;
+    }
+    CF_REQUIRE(q && w && (!ga || alpha_n), CF_ERR_INVALID_ARGUMENT, "cf_gauss_exponents_bwd: NULL operand");
+    const int64_t blocks = (N * H + GE_THREADS - 1) / GE_THREADS;
+    CF_REQUIRE(blocks < (1ll << 31), CF_ERR_INVALID_ARGUMENT, "cf_gauss_exponents_bwd: too many atoms");
+    if (gw)
+        CF_REQUIRE(workspace && workspace_bytes >= cf_gauss_exponents_bwd_workspace(N, H, D), CF_ERR_INVALID_ARGUMENT,
+                   "cf_gauss_exponents_bwd: workspace of %lld bytes needed",
+                   (long long)cf_gauss_exponents_bwd_workspace(N, H, D));
+    GaussBwdArgs p;
+    p.ga = ga; p.gqs = gqs; p.q = q; p.w = w; p.alpha_n = alpha_n; p.used_scale = used_scale;
+    p.N = N; p.H = H; p.D = D; p.total = N * H;
+    p.func = positive_func; p.beta = beta; p.lb = lower_bound; p.coef = coef; p.q_scale = q_scale;
+    p.part = gw ? (float *)workspace : nullptr;
+    p.blocks = (int)blocks;
+    p.gq = gq; p.gw = gw;
+    gauss_exponents_bwd_kernel<<<(int)blocks, GE_THREADS, 0, stream>>>(p);
+    CF_CHECK_LAUNCH("cf_gauss_exponents_bwd");
+    if (gw) {
+        const int64_t hd = H * D;
+        gauss_exponents_bwd_reduce_kernel<<<(int)((hd + 255) / 256), 256, 0, stream>>>(p.part, (int)blocks, hd, gw);
+        CF_CHECK_LAUNCH("cf_gauss_exponents_bwd: reduce");
+    }
+    return CF_OK;
+}
 
 extern "C" int cf_lattice_geometry(const float *trans, int64_t B, float *vcell, float *recip, float *rvlen,
                                    void *stream_)

@@ -244,31 +244,18 @@ class GaussianExponentsHIP(torch.autograd.Function):
         if need_grad:
             ctx.save_for_backward(q_ihd, w_hd, alpha_n, used)
         ctx.conf = (positive_func, beta, lower_bound, coef, q_scale)
+        ctx.w_shape = w_hd.shape
         return a, qs
 
     @staticmethod
     def backward(ctx, ga, gqs):
         q_ihd, w_hd, alpha_n, used = ctx.saved_tensors
         func, beta, lb, coef, q_scale = ctx.conf
-        n, h, d = q_ihd.shape
-        if func == "elu":
-            x = alpha_n * (beta / (1.0 - lb))
-            slope = torch.where(x > 0, torch.ones_like(x), torch.exp(x)) * beta
-        elif func == "abs":
-            slope = torch.sign(alpha_n) * (1.0 - lb)
-        else:
-            slope = torch.exp(alpha_n * (beta / (1.0 - lb))) * beta
-        g_alpha = ga * slope * coef
-        if used is not None:
-            g_alpha = g_alpha * used[0]
-        w = w_hd.reshape(1, h, d)
-        gq = gw = None
-        if ctx.needs_input_grad[0]:
-            gq = g_alpha[..., None] * w
-            if gqs is not None:
-                gq = gq + gqs * q_scale
-        if ctx.needs_input_grad[1]:
-            gw = (g_alpha[..., None] * q_ihd).sum(0).reshape(w_hd.shape)
+        gq, gw = ops.gauss_exponents_bwd(ga, gqs, q_ihd, w_hd, alpha_n, used, func, beta, lb, coef,
+                                         q_scale if q_scale is not None else 1.0,
+                                         want_gq=ctx.needs_input_grad[0], want_gw=ctx.needs_input_grad[1])
+        if gw is not None:
+            gw = gw.reshape(ctx.w_shape)
         return gq, gw, None, None, None, None, None, None, None, None
 
 

@@ -557,6 +557,38 @@ def gauss_exponents(q_ihd: Tensor, w_hd: Tensor, gauss_scale: Optional[Tensor], 
     return a, qs, alpha_n, (ws[-4:-2] if normalize else None)
 
 
+def gauss_exponents_bwd(ga: Optional[Tensor], gqs: Optional[Tensor], q_ihd: Tensor, w_hd: Tensor,
+                        alpha_n: Tensor, used: Optional[Tensor], positive_func: str, beta: float,
+                        lower_bound: float, coef: float, q_scale: float, want_gq: bool = True,
+                        want_gw: bool = True) -> Tuple[Optional[Tensor], Optional[Tensor]]:
+    """Gradients of :func:`gauss_exponents` with respect to the query and the head weights
+    (statistics held constant), one launch plus a fixed-order reduction."""
+    dev = require_device(ga, gqs, q_ihd, w_hd, alpha_n, used)
+    ga, gqs, q_ihd, w_hd, alpha_n = (_f32(t, n) for t, n in ((ga, "ga"), (gqs, "gqs"), (q_ihd, "q_ihd"),
+                                                              (w_hd, "w_hd"), (alpha_n, "alpha_n")))
+    N, H, D = q_ihd.shape
+    if w_hd.numel() != H * D or alpha_n.numel() != N * H or (ga is not None and ga.numel() != N * H) \
+            or (gqs is not None and gqs.shape != q_ihd.shape):
+        raise _lib.CrystalformerHipError("gauss_exponents_bwd: operand shapes disagree")
+    if positive_func not in POSITIVE_FUNCS:
+        raise _lib.CrystalformerHipError(f"positive map {positive_func!r} has no kernel")
+    if used is not None:
+        used = _f32(used, "used")
+    lib = _lib.load()
+    gq = torch.empty_like(q_ihd) if want_gq else None
+    gw = torch.empty((H, D), dtype=torch.float32, device=dev) if want_gw else None
+    if gq is None and gw is None:
+        return None, None
+    ws_bytes = int(lib.cf_gauss_exponents_bwd_workspace(N, H, D)) if want_gw else 0
+    ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=dev) if want_gw else None
+    with device_guard(dev):
+        rc = lib.cf_gauss_exponents_bwd(ptr(ga), ptr(gqs), ptr(q_ihd), ptr(w_hd), ptr(alpha_n), ptr(used), N, H, D,
+                                        POSITIVE_FUNCS[positive_func], float(beta), float(lower_bound), float(coef),
+                                        float(q_scale), ptr(ws), ws_bytes, ptr(gq), ptr(gw), stream_handle(dev))
+    check(rc, "cf_gauss_exponents_bwd")
+    return gq, gw
+
+
 def linear_rows_supported(x: Tensor, *weights: Tensor) -> bool:
     """True when :func:`linear_rows` serves these operands (float32 on the GPU, input
     width a multiple of 16, equal weight shapes)."""

@@ -267,6 +267,22 @@ int cf_gauss_exponents(const float *q_ihd, const float *w_hd, float *gauss_scale
                        void *stream);
 
 /*
+ * Backward of cf_gauss_exponents with the normalisation statistics held constant (the
+ * reference detaches them, models/indexed_lattice_multi_head_attention_cuda.py:700-712; what
+ * autograd computes for :636-722): g_alpha = ga * rho'(alpha_n) * coef * scale,
+ * gq = g_alpha w_head + gqs * q_scale, gw[h] = sum_i g_alpha[i,h] q[i,h] in a fixed order.
+ *   ga (N,H) or NULL (no gradient through a), gqs (N,H,D) or NULL, alpha_n (N,H) as left by the
+ *   forward, used_scale: DEVICE pointer to the scale the forward applied, NULL when it did
+ *   not normalise; gq (N,H,D) and gw (H,D): either may be NULL
+ *   workspace: cf_gauss_exponents_bwd_workspace(N,H,D) bytes, needed when gw is asked for
+ */
+int64_t cf_gauss_exponents_bwd_workspace(int64_t N, int64_t H, int64_t D);
+int cf_gauss_exponents_bwd(const float *ga, const float *gqs, const float *q, const float *w,
+                           const float *alpha_n, const float *used_scale, int64_t N, int64_t H, int64_t D,
+                           int positive_func, float beta, float lower_bound, float coef, float q_scale,
+                           void *workspace, int64_t workspace_bytes, float *gq, float *gw, void *stream);
+
+/*
  * Row-block linear layer(s): y_w = act(x W_w^T + b_w) (+ residual), w < n_weights <= 3,
  * for the small dense layers around the attention: the query/key/value
  * projections in one launch (models/indexed_lattice_multi_head_attention_cuda.py:865-867,

@@ -605,3 +605,40 @@ def test_fused_adamw_follows_torch(dev, clip):
     with pytest.raises(Exception):
         next(iter(mine.parameters())).grad = None
         fused.step()
+
+
+@pytest.mark.parametrize("func", ["elu", "abs", "exp"])
+@pytest.mark.parametrize("N,H,D,scaled", [(1774, 8, 16, True), (301, 3, 20, False), (5, 1, 4, True),
+                                          (700, 16, 8, True)])
+def test_gauss_exponents_bwd_kernel(dev, func, N, H, D, scaled):
+    """Backward kernel against float64 autograd of a = coef * rho((alpha + shift) * scale),
+    q_scaled = q * q_scale, with (scale, shift) constants; several blocks, ragged tails,
+    head counts that do not divide the block and widths beyond one 16-column pass."""
+    gen = torch.Generator().manual_seed(N + H + D)
+    q = torch.randn(N, H, D, generator=gen)
+    w = torch.randn(H, D, generator=gen) * 0.3
+    ga = torch.randn(N, H, generator=gen)
+    gqs = torch.randn(N, H, D, generator=gen) if scaled else None
+    beta, lb, coef, q_scale = 0.1, 0.5, -0.37, 0.25
+    used = torch.tensor([1.7, -0.2]) if scaled else None            # (scale, shift) of a normalising forward
+    qd, wd = q.double().requires_grad_(), w.double().requires_grad_()
+    alpha = (qd * wd[None]).sum(-1)
+    alpha_n = (alpha + used[1].double()) * used[0].double() if used is not None else alpha
+    if func == "elu":
+        rho = (1 - lb) * torch.nn.functional.elu(alpha_n * (beta / (1 - lb))) + 1.0
+    elif func == "abs":
+        rho = (1 - lb) * alpha_n.abs() + lb
+    else:
+        rho = (1 - lb) * torch.exp(alpha_n * (beta / (1 - lb))) + lb
+    obj = (rho * coef * ga.double()).sum()
+    if scaled:
+        obj = obj + (qd * q_scale * gqs.double()).sum()
+    obj.backward()
+    gq, gw = ops.gauss_exponents_bwd(ga.to(dev), gqs.to(dev) if scaled else None, q.to(dev), w.to(dev),
+                                     alpha_n.detach().float().to(dev), used.to(dev) if scaled else None,
+                                     func, beta, lb, coef, q_scale)
+    assert_close(gq, qd.grad.float(), "gq")
+    assert_close(gw, wd.grad.float(), "gw", rtol=3e-6)
+    only_w = ops.gauss_exponents_bwd(ga.to(dev), None, q.to(dev), w.to(dev), alpha_n.detach().float().to(dev),
+                                     used.to(dev) if scaled else None, func, beta, lb, coef, q_scale, want_gq=False)
+    assert only_w[0] is None and torch.equal(only_w[1], gw)
