@@ -157,7 +157,8 @@ __global__ __launch_bounds__(1024) void column_sum_kernel(const float *g, int64_
 constexpr int WG_SLICE_STEPS = 8;      // MFMA steps (of 4 rows) whose loads are issued together
 
 __global__ __launch_bounds__(256) void weight_grad_slices_kernel(const float *g, const float *x, int64_t N,
-                                                                 int C, int K, int rows_per_slice, float *part)
+                                                                 int C, int K, int rows_per_slice, float *part,
+                                                                 float *part_b)
 {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -168,6 +169,7 @@ __global__ __launch_bounds__(256) void weight_grad_slices_kernel(const float *g,
     const int64_t n_end = min(N, n_begin + rows_per_slice);
     const int gc = min(c0 + c, C - 1), xk = min(k0 + c, K - 1);
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    float colsum = 0.f;                     // bias gradient: this lane's rows of column c0 + c
     for (int64_t n0 = n_begin; n0 < n_end; n0 += 4 * WG_SLICE_STEPS) {
         float a[WG_SLICE_STEPS], b[WG_SLICE_STEPS];
 #pragma unroll
@@ -178,8 +180,15 @@ __global__ __launch_bounds__(256) void weight_grad_slices_kernel(const float *g,
             b[t] = in ? x[n * K + xk] : 0.f;
         }
 #pragma unroll
-        for (int t = 0; t < WG_SLICE_STEPS; t++)
+        for (int t = 0; t < WG_SLICE_STEPS; t++) {
             acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t], b[t], acc, 0, 0, 0);
+            colsum += a[t];
+        }
+    }
+    if (part_b && blockIdx.y == 0 && (wave & 1) == 0) {
+        // rows n = 4 t + q: add the four row classes in ascending q
+        const float s = (colsum + __shfl_xor(colsum, 16, 64)) + (__shfl_xor(colsum, 32, 64) + __shfl_xor(colsum, 48, 64));
+        if (q == 0 && c0 + c < C) part_b[(int64_t)blockIdx.z * C + c0 + c] = s;
     }
     // lane (q, c) holds gW[c0 + 4 q + r][k0 + c]
     float *dst = part + (int64_t)blockIdx.z * C * K;
@@ -190,10 +199,17 @@ __global__ __launch_bounds__(256) void weight_grad_slices_kernel(const float *g,
     }
 }
 
-__global__ __launch_bounds__(256) void add_slices_kernel(const float *part, int slices, int64_t total, float *out)
+// out[x] = sum over slices of part[s][x]; with out_b, elements past `total` belong to a second
+// array of `total_b` elements per slice (the bias gradient) summed the same way.
+__global__ __launch_bounds__(256) void add_slices_kernel(const float *part, int slices, int64_t total, float *out,
+                                                         const float *part_b, int64_t total_b, float *out_b)
 {
-    const int64_t x = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (x >= total) return;
+    int64_t x = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (x >= total) {
+        x -= total;
+        if (!out_b || x >= total_b) return;
+        part = part_b; total = total_b; out = out_b;
+    }
     float a0 = 0.f, a1 = 0.f;
     int s = 0;
     for (; s + 1 < slices; s += 2) {
@@ -259,11 +275,11 @@ static int weight_grad_slices(int64_t N) { return N >= 512 ? 16 : (N >= 64 ? 4 :
 extern "C" int64_t cf_linear_weight_grad_workspace(int64_t N, int64_t C, int64_t K)
 {
     if (N < 0 || C < 1 || K < 1) return -1;
-    return (int64_t)weight_grad_slices(N) * C * K * (int64_t)sizeof(float);
+    return (int64_t)weight_grad_slices(N) * C * (K + 1) * (int64_t)sizeof(float);
 }
 
 extern "C" int cf_linear_weight_grad(const float *g, const float *x, int64_t N, int64_t C, int64_t K,
-                                     void *workspace, int64_t workspace_bytes, float *gW, void *stream)
+                                     void *workspace, int64_t workspace_bytes, float *gW, float *gb, void *stream)
 {
     CF_REQUIRE(N >= 0 && C >= 1 && K >= 1 && C < (1 << 20) && K < (1 << 20), CF_ERR_INVALID_ARGUMENT,
                "cf_linear_weight_grad: bad sizes");
@@ -276,11 +292,14 @@ extern "C" int cf_linear_weight_grad(const float *g, const float *x, int64_t N, 
     const int rows = (int)(((N + slices - 1) / slices + 3) / 4 * 4);
     dim3 grid((unsigned)((C + 31) / 32), (unsigned)((K + 31) / 32), (unsigned)slices);
     CF_REQUIRE(grid.y < 65536, CF_ERR_UNSUPPORTED, "cf_linear_weight_grad: too wide");
-    weight_grad_slices_kernel<<<grid, 256, 0, st>>>(g, x, N, (int)C, (int)K, rows < 4 ? 4 : rows,
-                                                    (float *)workspace);
-    CF_CHECK_LAUNCH("cf_linear_weight_grad: slices");
     const int64_t total = C * K;
-    add_slices_kernel<<<(int)((total + 255) / 256), 256, 0, st>>>((const float *)workspace, slices, total, gW);
+    float *part_b = gb ? (float *)workspace + (int64_t)slices * total : nullptr;
+    weight_grad_slices_kernel<<<grid, 256, 0, st>>>(g, x, N, (int)C, (int)K, rows < 4 ? 4 : rows,
+                                                    (float *)workspace, part_b);
+    CF_CHECK_LAUNCH("cf_linear_weight_grad: slices");
+    const int64_t cells = total + (gb ? C : 0);
+    add_slices_kernel<<<(int)((cells + 255) / 256), 256, 0, st>>>((const float *)workspace, slices, total, gW,
+                                                                  part_b, C, gb);
     CF_CHECK_LAUNCH("cf_linear_weight_grad: sum");
     return CF_OK;
 }

@@ -260,9 +260,10 @@ class GaussianExponentsHIP(torch.autograd.Function):
 
 
 class LinearRowsHIP(torch.autograd.Function):
-    """y = x W^T + b for 2-D x on the training path: library GEMMs for the products, the
-    bias gradient as one fixed-order column-sum launch (autograd's own reduction records a
-    memset node per call under stream capture and takes three times as long)."""
+    """y = x W^T + b for 2-D x on the training path: library GEMMs for the forward and the
+    input gradient; weight and bias gradient from one fixed-order pass over the output
+    gradient (autograd's own bias reduction records a memset node per call under stream
+    capture and takes three times as long)."""
 
     @staticmethod
     def forward(ctx, x, weight, bias):
@@ -275,8 +276,14 @@ class LinearRowsHIP(torch.autograd.Function):
         x, weight = ctx.saved_tensors
         g = g.contiguous()
         gx = g @ weight if ctx.needs_input_grad[0] else None
-        gw = ops.linear_weight_grad(g, x.contiguous()) if ctx.needs_input_grad[1] else None
-        gb = ops.column_sum(g) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
+        want_b = ctx.has_bias and ctx.needs_input_grad[2]
+        gw = gb = None
+        if ctx.needs_input_grad[1]:
+            gw = ops.linear_weight_grad(g, x.contiguous(), with_bias=want_b)
+            if want_b:
+                gw, gb = gw
+        elif want_b:
+            gb = ops.column_sum(g)
         return gx, gw, gb
 
 

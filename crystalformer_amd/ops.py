@@ -639,8 +639,9 @@ def column_sum(g: Tensor) -> Tensor:
     return out
 
 
-def linear_weight_grad(g: Tensor, x: Tensor) -> Tensor:
-    """``g.T @ x`` for g (N,C), x (N,K): the weight gradient of a linear layer, fixed order."""
+def linear_weight_grad(g: Tensor, x: Tensor, with_bias: bool = False):
+    """``g.T @ x`` for g (N,C), x (N,K): the weight gradient of a linear layer, fixed order.
+    ``with_bias``: returns ``(gW, gb)``, gb the column sums of g from the same pass."""
     dev = require_device(g, x)
     g, x = _f32(g, "g"), _f32(x, "x")
     if g.dim() != 2 or x.dim() != 2 or g.shape[0] != x.shape[0]:
@@ -651,10 +652,12 @@ def linear_weight_grad(g: Tensor, x: Tensor) -> Tensor:
     ws_bytes = int(lib.cf_linear_weight_grad_workspace(N, C, K))
     ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=dev)
     out = torch.empty((C, K), dtype=torch.float32, device=dev)
+    gb = torch.empty((C,), dtype=torch.float32, device=dev) if with_bias else None
     with device_guard(dev):
-        rc = lib.cf_linear_weight_grad(ptr(g), ptr(x), N, C, K, ptr(ws), ws_bytes, ptr(out), stream_handle(dev))
+        rc = lib.cf_linear_weight_grad(ptr(g), ptr(x), N, C, K, ptr(ws), ws_bytes, ptr(out), ptr(gb),
+                                       stream_handle(dev))
     check(rc, "cf_linear_weight_grad")
-    return out
+    return (out, gb) if with_bias else out
 
 
 class AdamWPlan:

@@ -309,12 +309,13 @@ int cf_column_sum(const float *g, int64_t N, int64_t C, float *out, void *stream
 /*
  * Weight gradient of a linear layer, gW (C,K) = g^T x for g (N,C), x (N,K) (what autograd
  * computes for the F.linear calls cited at cf_linear_rows): rows cut into slices summed in a
- * fixed order, fp32 on the matrix cores.
+ * fixed order, fp32 on the matrix cores.  gb (C) or NULL: the bias gradient (column sums of
+ * g) from the same pass over g.
  *   workspace: cf_linear_weight_grad_workspace(N,C,K) bytes
  */
 int64_t cf_linear_weight_grad_workspace(int64_t N, int64_t C, int64_t K);
 int cf_linear_weight_grad(const float *g, const float *x, int64_t N, int64_t C, int64_t K,
-                          void *workspace, int64_t workspace_bytes, float *gW, void *stream);
+                          void *workspace, int64_t workspace_bytes, float *gW, float *gb, void *stream);
 
 /*
  * One optimiser update of a training step over n_tensors parameter tensors: global

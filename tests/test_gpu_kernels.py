@@ -561,6 +561,9 @@ def test_linear_weight_grad(dev, N, C, K):
     g, x = torch.randn(N, C, generator=gen), torch.randn(N, K, generator=gen)
     out = ops.linear_weight_grad(g.to(dev), x.to(dev))
     assert_close(out, (g.double().T @ x.double()).float(), "gW", rtol=3e-6)
+    both, gb = ops.linear_weight_grad(g.to(dev), x.to(dev), with_bias=True)   # bias gradient from the same pass
+    assert torch.equal(both, out)
+    assert_close(gb, g.double().sum(0).float(), "gb", rtol=3e-6)
 
 
 @pytest.mark.parametrize("clip", [1.0, 0.0, 1e4])
