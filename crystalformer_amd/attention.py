@@ -21,6 +21,7 @@ from torch.nn.init import constant_, normal_, xavier_uniform_
 
 from . import global_config as config
 from . import ops
+from . import hip_funcs
 from .hip_funcs import linear as linear_hip
 from .hip_funcs import (FusedDotProductAttentionCUDA, GaussianExponentsHIP, RealPeriodicEncodingFuncCUDA,
                         RealPeriodicEncodingWithProjFuncCUDA)
@@ -229,10 +230,19 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                         and ops.linear_rows_supported(query, self.q_proj_weight, self.k_proj_weight,
                                                       self.v_proj_weight)
                         and vd % 16 == 0)
+        # the same launches with autograd, inside a graphed training step
+        fused_train = (not fused_linear and hip_funcs.USE_LINEAR_FUNCTION and torch.is_grad_enabled()
+                       and query is key and key is value and kd == vd and vd % 16 == 0
+                       and ops.linear_rows_supported(query, self.q_proj_weight, self.k_proj_weight,
+                                                     self.v_proj_weight))
         if fused_linear:
             # the three projections in one launch
             q, k, v = ops.linear_rows(query, (self.q_proj_weight, self.k_proj_weight, self.v_proj_weight),
                                       self.in_proj_bias)
+            q, k, v = q.view(n, H, kd // H), k.view(n, H, kd // H), v.view(n, H, vd // H)
+        elif fused_train:
+            q, k, v = hip_funcs.FusedLinearHIP.apply(query, self.in_proj_bias, None, False, self.q_proj_weight,
+                                                     self.k_proj_weight, self.v_proj_weight)
             q, k, v = q.view(n, H, kd // H), k.view(n, H, kd // H), v.view(n, H, vd // H)
         else:
             q = linear_hip(query, self.q_proj_weight, b_q).contiguous().view(n, H, kd // H)
@@ -283,6 +293,8 @@ class CrystalformerMultiheadAttentionCUDA(Module):
         attn = attn.contiguous().view(n, vd)
         if fused_linear:
             attn, = ops.linear_rows(attn, (self.out_proj.weight,), self.out_proj.bias, residual=residual)
+        elif fused_train and ops.linear_rows_supported(attn, self.out_proj.weight):
+            attn, = hip_funcs.FusedLinearHIP.apply(attn, self.out_proj.bias, residual, False, self.out_proj.weight)
         else:
             attn = linear_hip(attn, self.out_proj.weight, self.out_proj.bias)
             if residual is not None:

@@ -220,6 +220,104 @@ __global__ __launch_bounds__(256) void add_slices_kernel(const float *part, int 
     out[x] = a0 + a1;
 }
 
+// ---- grouped weight gradients -------------------------------------------------
+// The weight (and bias) gradients of several linear layers in two launches: the layers'
+// 32 x 32 output tiles are numbered consecutively and a work-group finds its layer by
+// scanning the group's tile prefix.  Per layer the arithmetic, slicing and summation order
+// are those of weight_grad_slices_kernel / add_slices_kernel, so results are identical.
+constexpr int WG_GROUP = 16;
+
+struct WeightGradGroup {
+    const float *g[WG_GROUP], *x[WG_GROUP];
+    float *gw[WG_GROUP], *gb[WG_GROUP];
+    int64_t part_off[WG_GROUP];      // floats from the workspace start to this layer's slices
+    int N[WG_GROUP], C[WG_GROUP], K[WG_GROUP], slices[WG_GROUP];
+    int tile0[WG_GROUP + 1];         // prefix over 32 x 32 tiles
+    int cell0[WG_GROUP + 1];         // prefix over 256-element blocks of C (K + 1) outputs
+    int count;
+    float *part;
+};
+
+__global__ __launch_bounds__(256) void weight_grad_group_slices_kernel(WeightGradGroup a)
+{
+    int t = 0;
+    while (t + 1 < a.count && a.tile0[t + 1] <= (int)blockIdx.x) t++;
+    if ((int)blockIdx.y >= a.slices[t]) return;
+    const int tile = blockIdx.x - a.tile0[t];
+    const int C = a.C[t], K = a.K[t];
+    const int64_t N = a.N[t];
+    const int tiles_k = (K + 31) / 32;
+    const int tc = tile / tiles_k, tk = tile - tc * tiles_k;
+    const int slices = a.slices[t];
+    int rows = (int)(((N + slices - 1) / slices + 3) / 4 * 4);
+    if (rows < 4) rows = 4;
+    const float *g = a.g[t], *x = a.x[t];
+    float *part = a.part + a.part_off[t];
+    float *part_b = a.gb[t] ? part + (int64_t)slices * C * K : nullptr;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int q = lane >> 4, c = lane & 15;
+    const int c0 = tc * 32 + 16 * (wave >> 1);
+    const int k0 = tk * 32 + 16 * (wave & 1);
+    const int64_t n_begin = (int64_t)blockIdx.y * rows;
+    const int64_t n_end = min(N, n_begin + rows);
+    const int gc = min(c0 + c, C - 1), xk = min(k0 + c, K - 1);
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    float colsum = 0.f;
+    for (int64_t n0 = n_begin; n0 < n_end; n0 += 4 * WG_SLICE_STEPS) {
+        float av[WG_SLICE_STEPS], bv[WG_SLICE_STEPS];
+#pragma unroll
+        for (int u = 0; u < WG_SLICE_STEPS; u++) {
+            const int64_t n = n0 + 4 * u + q;
+            const bool in = n < n_end;
+            av[u] = in ? g[n * C + gc] : 0.f;
+            bv[u] = in ? x[n * K + xk] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < WG_SLICE_STEPS; u++) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u], acc, 0, 0, 0);
+            colsum += av[u];
+        }
+    }
+    if (part_b && tk == 0 && (wave & 1) == 0) {
+        const float s = (colsum + __shfl_xor(colsum, 16, 64)) + (__shfl_xor(colsum, 32, 64) + __shfl_xor(colsum, 48, 64));
+        if (q == 0 && c0 + c < C) part_b[(int64_t)blockIdx.y * C + c0 + c] = s;
+    }
+    float *dst = part + (int64_t)blockIdx.y * C * K;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int cc = c0 + 4 * q + r, kk = k0 + c;
+        if (cc < C && kk < K) dst[(int64_t)cc * K + kk] = acc[r];
+    }
+}
+
+__global__ __launch_bounds__(256) void weight_grad_group_add_kernel(WeightGradGroup a)
+{
+    int t = 0;
+    while (t + 1 < a.count && a.cell0[t + 1] <= (int)blockIdx.x) t++;
+    int64_t x = (int64_t)(blockIdx.x - a.cell0[t]) * 256 + threadIdx.x;
+    const int slices = a.slices[t];
+    int64_t total = (int64_t)a.C[t] * a.K[t];
+    const float *part = a.part + a.part_off[t];
+    float *out = a.gw[t];
+    if (x >= total) {
+        x -= total;
+        if (!a.gb[t] || x >= a.C[t]) return;
+        part += (int64_t)slices * total;
+        total = a.C[t];
+        out = a.gb[t];
+    }
+    float a0 = 0.f, a1 = 0.f;
+    int s = 0;
+    for (; s + 1 < slices; s += 2) {
+        a0 += part[(int64_t)s * total + x];
+        a1 += part[(int64_t)(s + 1) * total + x];
+    }
+    if (s < slices) a0 += part[(int64_t)s * total + x];
+    out[x] = a0 + a1;
+}
+
 }  // namespace
 
 extern "C" int cf_linear_rows(const float *x, int64_t N, int64_t K, const float *w0, const float *w1,
@@ -301,5 +399,77 @@ extern "C" int cf_linear_weight_grad(const float *g, const float *x, int64_t N, 
     add_slices_kernel<<<(int)((cells + 255) / 256), 256, 0, st>>>((const float *)workspace, slices, total, gW,
                                                                   part_b, C, gb);
     CF_CHECK_LAUNCH("cf_linear_weight_grad: sum");
+    return CF_OK;
+}
+
+extern "C" int64_t cf_linear_weight_grad_grouped_workspace(int n_layers, const int64_t *N, const int64_t *C,
+                                                           const int64_t *K)
+{
+    if (n_layers < 0 || (n_layers > 0 && (!N || !C || !K))) return -1;
+    int64_t bytes = 0;
+    for (int t = 0; t < n_layers; t++) {
+        const int64_t b = cf_linear_weight_grad_workspace(N[t], C[t], K[t]);
+        if (b < 0) return -1;
+        bytes += b;
+    }
+    return bytes > 0 ? bytes : (int64_t)sizeof(float);
+}
+
+extern "C" int cf_linear_weight_grad_grouped(int n_layers, const float *const *g, const float *const *x,
+                                             const int64_t *N, const int64_t *C, const int64_t *K,
+                                             float *const *gW, float *const *gb, void *workspace,
+                                             int64_t workspace_bytes, void *stream)
+{
+    CF_REQUIRE(n_layers >= 0, CF_ERR_INVALID_ARGUMENT, "cf_linear_weight_grad_grouped: negative layer count");
+    if (n_layers == 0) return CF_OK;
+    CF_REQUIRE(g && x && N && C && K && gW && gb, CF_ERR_INVALID_ARGUMENT,
+               "cf_linear_weight_grad_grouped: null table");
+    for (int t = 0; t < n_layers; t++) {
+        CF_REQUIRE(N[t] >= 0 && N[t] < (1ll << 31) && C[t] >= 1 && K[t] >= 1 && C[t] < (1 << 20) && K[t] < (1 << 20),
+                   CF_ERR_INVALID_ARGUMENT, "cf_linear_weight_grad_grouped: bad sizes of layer %d", t);
+        CF_REQUIRE(gW[t] && (N[t] == 0 || (g[t] && x[t])), CF_ERR_INVALID_ARGUMENT,
+                   "cf_linear_weight_grad_grouped: null pointer in layer %d", t);
+    }
+    const int64_t need = cf_linear_weight_grad_grouped_workspace(n_layers, N, C, K);
+    CF_REQUIRE(workspace && workspace_bytes >= need, CF_ERR_INVALID_ARGUMENT,
+               "cf_linear_weight_grad_grouped: workspace of %lld bytes needed", (long long)need);
+    hipStream_t st = (hipStream_t)stream;
+    int64_t off = 0;
+    for (int first = 0; first < n_layers; first += WG_GROUP) {
+        WeightGradGroup a;
+        a.count = n_layers - first < WG_GROUP ? n_layers - first : WG_GROUP;
+        a.part = (float *)workspace;
+        int64_t tiles = 0, cells = 0;
+        int max_slices = 1;
+        for (int k = 0; k < WG_GROUP; k++) {
+            const int t = first + k;
+            const bool live = k < a.count;
+            a.g[k] = live ? g[t] : nullptr;
+            a.x[k] = live ? x[t] : nullptr;
+            a.gw[k] = live ? gW[t] : nullptr;
+            a.gb[k] = live ? gb[t] : nullptr;
+            a.N[k] = live ? (int)N[t] : 0;
+            a.C[k] = live ? (int)C[t] : 1;
+            a.K[k] = live ? (int)K[t] : 1;
+            a.slices[k] = live ? weight_grad_slices(N[t]) : 1;
+            a.part_off[k] = off;
+            a.tile0[k] = (int)tiles;
+            a.cell0[k] = (int)cells;
+            if (live) {
+                off += cf_linear_weight_grad_workspace(N[t], C[t], K[t]) / (int64_t)sizeof(float);
+                tiles += ((C[t] + 31) / 32) * ((K[t] + 31) / 32);
+                cells += (C[t] * (K[t] + 1) + 255) / 256;
+                if (a.slices[k] > max_slices) max_slices = a.slices[k];
+                CF_REQUIRE(tiles < (1ll << 30) && cells < (1ll << 30), CF_ERR_UNSUPPORTED,
+                           "cf_linear_weight_grad_grouped: too large");
+            }
+        }
+        a.tile0[WG_GROUP] = (int)tiles;
+        a.cell0[WG_GROUP] = (int)cells;
+        weight_grad_group_slices_kernel<<<dim3((unsigned)tiles, (unsigned)max_slices), 256, 0, st>>>(a);
+        CF_CHECK_LAUNCH("cf_linear_weight_grad_grouped: slices");
+        weight_grad_group_add_kernel<<<(unsigned)cells, 256, 0, st>>>(a);
+        CF_CHECK_LAUNCH("cf_linear_weight_grad_grouped: sum");
+    }
     return CF_OK;
 }

@@ -21,6 +21,7 @@ from torch.nn.init import constant_, xavier_uniform_
 from . import ops
 from .attention import CrystalformerMultiheadAttentionCUDA
 from .hip_funcs import compile_kernels
+from . import hip_funcs
 from .hip_funcs import linear as linear_hip
 from .params import LatticeformerParams
 
@@ -122,6 +123,16 @@ class CrystalformerEncoderLayerCUDA(Module):
                 # 11 us against 8 us for the library GEMM plus the add at 1774 x 512 -> 128)
                 x = x + F.linear(h, self.linear2.weight, self.linear2.bias)
             return x
+        if self._fused_train(x):
+            # the same epilogues with autograd (graphed training step, no norm layers, no dropout)
+            x = self.self_attn(x, x, x, batch, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell,
+                               onehot, need_weights=False, residual=x)[0]
+            h, = hip_funcs.FusedLinearHIP.apply(x, self.linear1.bias, None, True, self.linear1.weight)
+            if self.linear2.weight.shape[1] <= 256:
+                x, = hip_funcs.FusedLinearHIP.apply(h, self.linear2.bias, x, False, self.linear2.weight)
+            else:
+                x = x + linear_hip(h, self.linear2.weight, self.linear2.bias)
+            return x
         if self.norm_first:
             x = x + self._sa_block(self.norm1(x), batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot)
             x = x + self._ff_block(self.norm2(x))
@@ -140,6 +151,13 @@ class CrystalformerEncoderLayerCUDA(Module):
                 and ops.linear_rows_supported(x, self.linear1.weight)
                 and ops.linear_rows_supported(x, self.self_attn.out_proj.weight)
                 and self.linear2.weight.is_cuda and self.linear2.weight.shape[1] % 16 == 0)
+
+    def _fused_train(self, x: Tensor) -> bool:
+        plain = isinstance(self.norm1, Identity) and isinstance(self.norm2, Identity)
+        no_drop = all(isinstance(d, Identity) for d in (self.dropout, self.dropout1, self.dropout2))
+        return (hip_funcs.USE_LINEAR_FUNCTION and torch.is_grad_enabled() and plain and no_drop
+                and self.activation is F.relu and ops.linear_rows_supported(x, self.linear1.weight)
+                and self.linear2.weight.shape[1] % 16 == 0)
 
     def _sa_block(self, x, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot):
         x = self.self_attn(x, x, x, batch, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell,

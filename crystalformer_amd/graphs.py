@@ -113,9 +113,11 @@ class GraphedTrainStep:
 
     def _step_body(self) -> torch.Tensor:
         import torch.nn.functional as F
+        from . import hip_funcs
         out = self.model(self.static)
         loss = F.l1_loss(out[:, 0], self.static.y, reduction="none").mean()
-        loss.backward()
+        with hip_funcs.deferred_weight_grads():           # all linear layers' weight gradients at the end
+            loss.backward()
         self.opt.step()
         return loss.detach()
 

@@ -269,6 +269,8 @@ class LinearRowsHIP(torch.autograd.Function):
     def forward(ctx, x, weight, bias):
         ctx.save_for_backward(x, weight)
         ctx.has_bias = bias is not None
+        # the parameters themselves (leaves only: no cycle through the graph), for deferred gradients
+        ctx.leaves = (weight if weight.is_leaf else None, bias if (bias is not None and bias.is_leaf) else None)
         return torch.nn.functional.linear(x, weight, bias)
 
     @staticmethod
@@ -278,13 +280,121 @@ class LinearRowsHIP(torch.autograd.Function):
         gx = g @ weight if ctx.needs_input_grad[0] else None
         want_b = ctx.has_bias and ctx.needs_input_grad[2]
         gw = gb = None
-        if ctx.needs_input_grad[1]:
+        weight_p, bias_p = ctx.leaves
+        if _deferred is not None and ctx.needs_input_grad[1] and weight_p is not None and weight_p.grad is None \
+                and (not want_b or (bias_p is not None and bias_p.grad is None)):
+            # all layers' weight gradients are computed together after the backward pass
+            _deferred.append((g, x.contiguous(), weight_p, bias_p if want_b else None, 0))
+        elif ctx.needs_input_grad[1]:
             gw = ops.linear_weight_grad(g, x.contiguous(), with_bias=want_b)
             if want_b:
                 gw, gb = gw
         elif want_b:
             gb = ops.column_sum(g)
         return gx, gw, gb
+
+
+class FusedLinearHIP(torch.autograd.Function):
+    """``(y_0, ..)`` with ``y_i = act(x W_i^T + b_i) (+ residual)`` for up to three equally
+    shaped weights sharing the input (query / key / value projections) in one row-block
+    launch, bias, ReLU and residual in its epilogue.  ``bias`` is one vector over all
+    outputs (n_weights * C).  Backward: the input gradient as library GEMMs accumulating
+    into one buffer, weight and bias gradients from the grouped fixed-order kernel (deferred
+    to the end of the backward pass inside :class:`deferred_weight_grads`)."""
+
+    @staticmethod
+    def forward(ctx, x, bias, residual, relu, *weights):
+        if relu and (residual is not None or len(weights) != 1):
+            raise ValueError("FusedLinearHIP: ReLU goes with a single weight and no residual")
+        x = x.contiguous()
+        ys = ops.linear_rows(x, weights, bias, residual=residual, relu=relu)
+        ctx.save_for_backward(x, *weights, *((ys[0],) if relu else ()))
+        ctx.relu, ctx.nw = relu, len(weights)
+        # the parameters themselves (leaves only: no cycle through the graph), for deferred gradients
+        ctx.leaves = ([w if w.is_leaf else None for w in weights],
+                      bias if (bias is not None and bias.is_leaf) else None, bias is not None)
+        return tuple(ys)
+
+    @staticmethod
+    def backward(ctx, *gs):
+        saved = ctx.saved_tensors
+        x, weights = saved[0], saved[1:1 + ctx.nw]
+        C = weights[0].shape[0]
+        gs = [g.contiguous() if g is not None else None for g in gs]
+        if ctx.relu and gs[0] is not None:
+            gs[0] = torch.ops.aten.threshold_backward(gs[0], saved[-1], 0)
+        g_res = gs[0] if ctx.needs_input_grad[2] else None
+        gx = None
+        if ctx.needs_input_grad[0]:
+            for g, w in zip(gs, weights):
+                if g is not None:
+                    gx = torch.mm(g, w) if gx is None else gx.addmm_(g, w)
+            if gx is None:
+                gx = torch.zeros_like(x)
+        need_w = [ctx.needs_input_grad[4 + i] for i in range(ctx.nw)]
+        leaves_w, bias_p, has_bias = ctx.leaves
+        want_b = has_bias and ctx.needs_input_grad[1]
+        gws = [None] * ctx.nw
+        gb = None
+        if any(need_w) or want_b:
+            gs = [g if g is not None else torch.zeros((x.shape[0], C), dtype=x.dtype, device=x.device) for g in gs]
+            if _deferred is not None and all(need_w) and all(w is not None and w.grad is None for w in leaves_w) \
+                    and (not has_bias or (want_b and bias_p is not None and bias_p.grad is None)):
+                for i in range(ctx.nw):
+                    _deferred.append((gs[i], x, leaves_w[i], bias_p, i * C))
+            else:
+                gb = torch.empty(ctx.nw * C, dtype=x.dtype, device=x.device) if want_b else None
+                gws = [torch.empty_like(w, memory_format=torch.contiguous_format) for w in weights]
+                ops.linear_weight_grad_grouped([(gs[i], x, gws[i], gb[i * C:(i + 1) * C] if want_b else None)
+                                                for i in range(ctx.nw)])
+                gws = [gw if need else None for gw, need in zip(gws, need_w)]
+        return (gx, gb, g_res, None, *gws)
+
+
+# A list while a training step defers its linear layers' weight gradients (see
+# :func:`deferred_weight_grads`), else None.
+_deferred = None
+
+
+class deferred_weight_grads:
+    """Context for ``loss.backward()``: linear layers routed through :class:`LinearRowsHIP`
+    leave their parameters' gradients unset during the backward pass and the context's exit
+    computes them all in one grouped launch pair, writing ``.grad`` directly.  Only
+    parameters without an existing gradient take part (no accumulation)."""
+
+    def __enter__(self):
+        global _deferred
+        self.previous = _deferred
+        _deferred = []
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        global _deferred
+        pending, _deferred = _deferred, self.previous
+        if exc_type is not None or not pending:
+            return False
+        layers, seen, bias_grads = [], set(), {}
+        for g, x, weight_p, bias_p, bias_off in pending:
+            if id(weight_p) in seen or weight_p.grad is not None or (bias_p is not None and bias_p.grad is not None):
+                raise RuntimeError("deferred weight gradients: a parameter is used by more than one layer")
+            seen.add(id(weight_p))
+            gw = torch.empty_like(weight_p, memory_format=torch.contiguous_format)
+            gb = None
+            if bias_p is not None:                  # several layers may own slices of one bias vector
+                entry = bias_grads.setdefault(id(bias_p), [bias_p, torch.empty(bias_p.numel(), dtype=bias_p.dtype,
+                                                                               device=bias_p.device), 0])
+                gb = entry[1][bias_off:bias_off + g.shape[1]]
+                entry[2] += g.shape[1]
+            layers.append((g, x, gw, gb))
+        for bias_p, full, covered in bias_grads.values():
+            if covered != bias_p.numel():
+                raise RuntimeError("deferred weight gradients: a bias vector is only partly used")
+        ops.linear_weight_grad_grouped(layers)
+        for (g, x, gw, gb), (_, _, weight_p, _, _) in zip(layers, pending):
+            weight_p.grad = gw
+        for bias_p, full, covered in bias_grads.values():
+            bias_p.grad = full.view(bias_p.shape)
+        return False
 
 
 # Set by the graphed training step (around capture and around its eager twin); plain eager

@@ -45,6 +45,8 @@ SIGNATURES = {
     "cf_linear_rows": (_int, [_ptr, _i64, _i64, _ptr, _ptr, _ptr, _int, _i64, _ptr, _ptr, _int, _ptr, _ptr, _ptr, _ptr]),
     "cf_linear_weight_grad_workspace": (_i64, [_i64, _i64, _i64]),
     "cf_linear_weight_grad": (_int, [_ptr, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),
+    "cf_linear_weight_grad_grouped_workspace": (_i64, [_int, _ptr, _ptr, _ptr]),
+    "cf_linear_weight_grad_grouped": (_int, [_int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
     "cf_column_sum": (_int, [_ptr, _i64, _i64, _ptr, _ptr]),
     "cf_gauss_exponents_bwd_workspace": (_i64, [_i64, _i64, _i64]),
     "cf_gauss_exponents_bwd": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _f32, _f32, _f32,

@@ -660,6 +660,39 @@ def linear_weight_grad(g: Tensor, x: Tensor, with_bias: bool = False):
     return (out, gb) if with_bias else out
 
 
+def linear_weight_grad_grouped(layers) -> None:
+    """Weight and bias gradients of several linear layers in two launches.  ``layers`` is a
+    list of ``(g (N,C), x (N,K), gW out (C,K), gb out (C) or None)``; the outputs are
+    written in place and equal :func:`linear_weight_grad` bit for bit."""
+    import ctypes
+    if not layers:
+        return
+    flat = [t for layer in layers for t in layer]
+    dev = require_device(*flat)
+    n = len(layers)
+    for g, x, gw, gb in layers:
+        for t in (g, x, gw, gb):
+            if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+                raise _lib.CrystalformerHipError("linear_weight_grad_grouped: contiguous float32 tensors expected")
+        if g.dim() != 2 or x.dim() != 2 or g.shape[0] != x.shape[0] or gw.shape != (g.shape[1], x.shape[1]) \
+                or (gb is not None and gb.numel() != g.shape[1]):
+            raise _lib.CrystalformerHipError("linear_weight_grad_grouped: g (N,C), x (N,K), gW (C,K), gb (C) expected")
+    PtrArr, I64Arr = ctypes.c_void_p * n, ctypes.c_int64 * n
+    Ns = I64Arr(*[l[0].shape[0] for l in layers])
+    Cs = I64Arr(*[l[0].shape[1] for l in layers])
+    Ks = I64Arr(*[l[1].shape[1] for l in layers])
+    lib = _lib.load()
+    ws_bytes = int(lib.cf_linear_weight_grad_grouped_workspace(n, Ns, Cs, Ks))
+    ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=dev)
+    with device_guard(dev):
+        rc = lib.cf_linear_weight_grad_grouped(
+            n, PtrArr(*[l[0].data_ptr() for l in layers]), PtrArr(*[l[1].data_ptr() for l in layers]), Ns, Cs, Ks,
+            PtrArr(*[l[2].data_ptr() for l in layers]),
+            PtrArr(*[(l[3].data_ptr() if l[3] is not None else None) for l in layers]),
+            ptr(ws), ws_bytes, stream_handle(dev))
+    check(rc, "cf_linear_weight_grad_grouped")
+
+
 class AdamWPlan:
     """Host-side tables for :func:`adamw_step`: the pointer arrays of the parameters and
     moments (fixed for the life of the optimiser), element counts, decay factors and the

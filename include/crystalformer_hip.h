@@ -318,6 +318,18 @@ int cf_linear_weight_grad(const float *g, const float *x, int64_t N, int64_t C, 
                           void *workspace, int64_t workspace_bytes, float *gW, float *gb, void *stream);
 
 /*
+ * cf_linear_weight_grad for n_layers linear layers at once (2 * ceil(n_layers / 16)
+ * launches instead of 2 * n_layers); per layer the result is bit-identical to the single
+ * call.  g, x, gW, gb: HOST arrays of device pointers (gb[t] may be NULL); N, C, K: HOST
+ * arrays.  workspace: cf_linear_weight_grad_grouped_workspace(n_layers, N, C, K) bytes.
+ */
+int64_t cf_linear_weight_grad_grouped_workspace(int n_layers, const int64_t *N, const int64_t *C,
+                                                const int64_t *K);
+int cf_linear_weight_grad_grouped(int n_layers, const float *const *g, const float *const *x, const int64_t *N,
+                                  const int64_t *C, const int64_t *K, float *const *gW, float *const *gb,
+                                  void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * One optimiser update of a training step over n_tensors parameter tensors: global
  * gradient-norm clip (nn.utils.clip_grad_norm_, models/regression.py:122), AdamW
  * (optim.AdamW, models/regression.py:254; decoupled weight decay per tensor, betas, eps)

@@ -645,3 +645,95 @@ def test_gauss_exponents_bwd_kernel(dev, func, N, H, D, scaled):
     only_w = ops.gauss_exponents_bwd(ga.to(dev), None, q.to(dev), w.to(dev), alpha_n.detach().float().to(dev),
                                      used.to(dev) if scaled else None, func, beta, lb, coef, q_scale, want_gq=False)
     assert only_w[0] is None and torch.equal(only_w[1], gw)
+
+
+def test_linear_weight_grad_grouped_equals_single_calls(dev):
+    """Twenty layers of ragged shapes (two kernel-argument groups, with and without bias,
+    different row counts and slice counts) in one grouped call: bit-identical to one call each."""
+    gen = torch.Generator().manual_seed(21)
+    shapes = [(1774, 128, 128), (1774, 512, 128), (1774, 128, 512), (70, 48, 32), (3, 5, 7), (600, 33, 100)]
+    shapes = shapes * 3 + [(1774, 128, 128), (40, 16, 16)]
+    layers, expect = [], []
+    for k, (N, C, K) in enumerate(shapes):
+        g, x = torch.randn(N, C, generator=gen).to(dev), torch.randn(N, K, generator=gen).to(dev)
+        bias = k % 3 != 0
+        expect.append(ops.linear_weight_grad(g, x, with_bias=True) if bias else (ops.linear_weight_grad(g, x), None))
+        layers.append((g, x, torch.full((C, K), float("nan"), device=dev),
+                       torch.full((C,), float("nan"), device=dev) if bias else None))
+    ops.linear_weight_grad_grouped(layers)
+    for k, ((g, x, gw, gb), (gw_ref, gb_ref)) in enumerate(zip(layers, expect)):
+        assert torch.equal(gw, gw_ref), (k, shapes[k])
+        assert (gb is None) == (gb_ref is None) and (gb is None or torch.equal(gb, gb_ref)), (k, shapes[k])
+
+
+def test_deferred_weight_grads_match_immediate(dev):
+    """Linear layers inside deferred_weight_grads(): parameter gradients appear at the
+    context's exit and equal, bit for bit, those of the same backward pass without deferral."""
+    from crystalformer_amd import hip_funcs
+    gen = torch.Generator().manual_seed(5)
+    x0 = torch.randn(300, 64, generator=gen).to(dev)
+    target = torch.randn(300, 32, generator=gen).to(dev)
+
+    def run(defer):
+        torch.manual_seed(3)
+        l1, l2 = torch.nn.Linear(64, 128).to(dev), torch.nn.Linear(128, 32, bias=False).to(dev)
+        x = x0.clone().requires_grad_()
+        h = torch.relu(hip_funcs.LinearRowsHIP.apply(x, l1.weight, l1.bias))
+        loss = (hip_funcs.LinearRowsHIP.apply(h, l2.weight, None) - target).square().mean()
+        if defer:
+            with hip_funcs.deferred_weight_grads():
+                loss.backward()
+                assert l1.weight.grad is None and l2.weight.grad is None      # not yet
+        else:
+            loss.backward()
+        return [x.grad, l1.weight.grad, l1.bias.grad, l2.weight.grad]
+
+    for a, b in zip(run(True), run(False)):
+        assert a is not None and torch.equal(a, b)
+    assert hip_funcs._deferred is None
+
+
+@pytest.mark.parametrize("defer", [False, True])
+def test_fused_linear_function_grads(dev, defer):
+    """FusedLinearHIP (three projections sharing an input and one bias vector; ReLU layer;
+    residual layer) against float64 autograd of the same expression, immediate and deferred
+    weight gradients."""
+    from crystalformer_amd import hip_funcs
+    gen = torch.Generator().manual_seed(17)
+    N, K, C = 333, 64, 48
+    x0 = torch.randn(N, K, generator=gen)
+    ws = [torch.randn(C, K, generator=gen) * 0.2 for _ in range(3)]
+    b3 = torch.randn(3 * C, generator=gen)
+    w1, b1 = torch.randn(K, C, generator=gen) * 0.2, torch.randn(K, generator=gen)
+    w2, b2 = torch.randn(K, K, generator=gen) * 0.2, torch.randn(K, generator=gen)
+    tq, tk, tv = (torch.randn(N, C, generator=gen) for _ in range(3))
+
+    def graph(x, ws, b3, w1, b1, w2, b2, lin3, lin_relu, lin_res):
+        q, k, v = lin3(x, b3, ws)
+        h = lin_relu(q * tq.to(q) + k * tk.to(q) - v * tv.to(q), b1, w1)        # (N, K)
+        y = lin_res(h, b2, x, w2)                                                # + residual x
+        return (y * y).mean()
+
+    leaves64 = [t.double().requires_grad_() for t in (x0, *ws, b3, w1, b1, w2, b2)]
+    x, a, b, c, bb, w1d, b1d, w2d, b2d = leaves64
+    graph(x, (a, b, c), bb, w1d, b1d, w2d, b2d,
+          lambda x, b3, ws: tuple(torch.nn.functional.linear(x, w, bs) for w, bs in zip(ws, b3.split(C))),
+          lambda x, b, w: torch.relu(torch.nn.functional.linear(x, w, b)),
+          lambda x, b, r, w: torch.nn.functional.linear(x, w, b) + r).backward()
+
+    leaves = [t.to(dev).requires_grad_() for t in (x0, *ws, b3, w1, b1, w2, b2)]
+    x, a, b, c, bb, w1d, b1d, w2d, b2d = leaves
+    loss = graph(x, (a, b, c), bb, w1d, b1d, w2d, b2d,
+                 lambda x, b3, ws: hip_funcs.FusedLinearHIP.apply(x, b3, None, False, *ws),
+                 lambda x, b, w: hip_funcs.FusedLinearHIP.apply(x, b, None, True, w)[0],
+                 lambda x, b, r, w: hip_funcs.FusedLinearHIP.apply(x, b, r, False, w)[0])
+    if defer:
+        with hip_funcs.deferred_weight_grads():
+            loss.backward()
+            assert a.grad is None and bb.grad is None
+    else:
+        loss.backward()
+    names = ["x", "wq", "wk", "wv", "b3", "w1", "b1", "w2", "b2"]
+    for name, t, r in zip(names, leaves, leaves64):
+        assert t.grad is not None, name
+        assert_close(t.grad, r.grad.float(), name, rtol=5e-6)
