@@ -142,16 +142,27 @@ def crystal_offsets(batch_i: Tensor, num_slots: Optional[int] = None) -> Tuple[T
 
 # Scheduling words of the pair-evaluated forward (two zeroed int32 the work-groups draw their
 # rounds from; the kernel leaves them zeroed).  Launches that may overlap need words of their
-# own: eager launches on one stream run in order and share one pair per (device, stream); under
-# stream capture every launch gets a fresh zero-filled pair, because graphs captured on one
-# stream can later be replayed side by side.
+# own: eager launches on one stream run in order and share one pair per (device, stream).
+# Graphs captured on one stream can later be replayed side by side, so under stream capture
+# every launch gets a pair no other launch ever uses, cut from a zeroed per-device buffer
+# that lives as long as the process (no fill node in the graph); once that is used up, or if
+# nothing ran eagerly on the device before the capture, a fresh zero-filled pair.
 DYNAMIC_ROUNDS = True
 _sched_words: dict = {}
+_capture_words: dict = {}            # device index -> [buffer, pairs handed out]
+_CAPTURE_PAIRS = 8192
 
 
 def _scheduling_words(dev: torch.device) -> Tensor:
     if torch.cuda.is_current_stream_capturing():
-        return torch.zeros(2, dtype=torch.int32, device=dev)
+        pool = _capture_words.get(dev.index)
+        if pool is None or pool[1] >= _CAPTURE_PAIRS:
+            return torch.zeros(2, dtype=torch.int32, device=dev)
+        k = pool[1]
+        pool[1] = k + 1
+        return pool[0][2 * k:2 * k + 2]
+    if dev.index not in _capture_words:
+        _capture_words[dev.index] = [torch.zeros(2 * _CAPTURE_PAIRS, dtype=torch.int32, device=dev), 0]
     key = (dev.index, stream_handle(dev))
     words = _sched_words.get(key)
     if words is None:
