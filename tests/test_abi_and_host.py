@@ -137,3 +137,67 @@ def test_benchmark_configs_have_the_stated_sizes():
     assert float(lens[:, 0].min()) >= 20 and float(lens[:, 1:].max()) <= 8 + 1e-4
     assert set(CONFIGS) == {"cfg1_simplified_b32", "cfg2_default_b128", "cfg3_7block_b256", "cfg4_train_b128",
                             "cfg5_stress_b16"}
+
+
+def test_crystal_data_and_collate_follow_the_reference_contract():
+    """Fields as the reference's make_data builds them (dataloaders/dataset_latticeformer.py:32-38,
+    species one-hot at Z-1 per dataloaders/common.py:44-46) and as batching concatenates them."""
+    from crystalformer_amd.data import collate, crystal_data
+    lat = [[4.0, 0.0, 0.0], [1.0, 5.0, 0.0], [0.5, 0.25, 6.0]]
+    a = crystal_data([11, 17], [[0.0, 0.0, 0.0], [2.0, 2.5, 3.0]], lat, y=1.5)
+    b = crystal_data([26], [[0.5, 0.5, 0.5]], lat, y=-0.5, frac_coords=True)
+    c = crystal_data([1, 8, 8], [[0.1, 0.2, 0.3], [0.0, 0.0, 0.0], [0.9, 0.9, 0.9]], torch.eye(3) * 3, y=0.0)
+    assert a.x.shape == (2, 98) and a.x[0, 10] == 1 and a.x[1, 16] == 1 and float(a.x.sum()) == 2
+    assert a.trans_vec.shape == (1, 3, 3) and a.sizes.tolist() == [2] and a.batch.tolist() == [0, 0]
+    assert torch.allclose(b.pos, torch.tensor([[2.75, 2.625, 3.0]]))       # 0.5 * (sum of the lattice rows)
+    batch = collate([a, b, c])
+    assert batch.sizes.tolist() == [2, 1, 3] and batch.batch.tolist() == [0, 0, 1, 2, 2, 2]
+    assert batch.pos.shape == (6, 3) and batch.trans_vec.shape == (3, 3, 3) and batch.y.tolist() == [1.5, -0.5, 0.0]
+    assert torch.equal(batch.x[3], torch.eye(98)[0]) and torch.equal(batch.trans_vec[2], torch.eye(3) * 3)
+    again = collate([collate([a, b]), c])                                  # batches collate like crystals
+    assert torch.equal(again.batch, batch.batch) and torch.equal(again.pos, batch.pos)
+    assert collate([a, crystal_data([3], [[0, 0, 0]], lat)]).y is None      # a part without target drops them
+    for bad in ([0], [99], []):
+        with pytest.raises(ValueError):
+            crystal_data(bad, [[0.0, 0.0, 0.0]] * len(bad), lat)
+
+
+def test_reference_checkpoint_loading(tmp_path):
+    """A checkpoint laid out as the reference's trainer writes it (model under
+    ``swa_model.module.``, a second copy under ``model.``, the averaging counter, target
+    statistics; demo.py:67-89): the averaged weights are loaded and the target statistics
+    folded into the last linear layer, through the safe loader."""
+    from crystalformer_amd.data import load_reference_checkpoint, reference_state_dict
+    from crystalformer_amd.latticeformer import Latticeformer, default_params
+    cfg = default_params(num_layers=1, value_pe_dist_real=8)
+    torch.manual_seed(3)
+    source = Latticeformer(cfg)
+    torch.manual_seed(4)
+    other = Latticeformer(cfg)
+    state = {f"swa_model.module.{k}": v.clone() for k, v in source.state_dict().items()}
+    state.update({f"model.{k}": v.clone() for k, v in other.state_dict().items()})
+    state["swa_model.n_averaged"] = torch.tensor(7)
+    state["target_std"] = torch.tensor([2.5])
+    state["target_mean"] = torch.tensor([-0.75])
+    path = tmp_path / "last.ckpt"
+    torch.save({"epoch": 3, "global_step": 100, "state_dict": state}, path)
+
+    torch.manual_seed(5)
+    model = load_reference_checkpoint(Latticeformer(cfg), str(path))
+    want = source.state_dict()
+    assert set(reference_state_dict({"state_dict": state})) == set(want)
+    last_w, last_b = [k for k in want if k.startswith("mlp.")][-2:]
+    for k, v in model.state_dict().items():
+        if k == last_w:
+            assert torch.equal(v, want[k] * 2.5)
+        elif k == last_b:
+            assert torch.equal(v, want[k] * 2.5 - 0.75)
+        else:
+            assert torch.equal(v, want[k]), k
+    feats = torch.randn(5, want[[k for k in want if k.startswith("mlp.")][0]].shape[1])
+    assert torch.allclose(model.mlp(feats), source.mlp(feats) * 2.5 - 0.75, atol=1e-6)
+    plain = load_reference_checkpoint(Latticeformer(cfg), {"state_dict": state}, prefix="model.",
+                                      fold_target_normalisation=False)
+    assert all(torch.equal(v, other.state_dict()[k]) for k, v in plain.state_dict().items())
+    with pytest.raises(KeyError):
+        load_reference_checkpoint(Latticeformer(cfg), {"state_dict": {"x": torch.zeros(1)}})

@@ -341,3 +341,29 @@ def test_graph_survives_index_cache_eviction(dev):
     y = graphed().clone()
     torch.cuda.synchronize()
     assert torch.equal(y, y_eager) and held and junk
+
+
+def test_forward_from_plain_structures_and_checkpoint(dev, tmp_path):
+    """Crystals given as atomic numbers / coordinates / lattice rows, weights from a checkpoint
+    laid out like the reference's (demo.py:67-89): the HIP model's de-normalised output equals
+    the CPU oracle's output * std + mean on the same crystals."""
+    from crystalformer_amd.data import collate, crystal_data, load_reference_checkpoint
+    gen = torch.Generator().manual_seed(12)
+    crystals = []
+    for n in (1, 3, 7, 2):
+        lat = torch.eye(3) * (4.0 + torch.rand(3, generator=gen) * 3) + torch.rand(3, 3, generator=gen) * 0.7
+        crystals.append(crystal_data(torch.randint(1, 95, (n,), generator=gen).tolist(),
+                                     torch.rand(n, 3, generator=gen), lat, frac_coords=True))
+    b = collate(crystals)
+    cfg, source = build_model("cfg2_default_b128", num_layers=2, value_pe_dist_real=16, adaptive_cutoff_sigma=0.0)
+    state = {f"swa_model.module.{k}": v.clone() for k, v in source.state_dict().items()}
+    state["target_std"], state["target_mean"] = torch.tensor([3.0]), torch.tensor([0.25])
+    torch.save({"state_dict": state}, tmp_path / "m.ckpt")
+    P = {k: v.detach().clone() for k, v in source.state_dict().items()}
+    with torch.no_grad():
+        y_ref = om.latticeformer_forward(P, cfg, b) * 3.0 + 0.25
+    _, model = build_model("cfg2_default_b128", seed=9, num_layers=2, value_pe_dist_real=16, adaptive_cutoff_sigma=0.0)
+    load_reference_checkpoint(model, str(tmp_path / "m.ckpt")).to(dev).eval()
+    with torch.no_grad():
+        y = model(b.to(dev))
+    assert_close(y, y_ref, "de-normalised output")
