@@ -32,6 +32,7 @@ __all__ = [
     "KernelManager", "compile_kernels", "CUPY_AVAILABLE", "HIP_AVAILABLE",
     "RealPeriodicEncodingFuncCUDA", "RealPeriodicEncodingWithProjFuncCUDA",
     "FusedDotProductAttentionCUDA", "IrregularMeanCUDA", "compute_minimum_distance",
+    "ReciPeriodicEncodingFuncCUDA",
 ]
 
 
@@ -224,6 +225,32 @@ class FusedDotProductAttentionCUDA(torch.autograd.Function):
             que_ihk, key_ihk, val_ihk, bij_ehk, batch_i, edge_ij_e, e_start_i, prob_eh, output,
             go_ihk.contiguous().detach())
         return gque, gkey, gval, (gaij if ctx.has_aij else None), gbij, None, None
+
+
+class ReciPeriodicEncodingFuncCUDA(torch.autograd.Function):
+    """z[e,h] = log(max(sum_k exp(a[i,h] k^2) cos(k.r_e), 1e-6)) + 1.5 log(-4 pi a[i,h]) - log V, the
+    reciprocal-space lattice sum over the cube of ``KernelManager.LATTICE_RANGE``; gradient for
+    ``a_ik`` only, as the reference defines it (models/cuda_funcs/reci_space_enc.py:17-99: the
+    backward kernel differentiates the logarithm of the sum, not the normalisation term)."""
+
+    @staticmethod
+    def forward(ctx, a_ik, kr_base_e, rvecs_n, vcell_n, batch_i, edge_ij_e):
+        a_ik = a_ik.contiguous().detach()
+        kr_base_e, rvecs_n, vcell_n = kr_base_e.contiguous(), rvecs_n.contiguous(), vcell_n.contiguous()
+        batch_i, edge_ij_e = batch_i.contiguous(), edge_ij_e.contiguous()
+        e_start_i = ops.cached_edge_row_offsets(edge_ij_e, a_ik.shape[0])
+        z_ek, sumexp_ek = ops.reci_enc_fwd(a_ik, kr_base_e, rvecs_n, vcell_n, batch_i, e_start_i,
+                                           KernelManager.LATTICE_RANGE)
+        ctx.save_for_backward(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, sumexp_ek)
+        ctx.lattice_range = KernelManager.LATTICE_RANGE
+        return z_ek
+
+    @staticmethod
+    def backward(ctx, gz_ek):
+        a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, sumexp_ek = ctx.saved_tensors
+        ga_ik = ops.reci_enc_bwd(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, gz_ek.detach().contiguous(),
+                                 sumexp_ek, ctx.lattice_range)
+        return ga_ik, None, None, None, None, None
 
 
 class GaussianExponentsHIP(torch.autograd.Function):

@@ -568,6 +568,73 @@ def gauss_exponents(q_ihd: Tensor, w_hd: Tensor, gauss_scale: Optional[Tensor], 
     return a, qs, alpha_n, (ws[-4:-2] if normalize else None)
 
 
+def kr_base(rpos_ij_e: Tensor, rvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor) -> Tensor:
+    """(E,3) phases <b_d, p_j - p_i> of the reciprocal-space encoding
+    (models/indexed_latticeformer_encoder.py:245-251)."""
+    dev = require_device(rpos_ij_e, rvecs_n, batch_i, edge_ij_e)
+    rpos_ij_e, rvecs_n = _f32(rpos_ij_e, "rpos_ij_e"), _f32(rvecs_n, "rvecs_n")
+    batch_i, edge_ij_e = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e")
+    E = edge_ij_e.shape[1]
+    if rpos_ij_e.shape != (E, 3) or rvecs_n.shape[1:] != (3, 3):
+        raise _lib.CrystalformerHipError("kr_base: rpos (E,3) and rvecs (B,3,3) expected")
+    out = torch.empty((E, 3), dtype=torch.float32, device=dev)
+    with device_guard(dev):
+        rc = _lib.load().cf_kr_base(ptr(rpos_ij_e), ptr(rvecs_n), ptr(batch_i), ptr(edge_ij_e), E, ptr(out),
+                                    stream_handle(dev))
+    check(rc, "cf_kr_base")
+    return out
+
+
+def _reci_operands(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i):
+    a_ik, kr_base_e, rvecs_n = _f32(a_ik, "a_ik"), _f32(kr_base_e, "kr_base_e"), _f32(rvecs_n, "rvecs_n")
+    batch_i, e_start_i = _i64(batch_i, "batch_i"), _i64(e_start_i, "e_start_i")
+    if a_ik.dim() != 2 or kr_base_e.dim() != 2 or kr_base_e.shape[1] != 3 or rvecs_n.shape[1:] != (3, 3) \
+            or batch_i.shape != (a_ik.shape[0],) or e_start_i.shape != (a_ik.shape[0] + 1,):
+        raise _lib.CrystalformerHipError("reciprocal encoding: a (N,H), kr_base (E,3), rvecs (B,3,3), batch (N), "
+                                         "e_start (N+1) expected")
+    return a_ik, kr_base_e, rvecs_n, batch_i, e_start_i
+
+
+def reci_enc_fwd(a_ik: Tensor, kr_base_e: Tensor, rvecs_n: Tensor, vcell_n: Tensor, batch_i: Tensor,
+                 e_start_i: Tensor, lattice_range: int) -> Tuple[Tensor, Tensor]:
+    """``(z_ek, sumexp_ek)`` of the reciprocal-space lattice sum."""
+    dev = require_device(a_ik, kr_base_e, rvecs_n, vcell_n, batch_i, e_start_i)
+    a_ik, kr_base_e, rvecs_n, batch_i, e_start_i = _reci_operands(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i)
+    vcell_n = _f32(vcell_n, "vcell_n")
+    N, H = a_ik.shape
+    E = kr_base_e.shape[0]
+    if vcell_n.numel() != rvecs_n.shape[0]:
+        raise _lib.CrystalformerHipError("reciprocal encoding: one cell volume per crystal expected")
+    z = torch.empty((E, H), dtype=torch.float32, device=dev)
+    se = torch.empty((E, H), dtype=torch.float32, device=dev)
+    with device_guard(dev):
+        rc = _lib.load().cf_reci_enc_fwd(ptr(a_ik), ptr(kr_base_e), ptr(rvecs_n), ptr(vcell_n), ptr(batch_i),
+                                         ptr(e_start_i), N, H, E, int(lattice_range), ptr(z), ptr(se),
+                                         stream_handle(dev))
+    check(rc, "cf_reci_enc_fwd")
+    return z, se
+
+
+def reci_enc_bwd(a_ik: Tensor, kr_base_e: Tensor, rvecs_n: Tensor, batch_i: Tensor, e_start_i: Tensor,
+                 gz_ek: Tensor, sumexp_ek: Tensor, lattice_range: int) -> Tensor:
+    """``ga_ik`` of the reciprocal-space lattice sum (the reference's definition, which leaves
+    the normalisation term's derivative out)."""
+    dev = require_device(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, gz_ek, sumexp_ek)
+    a_ik, kr_base_e, rvecs_n, batch_i, e_start_i = _reci_operands(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i)
+    gz_ek, sumexp_ek = _f32(gz_ek, "gz_ek"), _f32(sumexp_ek, "sumexp_ek")
+    N, H = a_ik.shape
+    E = kr_base_e.shape[0]
+    if gz_ek.shape != (E, H) or sumexp_ek.shape != (E, H):
+        raise _lib.CrystalformerHipError("reciprocal encoding: gz and sumexp must be (E,H)")
+    ga = torch.empty((N, H), dtype=torch.float32, device=dev)
+    with device_guard(dev):
+        rc = _lib.load().cf_reci_enc_bwd(ptr(a_ik), ptr(kr_base_e), ptr(rvecs_n), ptr(batch_i), ptr(e_start_i),
+                                         ptr(gz_ek), ptr(sumexp_ek), N, H, E, int(lattice_range), ptr(ga),
+                                         stream_handle(dev))
+    check(rc, "cf_reci_enc_bwd")
+    return ga
+
+
 def gauss_exponents_bwd(ga: Optional[Tensor], gqs: Optional[Tensor], q_ihd: Tensor, w_hd: Tensor,
                         alpha_n: Tensor, used: Optional[Tensor], positive_func: str, beta: float,
                         lower_bound: float, coef: float, q_scale: float, want_gq: bool = True,

@@ -162,3 +162,27 @@ def minimum_distance(rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, cutoff_rad
                                _p(rvlen_n), _dbl(cutoff_radius), _int(lattice_range),
                                _int(minimum_range), _p(out))
     return out
+
+
+def reci_enc_fwd(a_ik, kr_base_e, rvecs_n, vcell_n, batch_i, edge_ij_e, lattice_range=2) -> Tuple[Tensor, Tensor]:
+    """(z_ek, sumexp_ek) of the reciprocal-space lattice sum (models/kernels/reci_enc_fwd.cu)."""
+    a_ik, kr_base_e, rvecs_n, vcell_n = _f(a_ik), _f(kr_base_e), _f(rvecs_n), _f(vcell_n)
+    batch_i, edge_ij_e = _l(batch_i), _l(edge_ij_e)
+    N, H = a_ik.shape
+    E = edge_ij_e.shape[1]
+    z = torch.empty((E, H), dtype=torch.float32)
+    se = torch.empty((E, H), dtype=torch.float32)
+    lib().ref_reci_enc_fwd(_p(a_ik), _p(kr_base_e), _p(rvecs_n), _p(vcell_n), _p(batch_i), _p(edge_ij_e),
+                           _i64(N), _i64(H), _i64(E), _int(lattice_range), _p(z), _p(se))
+    return z, se
+
+
+def reci_enc_bwd(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, gz_ek, sumexp_ek, lattice_range=2) -> Tensor:
+    """ga_ik (models/kernels/reci_enc_bwd.cu; without the normalisation term's derivative)."""
+    a_ik, kr_base_e, rvecs_n, gz_ek, sumexp_ek = _f(a_ik), _f(kr_base_e), _f(rvecs_n), _f(gz_ek), _f(sumexp_ek)
+    batch_i, e_start_i = _l(batch_i), _l(e_start_i)
+    N, H = a_ik.shape
+    ga = torch.empty((N, H), dtype=torch.float32)
+    lib().ref_reci_enc_bwd(_p(a_ik), _p(kr_base_e), _p(rvecs_n), _p(batch_i), _p(e_start_i), _p(gz_ek),
+                           _p(sumexp_ek), _i64(N), _i64(H), _int(lattice_range), _p(ga))
+    return ga

@@ -19,11 +19,17 @@
  *                            models/kernels/fused_dpa_bwd_q.cu:14-53
  *   ref_irregular_mean       models/kernels/irregular_mean_fwd.cu:4-90
  *   ref_minimum_distance     models/kernels/minimum_distance.cu:4-67
+ *   ref_reci_enc_fwd         models/kernels/reci_enc_fwd.cu:3-68
+ *   ref_reci_enc_bwd         models/kernels/reci_enc_bwd.cu:3-71
  *
  * Pins: tests/test_oracle_kernels.py checks these against the torch-path
  * oracle under rule A (cutoff 0), against brute force / closed forms, and the
  * range rule against its geometric invariant (every lattice point within the
- * cut-off lies in the box).
+ * cut-off lies in the box).  The reciprocal-space pair is pinned by the full-cube
+ * sum in float64, by the Poisson summation identity against the real-space
+ * lattice sum, by the torch-path restatement (other enumeration of the half
+ * space) and, for the backward, by finite differences of the forward minus the
+ * normalisation term the reference's kernel leaves out.
  */
 #include <math.h>
 #include <stdint.h>
@@ -363,5 +369,82 @@ void ref_minimum_distance(const float *rpos_ij_e, const float *tvecs_n, const i6
                     if (d2 < d2min) d2min = d2;
                 }
         dist2_min_e[e] = d2min;
+    }
+}
+
+/* Reciprocal-space lattice sum.  z[e,h] = log(max(S, 1e-6)) + 1.5 log(-4 pi a) - log(V) with
+ * S = sum over the half space n1 in [0,R] (weight 2 for n1 != 0), n2, n3 in [-R,R] of
+ * exp(a |k_n|^2) cos(<kr_base, n>), k_n = n1 b1 + n2 b2 + n3 b3 (rows of rvecs).  k_n, its
+ * square and the phase are float expressions as in the kernel; exp, cos and the sum are
+ * double here.  sumexp[e,h] = S. */
+void ref_reci_enc_fwd(const float *a_ik, const float *kr_base_e, const float *rvecs_n, const float *vcell_n,
+                      const i64 *batch_i, const i64 *edge_ij_e, i64 N, i64 H, i64 E, int lattice_range,
+                      float *z_ek, float *sumexp_ek)
+{
+    (void)N;
+    const int R = lattice_range;
+    for (i64 e = 0; e < E; e++) {
+        const i64 i = edge_ij_e[e];
+        const i64 n = batch_i[i];
+        const float *kr = kr_base_e + e * 3;
+        const float *rv = rvecs_n + n * 9;
+        for (i64 h = 0; h < H; h++) {
+            const float a = a_ik[i * H + h];
+            double sum = 0.0;
+            for (int m1 = 0; m1 <= R; m1++) {
+                const double scale = m1 == 0 ? 1.0 : 2.0;
+                for (int m2 = -R; m2 <= R; m2++)
+                    for (int m3 = -R; m3 <= R; m3++) {
+                        const float n1 = (float)m1, n2 = (float)m2, n3 = (float)m3;
+                        const float k1 = rv[0] * n1 + rv[3] * n2 + rv[6] * n3;
+                        const float k2 = rv[1] * n1 + rv[4] * n2 + rv[7] * n3;
+                        const float k3 = rv[2] * n1 + rv[5] * n2 + rv[8] * n3;
+                        const float kk = k1 * k1 + k2 * k2 + k3 * k3;
+                        const float ph = kr[0] * n1 + kr[1] * n2 + kr[2] * n3;
+                        sum += exp((double)(a * kk)) * cos((double)ph) * scale;
+                    }
+            }
+            const double log_ci = 1.5 * log(-12.5663706144 * (double)a) - log((double)vcell_n[n]);
+            z_ek[e * H + h] = (float)(log(sum > 1e-6 ? sum : 1e-6) + log_ci);
+            sumexp_ek[e * H + h] = (float)sum;
+        }
+    }
+}
+
+/* ga[i,h] = sum over the edges of row i of gz[e,h] / S[e,h] * sum_n |k_n|^2 exp(a |k_n|^2) cos(.)
+ * (zero where S < 1e-6).  As in the reference's kernel, the derivative of the normalisation
+ * term 1.5 log(-4 pi a) is NOT part of the result. */
+void ref_reci_enc_bwd(const float *a_ik, const float *kr_base_e, const float *rvecs_n, const i64 *batch_i,
+                      const i64 *e_start_i, const float *gz_ek, const float *sumexp_ek, i64 N, i64 H,
+                      int lattice_range, float *ga_ik)
+{
+    const int R = lattice_range;
+    for (i64 i = 0; i < N; i++) {
+        const i64 n = batch_i[i];
+        const float *rv = rvecs_n + n * 9;
+        for (i64 h = 0; h < H; h++) {
+            const float a = a_ik[i * H + h];
+            double total = 0.0;
+            for (i64 e = e_start_i[i]; e < e_start_i[i + 1]; e++) {
+                const float *kr = kr_base_e + e * 3;
+                double s = 0.0;
+                for (int m1 = 0; m1 <= R; m1++) {
+                    const double scale = m1 == 0 ? 1.0 : 2.0;
+                    for (int m2 = -R; m2 <= R; m2++)
+                        for (int m3 = -R; m3 <= R; m3++) {
+                            const float n1 = (float)m1, n2 = (float)m2, n3 = (float)m3;
+                            const float k1 = rv[0] * n1 + rv[3] * n2 + rv[6] * n3;
+                            const float k2 = rv[1] * n1 + rv[4] * n2 + rv[7] * n3;
+                            const float k3 = rv[2] * n1 + rv[5] * n2 + rv[8] * n3;
+                            const float kk = k1 * k1 + k2 * k2 + k3 * k3;
+                            const float ph = kr[0] * n1 + kr[1] * n2 + kr[2] * n3;
+                            s += (double)kk * exp((double)(a * kk)) * cos((double)ph) * scale;
+                        }
+                }
+                const float se = sumexp_ek[e * H + h];
+                total += s * (double)gz_ek[e * H + h] * (se < 1e-6f ? 0.0 : 1.0 / (double)se);
+            }
+            ga_ik[i * H + h] = (float)total;
+        }
     }
 }

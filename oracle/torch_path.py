@@ -15,6 +15,8 @@ What it restates (all paths relative to the reference checkout):
 * Gaussian value PE + proj      models/indexed_lattice_multi_head_attention.py:741-815, 1433-1445
 * per-crystal softmax/aggregate models/indexed_lattice_multi_head_attention.py:140-272
 * mean pooling                  models/pooling.py:19-25
+* reciprocal-space geometry     models/indexed_latticeformer_encoder.py:138-161
+* reciprocal-space lattice sum  models/indexed_lattice_multi_head_attention.py:925-950
 
 The translation set here is the fixed cube n in [-r, r]^3 ("rule A").  The
 adaptive per-head boxes of the device kernels ("rule B") live in
@@ -141,6 +143,49 @@ def lattice_dist2(pos: Tensor, batch: Tensor, trans: Tensor, edges: Tensor,
     disp = rel[:, None] + shifts[batch[ei]]              # (e,R,3)
     dist = torch.norm(disp, dim=-1)
     return dist * dist
+
+
+# --------------------------------------------------------------------------
+# reciprocal space
+# --------------------------------------------------------------------------
+def reciprocal_half_terms(pos: Tensor, batch: Tensor, trans: Tensor, edges: Tensor,
+                          lattice_range: int) -> Tuple[Tensor, Tensor, Tensor]:
+    """(cos_kr (E,Rh), k2 (B,Rh), vcell (B)) over the half grid: the second half of the
+    'ij'-ordered cube starting at its centre n = 0 (Rh = ((2r+1)^3 + 1) / 2 points), every
+    cosine but the first doubled to stand for the mirrored point.  k2 through the Gram
+    matrix of the reciprocal rows, as the reference prefers for accuracy.
+    Follows models/indexed_latticeformer_encoder.py:138-161."""
+    rec, vcell = reciprocal_vectors(trans)
+    grid = translation_grid(lattice_range, pos.dtype)
+    half = grid[grid.shape[0] // 2:]
+    rel = relative_positions(pos, edges)
+    b2e = batch[edges[0]]
+    kr = (rel[:, None] @ rec.transpose(1, 2)[b2e]).squeeze(1)           # (E,3): <r, b_d>
+    cos_kr = torch.cos((half @ kr[..., None]).squeeze(2))               # (E,Rh)
+    cos_kr[:, 1:] += cos_kr[:, 1:]
+    gram = rec @ rec.transpose(1, 2)                                    # (B,3,3)
+    outer = half[:, :, None] @ half[:, None, :]                         # (Rh,3,3)
+    k2 = (gram[:, None] * outer[None]).sum(dim=(2, 3))                  # (B,Rh)
+    return cos_kr, k2, vcell
+
+
+def reciprocal_bias(alpha: Tensor, cos_kr: Tensor, k2: Tensor, vcell: Tensor, edges0: Tensor,
+                    batch: Tensor) -> Tensor:
+    """z[e,h] = log(max(sum_k exp(a[i,h] k^2) cos(k.r), 1e-6)) + 1.5 log(-4 pi a[i,h]) - log V.
+    Follows models/indexed_lattice_multi_head_attention.py:925-950."""
+    alpha_k2 = alpha.unsqueeze(2) * k2.unsqueeze(1)[batch]              # (N,H,Rh)
+    s = (torch.exp(alpha_k2)[edges0] * cos_kr.unsqueeze(1)).sum(dim=-1)
+    z = torch.log(s.clamp(min=1e-6))
+    log_ci = 1.5 * torch.log((-4 * math.pi) * alpha) - torch.log(vcell)[batch, None]
+    return z + log_ci[edges0]
+
+
+def kr_base(pos: Tensor, batch: Tensor, trans: Tensor, edges: Tensor) -> Tensor:
+    """(E,3) phases <b_d, p_j - p_i> handed to the reciprocal-space kernels
+    (models/indexed_latticeformer_encoder.py:245-251)."""
+    rec, _ = reciprocal_vectors(trans)
+    rel = relative_positions(pos, edges)
+    return (rec[batch[edges[0]]] @ rel[..., None]).squeeze(2)
 
 
 # --------------------------------------------------------------------------

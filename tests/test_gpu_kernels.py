@@ -737,3 +737,60 @@ def test_fused_linear_function_grads(dev, defer):
     for name, t, r in zip(names, leaves, leaves64):
         assert t.grad is not None, name
         assert_close(t.grad, r.grad.float(), name, rtol=5e-6)
+
+
+# ------------------------------------------------- reciprocal-space encoding
+def _reci_problem(sizes, H, seed, a_lo=0.8, a_hi=4.0):
+    b = make_sized_batch(sizes, seed)
+    edges = tp.get_edge_index(b.sizes)
+    g = torch.Generator().manual_seed(seed + 50)
+    a = -(torch.rand(b.pos.shape[0], H, generator=g) * (a_hi - a_lo) + a_lo)
+    rec, vcell = tp.reciprocal_vectors(b.trans_vec)
+    rpos = tp.relative_positions(b.pos, edges)
+    e_start = tp.edge_row_offsets(edges, b.pos.shape[0])
+    return b, edges, a, rec, vcell, rpos, e_start, g
+
+
+@pytest.mark.parametrize("sizes,H,R", [([1, 3, 5, 2], 4, 2), ([7, 1, 70, 12], 8, 2), ([4, 9], 2, 1), ([3, 130], 16, 3),
+                                       ([5, 6], 3, 0)])
+def test_reci_enc_fwd_bwd_against_oracle(dev, sizes, H, R):
+    """Forward (z, S) and backward (ga) of the reciprocal-space kernels against the C restatement
+    of the reference's kernels (double accumulation): rows longer than a wavefront, head counts
+    that need padding, ranges 0..3.  z to 2e-5 absolute: the float phases reach tens of radians,
+    so the sum itself carries ~1e-6 relative of its largest term."""
+    b, edges, a, rec, vcell, rpos, e_start, g = _reci_problem(sizes, H, seed=H + R)
+    kr = ops.kr_base(rpos.to(dev), rec.to(dev), b.batch.to(dev), edges.to(dev))
+    kr_ref = tp.kr_base(b.pos, b.batch, b.trans_vec, edges)
+    assert float((kr.cpu() - kr_ref).abs().max()) < 1e-5
+    z_ref, se_ref = ks.reci_enc_fwd(a, kr_ref, rec, vcell, b.batch, edges, R)
+    z, se = ops.reci_enc_fwd(a.to(dev), kr, rec.to(dev), vcell.to(dev), b.batch.to(dev), e_start.to(dev), R)
+    assert_close(se, se_ref, "S", rtol=5e-6)
+    assert float((z.cpu() - z_ref).abs().max()) < 2e-5
+    gz = torch.randn(edges.shape[1], H, generator=g)
+    ga_ref = ks.reci_enc_bwd(a, kr_ref, rec, b.batch, e_start, gz, se_ref, R)
+    ga = ops.reci_enc_bwd(a.to(dev), kr, rec.to(dev), b.batch.to(dev), e_start.to(dev), gz.to(dev), se, R)
+    assert_close(ga, ga_ref, "ga", rtol=1e-5)
+
+
+def test_reci_enc_clamp_and_function(dev):
+    """Sums below 1e-6 (wide Gaussians): z takes log(1e-6) and the edge drops out of ga; the
+    autograd Function returns the same z and ga and no other gradient."""
+    from crystalformer_amd.hip_funcs import KernelManager, ReciPeriodicEncodingFuncCUDA
+    b, edges, a, rec, vcell, rpos, e_start, g = _reci_problem([3, 4], 2, seed=9, a_lo=1e-4, a_hi=2e-3)
+    kr_ref = tp.kr_base(b.pos, b.batch, b.trans_vec, edges)
+    z_ref, se_ref = ks.reci_enc_fwd(a, kr_ref, rec, vcell, b.batch, edges, 2)
+    assert bool((se_ref < 1e-6).any()) and bool((se_ref > 1e-3).any())
+    old = KernelManager.LATTICE_RANGE
+    KernelManager.LATTICE_RANGE = 2
+    try:
+        ad = a.to(dev).requires_grad_()
+        z = ReciPeriodicEncodingFuncCUDA.apply(ad, kr_ref.to(dev), rec.to(dev), vcell.to(dev), b.batch.to(dev),
+                                               edges.to(dev))
+        gz = torch.randn(z.shape, generator=g)
+        (z * gz.to(dev)).sum().backward()
+    finally:
+        KernelManager.LATTICE_RANGE = old
+    solid = (se_ref - 1e-6).abs() > 1e-4                 # away from the switch itself
+    assert float((z.detach().cpu() - z_ref)[solid].abs().max()) < 1e-4
+    ga_ref = ks.reci_enc_bwd(a, kr_ref, rec, b.batch, e_start, gz, se_ref, 2)
+    assert_close(ad.grad, ga_ref, "ga", rtol=2e-4)
