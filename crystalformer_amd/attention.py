@@ -24,7 +24,7 @@ from . import ops
 from . import hip_funcs
 from .hip_funcs import linear as linear_hip
 from .hip_funcs import (FusedDotProductAttentionCUDA, GaussianExponentsHIP, RealPeriodicEncodingFuncCUDA,
-                        RealPeriodicEncodingWithProjFuncCUDA)
+                        RealPeriodicEncodingWithProjFuncCUDA, ReciPeriodicEncodingFuncCUDA)
 from .params import LatticeformerParams
 
 ATOM_NUM = 98
@@ -47,10 +47,10 @@ def make_positive_func(spec: str):
     raise NotImplementedError(f"Unknown positive_func: {spec}")
 
 
-def gaussian_exponents(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, gauss_scale: Tensor,
-                       params: LatticeformerParams, training: bool) -> Tensor:
-    """a[i,h] = -rho(normalised alpha) / (2 r0^2), alpha from the un-scaled
-    per-head query (models/indexed_lattice_multi_head_attention_cuda.py:636-722)."""
+def normalised_alpha(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, gauss_scale: Tensor,
+                     params: LatticeformerParams, training: bool) -> Tensor:
+    """alpha[i,h] from the un-scaled per-head query, normalised by the stored or the batch
+    statistics (models/indexed_lattice_multi_head_attention_cuda.py:636-673)."""
     n, h, d = q.shape
     # (per-head dot products; written as a product + sum rather than the reference's
     # batch of N*H 1xd @ dx1 matmuls, which is two orders of magnitude slower on hipBLASLt)
@@ -71,6 +71,14 @@ def gaussian_exponents(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, ga
         if training:   # written once, by the first training step
             with torch.no_grad():
                 gauss_scale.copy_(torch.stack([scale, shift]))
+    return alpha
+
+
+def gaussian_exponents(q: Tensor, query: Tensor, lattice_pos_weights: Tensor, gauss_scale: Tensor,
+                       params: LatticeformerParams, training: bool) -> Tensor:
+    """a[i,h] = -rho(normalised alpha) / (2 r0^2)
+    (models/indexed_lattice_multi_head_attention_cuda.py:636-722, real domain)."""
+    alpha = normalised_alpha(q, query, lattice_pos_weights, gauss_scale, params, training)
     rho = make_positive_func(params.positive_func)(alpha, params.gauss_lb_real)
     return rho * (-0.5 * params.scale_real ** -2)
 
@@ -139,9 +147,9 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                  params: LatticeformerParams = LatticeformerParams(), device=None, dtype=None) -> None:
         kw = {"device": device, "dtype": dtype}
         super().__init__()
-        if params.domain not in ("real", "no"):
-            raise NotImplementedError(
-                f"domain={params.domain!r}: only the real-space encoding has HIP kernels")
+        assert params.domain in ("real", "reci", "RECI", "multihead", "no")
+        if params.domain == "multihead":
+            assert num_heads % 2 == 0, "multihead: each domain takes half of the heads"
         self.embed_dim = embed_dim
         self.kdim = kdim * num_heads if kdim is not None and kdim > 0 else embed_dim
         self.vdim = vdim * num_heads if vdim is not None and vdim > 0 else embed_dim
@@ -175,10 +183,15 @@ class CrystalformerMultiheadAttentionCUDA(Module):
         cond = 1 if params.value_pe_condproj == "no" else ATOM_NUM
         self.pe_dist_proj = None
         self.pe_wave_proj = None
-        if params.domain == "real" and params.value_pe_dist_real > 0:
-            self.pe_dist_proj = Parameter(torch.empty(cond, heads, self.head_dim, params.value_pe_dist_real, **kw))
-        if params.domain == "real" and params.value_pe_wave_real > 0:
-            raise NotImplementedError("value_pe_wave_real > 0 has no HIP kernel")
+        # (models/indexed_lattice_multi_head_attention_cuda.py:869-878: the reciprocal-space blocks own a
+        # projection too when value_pe_dist_reci > 0, although their kernel path yields no value encoding)
+        bins = params.value_pe_dist_real if params.domain in ("real", "multihead") else \
+            (params.value_pe_dist_reci if params.domain in ("reci", "RECI") else 0)
+        if bins > 0:
+            self.pe_dist_proj = Parameter(torch.empty(cond, heads, self.head_dim, bins, **kw))
+        if (params.domain in ("real", "multihead") and params.value_pe_wave_real > 0) or \
+                (params.domain in ("reci", "RECI") and params.value_pe_wave_reci > 0):
+            raise NotImplementedError("value_pe_wave_* > 0 has no HIP kernel")
         self._reset_parameters()
 
     def _reset_parameters(self):
@@ -250,6 +263,9 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             v = linear_hip(value, self.v_proj_weight, b_v).contiguous().view(value.shape[0], H, vd // H)
 
         bias = values = qs = None
+        if P.domain in ("reci", "RECI", "multihead"):
+            bias, values, qs = self._reciprocal_domains(q, query, batch_q, edges, points, dist2_min, tvecs,
+                                                        kr_base, rvecs, vcell, onehot)
         if P.domain == "real":
             proj = self.pe_dist_proj
             if proj is not None and P.value_pe_condproj != "no":
@@ -302,6 +318,72 @@ class CrystalformerMultiheadAttentionCUDA(Module):
         if need_weights:
             raise NotImplementedError("need_weights=True: attention weights are not returned by the fused path")
         return attn, values
+
+
+    def _real_encoding(self, a: Tensor, proj: Optional[Tensor], heads: int, batch_q, edges, points, dist2_min,
+                       tvecs, rvecs, onehot):
+        """Real-space bias and value encoding for ``heads`` heads with exponents ``a``
+        (models/indexed_lattice_multi_head_attention_cuda.py:393-421, 694-723)."""
+        P = self.params
+        if proj is not None and P.value_pe_condproj != "no":
+            proj = conditional_projection(proj, onehot, edges, P.value_pe_condproj)
+        dist_max = P.value_pe_dist_max
+        if dist_max < 0:
+            dist_max = (-dist_max) * P.scale_real
+        adaptive = ()
+        if P.adaptive_cutoff_sigma != 0:
+            rvlen = rvecs if rvecs.dim() == 2 else torch.norm(rvecs, 2, dim=-1)
+            cutoff = P.adaptive_cutoff_sigma if P.adaptive_cutoff_sigma < 0 else \
+                P.scale_real * P.gauss_lb_real ** (-0.5) * P.adaptive_cutoff_sigma
+            adaptive = (rvlen, cutoff)
+        if proj is not None and proj.shape[1] == 1 and heads > 1:
+            proj = proj.expand(proj.shape[0], heads, proj.shape[2], proj.shape[3])
+        enc = RealPeriodicEncodingWithProjFuncCUDA if P.use_low_memory else RealPeriodicEncodingFuncCUDA
+        out = enc.apply(a.contiguous(), points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real, dist_max,
+                        P.value_pe_width_scale, proj, *adaptive)
+        return out[0], (out[1] if len(out) >= 2 else None)
+
+    def _reciprocal_domains(self, q, query, batch_q, edges, points, dist2_min, tvecs, kr_base, rvecs, vcell,
+                            onehot):
+        """Bias (and value encoding) of the blocks that involve the reciprocal-space lattice sum
+        (models/indexed_lattice_multi_head_attention_cuda.py:724-746)."""
+        P = self.params
+        H = self.num_heads
+        if kr_base is None or rvecs is None or rvecs.dim() != 3 or vcell is None:
+            raise ValueError("reciprocal-space blocks need kr_base (E,3), rvecs (B,3,3) and vcell (B)")
+        coef_real, coef_reci = -0.5 * P.scale_real ** -2, -0.5 * P.scale_reci ** 2
+        qs = None
+        spec = fused_exponents_spec(P) if q.is_cuda else None
+        if spec is not None and (P.domain == "reci" or
+                                 (P.domain == "multihead" and P.gauss_lb_real == P.gauss_lb_reci)):
+            # rho(normalised alpha) and the scaled query from the fused kernel (two launches);
+            # the domains differ in the factor applied to rho only
+            rho, qs = GaussianExponentsHIP.apply(
+                q, self.lattice_pos_weights, self.gauss_scale, P.normalize_gauss, self.training, spec[0], spec[1],
+                P.gauss_lb_reci, 1.0, 1.0 / math.sqrt(q.shape[-1]))
+            if P.domain == "reci":
+                return ReciPeriodicEncodingFuncCUDA.apply(rho * coef_reci, kr_base, rvecs, vcell, batch_q,
+                                                          edges), None, qs
+            a1, a2 = rho[:, :H // 2] * coef_real, rho[:, H // 2:] * coef_reci
+        else:
+            func = make_positive_func(P.positive_func)
+            alpha = normalised_alpha(q, query, self.lattice_pos_weights, self.gauss_scale, P, self.training)
+            if P.domain == "reci":
+                a = func(alpha, P.gauss_lb_reci) * coef_reci
+                return ReciPeriodicEncodingFuncCUDA.apply(a, kr_base, rvecs, vcell, batch_q, edges), None, qs
+            if P.domain == "RECI":
+                a = 1 / func(alpha, P.gauss_lb_reci) * coef_reci
+                return ReciPeriodicEncodingFuncCUDA.apply(a, kr_base, rvecs, vcell, batch_q, edges), None, qs
+            a1, a2 = alpha.chunk(2, 1)
+            a1 = func(a1, P.gauss_lb_real) * coef_real
+            a2 = func(a2, P.gauss_lb_reci) * coef_reci
+        # multihead: first half of the heads in real space, second half in reciprocal space
+        proj = self.pe_dist_proj[:, :H // 2] if self.pe_dist_proj is not None else None
+        w1, v1 = self._real_encoding(a1, proj, H // 2, batch_q, edges, points, dist2_min, tvecs, rvecs, onehot)
+        w2 = ReciPeriodicEncodingFuncCUDA.apply(a2.contiguous(), kr_base, rvecs, vcell, batch_q, edges)
+        bias = torch.cat([w1, w2], dim=1)
+        values = None if v1 is None else torch.cat([v1, torch.zeros_like(v1)], dim=1)
+        return bias, values, qs
 
 
 CrystalformerMultiheadAttentionHIP = CrystalformerMultiheadAttentionCUDA

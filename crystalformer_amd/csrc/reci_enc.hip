@@ -25,6 +25,7 @@ struct ReciArgs {
     const float *gz, *sumexp_in;
     int64_t N, E;
     int H, R;
+    int norm_grad;             // backward: include d/da of 1.5 log(-4 pi a)
     float *z, *sumexp, *ga;
 };
 
@@ -129,7 +130,9 @@ __global__ __launch_bounds__(WAVE) void reci_enc_kernel(ReciArgs p)
             for (int h = 0; h < HP; h++) {
                 if (on && h < H) {
                     const float se = p.sumexp_in[e * H + h];
-                    part[h] += acc[h] * p.gz[e * H + h] * (se < 1e-6f ? 0.f : 1.0f / se);
+                    const float g = p.gz[e * H + h];
+                    part[h] += acc[h] * g * (se < 1e-6f ? 0.f : 1.0f / se);
+                    if (p.norm_grad) part[h] += g * (1.5f / p.a[i * H + h]);
                 }
             }
         }
@@ -219,7 +222,7 @@ extern "C" int cf_reci_enc_fwd(const float *a_ik, const float *kr_base_e, const 
 extern "C" int cf_reci_enc_bwd(const float *a_ik, const float *kr_base_e, const float *rvecs_n,
                                const int64_t *batch_i, const int64_t *e_start_i, const float *gz_ek,
                                const float *sumexp_ek, int64_t N, int64_t H, int64_t E, int lattice_range,
-                               float *ga_ik, void *stream)
+                               int normalisation_grad, float *ga_ik, void *stream)
 {
     int rc = reci_check("cf_reci_enc_bwd", N, H, E, lattice_range);
     if (rc) return rc;
@@ -229,7 +232,7 @@ extern "C" int cf_reci_enc_bwd(const float *a_ik, const float *kr_base_e, const 
     ReciArgs p{};
     p.a = a_ik; p.kr = kr_base_e; p.rvecs = rvecs_n; p.batch = batch_i; p.e_start = e_start_i;
     p.gz = gz_ek; p.sumexp_in = sumexp_ek;
-    p.N = N; p.E = E; p.H = (int)H; p.R = lattice_range; p.ga = ga_ik;
+    p.N = N; p.E = E; p.H = (int)H; p.R = lattice_range; p.norm_grad = normalisation_grad; p.ga = ga_ik;
     rc = launch_reci<true>(p, (hipStream_t)stream, "cf_reci_enc_bwd");
     if (rc) return rc;
     CF_CHECK_LAUNCH("cf_reci_enc_bwd");

@@ -47,15 +47,14 @@ def compute_lattice_distances_for_cuda(pos: Tensor, batch: Tensor, trans_vec: Te
     """Geometry prologue of the kernel path
     (models/indexed_latticeformer_encoder.py:183-253): relative positions per
     edge, reciprocal vectors, cell volume and the dense edge list.  Returns
-    ``(pos_ij, dist2_min, kr_base, recip_vec, vcell, edges)``; ``dist2_min`` and
-    ``kr_base`` are None (the kernels find the minimum themselves; there is no
-    reciprocal-space kernel here)."""
-    if output_reci:
-        raise NotImplementedError("reciprocal-space outputs are not served by the HIP path")
+    ``(pos_ij, dist2_min, kr_base, recip_vec, vcell, edges)``; ``dist2_min`` is None (the
+    kernels find the minimum themselves), ``kr_base`` (E,3) the reciprocal-space phases when
+    ``output_reci``."""
     sizes = _sizes_on_device(sizes, batch, trans_vec.shape[0], pos.device)
     vcell, recip_vec, _ = ops.lattice_geometry(trans_vec)
     edges, pos_ij = ops.edge_index(sizes, pos.contiguous())
-    return pos_ij, None, None, recip_vec, vcell, edges
+    kr_base = ops.kr_base(pos_ij, recip_vec, batch - batch[0], edges) if output_reci else None
+    return pos_ij, None, kr_base, recip_vec, vcell, edges
 
 
 def _activation(name):
@@ -74,7 +73,7 @@ class CrystalformerEncoderLayerCUDA(Module):
                  norm_first: bool = False, no_layer_norm=False, params=LatticeformerParams(),
                  k_dim=0, v_dim=0, device=None, dtype=None) -> None:
         super().__init__()
-        assert params.domain in ("real",), "only the real-space domain is served"
+        assert params.domain in ("real", "reci", "RECI", "multihead")
         self.domain = params.domain
         self.self_attn = CrystalformerMultiheadAttentionCUDA(d_model, nhead, dropout=dropout, kdim=k_dim,
                                                              vdim=v_dim, params=params)
@@ -108,7 +107,10 @@ class CrystalformerEncoderLayerCUDA(Module):
     def forward(self, src: Tensor, batch: Tensor, edges: Tensor, pos_ij: Tensor = None,
                 dist2_min: Tensor = None, trans: Tensor = None, kr_base: Tensor = None,
                 rvecs: Tensor = None, vcell: Tensor = None, onehot: Tensor = None) -> Tensor:
-        assert pos_ij is not None and trans is not None
+        if self.domain in ("real", "multihead"):
+            assert pos_ij is not None and trans is not None
+        if self.domain in ("reci", "multihead", "RECI"):
+            assert kr_base is not None and rvecs is not None and rvecs.dim() == 3 and vcell is not None
         x = src
         if self._fused_tail(x):
             # inference without norm layers: residuals, bias and ReLU ride in the epilogues of
@@ -205,12 +207,17 @@ class CrystalformerEncoderCUDA(Module):
             sizes = _sizes_on_device(sizes, batch, trans.shape[0], pos.device)
         layout = ops.batch_layout(sizes, batch)       # index structure: built once per batch
         batch, edges = layout.batch, layout.edges
-        vcell, _, rvlen = ops.lattice_geometry(trans)
+        vcell, recip, rvlen = ops.lattice_geometry(trans)
         pos_ij = ops.relative_positions(layout, pos)
         dist2_min = kr_base = None
+        rvecs = rvlen                                  # real-space blocks only need the lengths
+        if any(layer.domain != "real" for layer in self.layers):
+            # reciprocal-space blocks: the vectors themselves and the phases <b_d, p_j - p_i>
+            rvecs = recip
+            kr_base = ops.kr_base(pos_ij, recip, batch, edges)
         output = src
         for layer in self.layers:
-            output = layer(output, batch, edges, pos_ij, dist2_min, trans, kr_base, rvlen, vcell, onehot)
+            output = layer(output, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot)
         if self.norm is not None:
             output = self.norm(output)
         return output

@@ -63,6 +63,10 @@ class KernelManager:
     # the encoding evaluates both directions of an atom pair together; set False
     # for arbitrary edge lists (per-edge kernels; attention backward unavailable).
     DENSE_EDGE_BLOCKS: bool = True
+    # The reference's reciprocal-space backward kernel differentiates log(sum) only and drops
+    # d/da of the normalisation term 1.5 log(-4 pi a) (models/kernels/reci_enc_bwd.cu:41-69),
+    # unlike autograd on its PyTorch path.  False reproduces the kernel, True the full derivative.
+    RECI_NORMALISATION_GRAD: bool = False
     compiled: bool = False
 
 
@@ -249,7 +253,7 @@ class ReciPeriodicEncodingFuncCUDA(torch.autograd.Function):
     def backward(ctx, gz_ek):
         a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, sumexp_ek = ctx.saved_tensors
         ga_ik = ops.reci_enc_bwd(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, gz_ek.detach().contiguous(),
-                                 sumexp_ek, ctx.lattice_range)
+                                 sumexp_ek, ctx.lattice_range, KernelManager.RECI_NORMALISATION_GRAD)
         return ga_ik, None, None, None, None, None
 
 

@@ -53,7 +53,7 @@ SIGNATURES = {
                                       _f32, _ptr, _i64, _ptr, _ptr, _ptr]),
     "cf_kr_base": (_int, [_ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
     "cf_reci_enc_fwd": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _ptr, _ptr, _ptr]),
-    "cf_reci_enc_bwd": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _ptr, _ptr]),
+    "cf_reci_enc_bwd": (_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _int, _ptr, _ptr]),
     "cf_adamw_step_workspace": (_i64, [_int, _ptr]),
     "cf_adamw_step": (_int, [_int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _f32, _f32, _f32, _f32, _f32, _f32, _ptr,
                              _ptr, _i64, _ptr]),

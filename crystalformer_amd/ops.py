@@ -616,9 +616,10 @@ def reci_enc_fwd(a_ik: Tensor, kr_base_e: Tensor, rvecs_n: Tensor, vcell_n: Tens
 
 
 def reci_enc_bwd(a_ik: Tensor, kr_base_e: Tensor, rvecs_n: Tensor, batch_i: Tensor, e_start_i: Tensor,
-                 gz_ek: Tensor, sumexp_ek: Tensor, lattice_range: int) -> Tensor:
-    """``ga_ik`` of the reciprocal-space lattice sum (the reference's definition, which leaves
-    the normalisation term's derivative out)."""
+                 gz_ek: Tensor, sumexp_ek: Tensor, lattice_range: int, normalisation_grad: bool = False) -> Tensor:
+    """``ga_ik`` of the reciprocal-space lattice sum: by default the reference kernel's
+    definition, which leaves the normalisation term's derivative out; with
+    ``normalisation_grad`` the full derivative of z."""
     dev = require_device(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, gz_ek, sumexp_ek)
     a_ik, kr_base_e, rvecs_n, batch_i, e_start_i = _reci_operands(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i)
     gz_ek, sumexp_ek = _f32(gz_ek, "gz_ek"), _f32(sumexp_ek, "sumexp_ek")
@@ -629,7 +630,8 @@ def reci_enc_bwd(a_ik: Tensor, kr_base_e: Tensor, rvecs_n: Tensor, batch_i: Tens
     ga = torch.empty((N, H), dtype=torch.float32, device=dev)
     with device_guard(dev):
         rc = _lib.load().cf_reci_enc_bwd(ptr(a_ik), ptr(kr_base_e), ptr(rvecs_n), ptr(batch_i), ptr(e_start_i),
-                                         ptr(gz_ek), ptr(sumexp_ek), N, H, E, int(lattice_range), ptr(ga),
+                                         ptr(gz_ek), ptr(sumexp_ek), N, H, E, int(lattice_range),
+                                         int(bool(normalisation_grad)), ptr(ga),
                                          stream_handle(dev))
     check(rc, "cf_reci_enc_bwd")
     return ga

@@ -323,8 +323,10 @@ int cf_linear_weight_grad(const float *g, const float *x, int64_t N, int64_t C, 
  *   S[e,h] = sum over n1 in [0,R] (weight 2 for n1 != 0), n2, n3 in [-R,R] of
  *            exp(a[i,h] |n1 b1 + n2 b2 + n3 b3|^2) cos(<kr_base[e], n>),  b_d = rows of rvecs_n[batch[i]]
  *   z[e,h] = log(max(S, 1e-6)) + 1.5 log(-4 pi a[i,h]) - log(vcell_n[batch[i]]),  sumexp[e,h] = S
- *   ga[i,h] = sum over the edges e of row i of gz[e,h] / S[e,h] * dS/da (0 where S < 1e-6); like the
- *            reference's kernel, without the derivative of the 1.5 log(-4 pi a) term.
+ *   ga[i,h] = sum over the edges e of row i of gz[e,h] / S[e,h] * dS/da (0 where S < 1e-6); with
+ *            normalisation_grad == 0 as the reference's kernel, which leaves out the derivative
+ *            of the 1.5 log(-4 pi a) term; != 0 adds it (1.5 / a[i,h] * sum_e gz[e,h]), which is
+ *            what autograd gives on the reference's PyTorch path.
  * Edges are addressed through their row offsets e_start_i (N+1) (edges sorted by source atom, as
  * the reference's backward assumes, reci_space_enc.py:66-68); kr_base_e (E,3) are the phases
  * <b_d, p_j - p_i> (models/indexed_latticeformer_encoder.py:245-251), which cf_kr_base computes.
@@ -337,7 +339,7 @@ int cf_reci_enc_fwd(const float *a_ik, const float *kr_base_e, const float *rvec
                     int lattice_range, float *z_ek, float *sumexp_ek, void *stream);
 int cf_reci_enc_bwd(const float *a_ik, const float *kr_base_e, const float *rvecs_n, const int64_t *batch_i,
                     const int64_t *e_start_i, const float *gz_ek, const float *sumexp_ek, int64_t N, int64_t H,
-                    int64_t E, int lattice_range, float *ga_ik, void *stream);
+                    int64_t E, int lattice_range, int normalisation_grad, float *ga_ik, void *stream);
 
 /*
  * cf_linear_weight_grad for n_layers linear layers at once (2 * ceil(n_layers / 16)

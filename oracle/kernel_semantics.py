@@ -177,12 +177,15 @@ def reci_enc_fwd(a_ik, kr_base_e, rvecs_n, vcell_n, batch_i, edge_ij_e, lattice_
     return z, se
 
 
-def reci_enc_bwd(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, gz_ek, sumexp_ek, lattice_range=2) -> Tensor:
-    """ga_ik (models/kernels/reci_enc_bwd.cu; without the normalisation term's derivative)."""
+def reci_enc_bwd(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, gz_ek, sumexp_ek, lattice_range=2,
+                 normalisation_grad=False) -> Tensor:
+    """ga_ik (models/kernels/reci_enc_bwd.cu: without the normalisation term's derivative unless
+    ``normalisation_grad``)."""
     a_ik, kr_base_e, rvecs_n, gz_ek, sumexp_ek = _f(a_ik), _f(kr_base_e), _f(rvecs_n), _f(gz_ek), _f(sumexp_ek)
     batch_i, e_start_i = _l(batch_i), _l(e_start_i)
     N, H = a_ik.shape
     ga = torch.empty((N, H), dtype=torch.float32)
     lib().ref_reci_enc_bwd(_p(a_ik), _p(kr_base_e), _p(rvecs_n), _p(batch_i), _p(e_start_i), _p(gz_ek),
-                           _p(sumexp_ek), _i64(N), _i64(H), _int(lattice_range), _p(ga))
+                           _p(sumexp_ek), _i64(N), _i64(H), _int(lattice_range), _int(int(normalisation_grad)),
+                           _p(ga))
     return ga

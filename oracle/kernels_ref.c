@@ -413,10 +413,11 @@ void ref_reci_enc_fwd(const float *a_ik, const float *kr_base_e, const float *rv
 
 /* ga[i,h] = sum over the edges of row i of gz[e,h] / S[e,h] * sum_n |k_n|^2 exp(a |k_n|^2) cos(.)
  * (zero where S < 1e-6).  As in the reference's kernel, the derivative of the normalisation
- * term 1.5 log(-4 pi a) is NOT part of the result. */
+ * term 1.5 log(-4 pi a) is NOT part of the result unless normalisation_grad is set (then it is
+ * the derivative of z that autograd gives on the reference's PyTorch path). */
 void ref_reci_enc_bwd(const float *a_ik, const float *kr_base_e, const float *rvecs_n, const i64 *batch_i,
                       const i64 *e_start_i, const float *gz_ek, const float *sumexp_ek, i64 N, i64 H,
-                      int lattice_range, float *ga_ik)
+                      int lattice_range, int normalisation_grad, float *ga_ik)
 {
     const int R = lattice_range;
     for (i64 i = 0; i < N; i++) {
@@ -443,6 +444,7 @@ void ref_reci_enc_bwd(const float *a_ik, const float *kr_base_e, const float *rv
                 }
                 const float se = sumexp_ek[e * H + h];
                 total += s * (double)gz_ek[e * H + h] * (se < 1e-6f ? 0.0 : 1.0 / (double)se);
+                if (normalisation_grad) total += (double)gz_ek[e * H + h] * 1.5 / (double)a;
             }
             ga_ik[i * H + h] = (float)total;
         }

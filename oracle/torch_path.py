@@ -197,15 +197,36 @@ def positive_elu(x: Tensor, lower_bound: float, beta: float) -> Tensor:
     return (1.0 - lower_bound) * F.elu(x * (beta / (1.0 - lower_bound))) + 1.0
 
 
-def gaussian_exponents(q: Tensor, lattice_pos_weights: Tensor, gauss_scale: Tensor,
-                       training: bool, normalize: bool, lower_bound: float,
-                       beta: float, scale_real: float) -> Tensor:
-    """a[i,h] = -rho(normalised q_h . w_h) / (2 r0^2)   (negative).
+def normalised_alpha(q: Tensor, lattice_pos_weights: Tensor, gauss_scale: Tensor,
+                     training: bool, normalize: bool) -> Tensor:
+    """alpha[i,h] = q_h . w_h, shifted and scaled by the stored or the batch statistics.
 
     q is the *unscaled* query (N,H,D).  When ``gauss_scale[0]`` is not
     positive the normalisation uses the statistics of this very batch
     (unbiased std over all N*H entries), and in training mode stores them
-    once.  Follows models/indexed_lattice_multi_head_attention.py:1300-1357.
+    once.  Follows models/indexed_lattice_multi_head_attention.py:1300-1330.
+    """
+    n, h, d = q.shape
+    alpha = (q.reshape(n, h, 1, d) @ lattice_pos_weights.reshape(h, d, 1)).view(n, h)
+    if normalize:
+        if bool(gauss_scale[0] > 0):
+            scale, shift = gauss_scale[0], gauss_scale[1]
+        else:
+            scale = torch.reciprocal(alpha.detach().std())
+            shift = -alpha.detach().mean()
+            if training:
+                with torch.no_grad():
+                    gauss_scale[0] = scale
+                    gauss_scale[1] = shift
+        alpha = (alpha + shift) * scale
+    return alpha
+
+
+def gaussian_exponents(q: Tensor, lattice_pos_weights: Tensor, gauss_scale: Tensor,
+                       training: bool, normalize: bool, lower_bound: float,
+                       beta: float, scale_real: float) -> Tensor:
+    """a[i,h] = -rho(normalised q_h . w_h) / (2 r0^2)   (negative).
+    Follows models/indexed_lattice_multi_head_attention.py:1300-1357.
     """
     n, h, d = q.shape
     alpha = (q.reshape(n, h, 1, d) @ lattice_pos_weights.reshape(h, d, 1)).view(n, h)

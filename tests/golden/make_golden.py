@@ -117,6 +117,14 @@ def main():
     run_case(ref_root, "k0_r2", small_cfg(value_pe_dist_real=0, lattice_range=2), batch, 12, out)
     torch.save(out, os.path.join(HERE, "reference_small_model.pt"))
 
+    # reciprocal-space blocks: alternating real / reciprocal layers, and half-and-half heads
+    out = {"batch": out["batch"]}
+    run_case(ref_root, "real_reci_k16_r1", small_cfg(domain="real-reci"), batch, 13, out)
+    run_case(ref_root, "multihead_k0_r2", small_cfg(domain="multihead", value_pe_dist_real=0, lattice_range=2),
+             batch, 14, out)
+    run_case(ref_root, "reci_r2", small_cfg(domain="reci", value_pe_dist_real=0, lattice_range=2), batch, 15, out)
+    torch.save(out, os.path.join(HERE, "reference_small_model_reciprocal.pt"))
+
     # full-size default model: digests of the seeded initial parameters only
     cfg = SimpleNamespace(**dict(DEFAULT_MODEL_PARAMS, use_cuda_code=False))
     model = reference_model(ref_root, cfg, 123)

@@ -770,6 +770,10 @@ def test_reci_enc_fwd_bwd_against_oracle(dev, sizes, H, R):
     ga_ref = ks.reci_enc_bwd(a, kr_ref, rec, b.batch, e_start, gz, se_ref, R)
     ga = ops.reci_enc_bwd(a.to(dev), kr, rec.to(dev), b.batch.to(dev), e_start.to(dev), gz.to(dev), se, R)
     assert_close(ga, ga_ref, "ga", rtol=1e-5)
+    full_ref = ks.reci_enc_bwd(a, kr_ref, rec, b.batch, e_start, gz, se_ref, R, normalisation_grad=True)
+    full = ops.reci_enc_bwd(a.to(dev), kr, rec.to(dev), b.batch.to(dev), e_start.to(dev), gz.to(dev), se, R,
+                            normalisation_grad=True)
+    assert_close(full, full_ref, "ga with the normalisation term", rtol=1e-5)
 
 
 def test_reci_enc_clamp_and_function(dev):

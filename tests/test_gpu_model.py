@@ -367,3 +367,79 @@ def test_forward_from_plain_structures_and_checkpoint(dev, tmp_path):
     with torch.no_grad():
         y = model(b.to(dev))
     assert_close(y, y_ref, "de-normalised output")
+
+
+# ------------------------------------------------- reciprocal-space blocks
+RECI_CASES = [("real_reci_k16_r1", dict(domain="real-reci")),
+              ("multihead_k0_r2", dict(domain="multihead", value_pe_dist_real=0, lattice_range=2)),
+              ("reci_r2", dict(domain="reci", value_pe_dist_real=0, lattice_range=2))]
+
+
+@pytest.fixture(scope="module")
+def gold_reci():
+    return torch.load(os.path.join(GOLD, "reference_small_model_reciprocal.pt"), weights_only=True)
+
+
+@pytest.mark.parametrize("name,over", RECI_CASES)
+def test_reciprocal_blocks_match_reference_golden(dev, gold_reci, name, over):
+    """Models with reciprocal-space blocks (alternating with real-space ones, half of the heads,
+    all blocks) against the reference's own outputs and gradients.  The reference's PyTorch
+    path, which wrote the vectors, differentiates the normalisation term 1.5 log(-4 pi a) as
+    well, so the gradient check runs with that term switched on; the default (the reference
+    kernel's backward, without it) is covered at operator level against the C oracle."""
+    gold = gold_reci
+    cfg = small_cfg(adaptive_cutoff_sigma=0.0, **over)
+    model = Latticeformer(cfg)
+    model.load_state_dict(gold[f"{name}.state"])
+    model.to(dev).eval()
+    data = ns_to(dev, SimpleNamespace(**gold["batch"]))
+    outs = {}
+    for li, layer in enumerate(model.encoder.layers):
+        layer.register_forward_hook(lambda m, i, o, li=li: outs.__setitem__(li, o))
+    with torch.no_grad():
+        y = model(data)
+    assert_close(y, gold[f"{name}.eval.y"], "y")
+    for li in range(cfg.num_layers):
+        assert_close(outs[li], gold[f"{name}.eval.layer{li}.out"], f"layer {li} output")
+    model.train()
+    old = hip_funcs.KernelManager.RECI_NORMALISATION_GRAD
+    hip_funcs.KernelManager.RECI_NORMALISATION_GRAD = True
+    try:
+        y = model(data)
+        loss = torch.nn.functional.l1_loss(y.squeeze(-1), data.y)
+        loss.backward()
+    finally:
+        hip_funcs.KernelManager.RECI_NORMALISATION_GRAD = old
+    assert abs(float(loss.detach()) - float(gold[f"{name}.train.loss"])) < 1e-6
+    params = dict(model.named_parameters())
+    for k, g in gold[f"{name}.train.grads"].items():
+        assert_close(params[k].grad, g, f"grad {k}", rtol=3e-5)
+    model.eval()
+    with torch.no_grad():
+        assert_close(model(data), gold[f"{name}.eval2.y"], "second eval")
+
+
+def test_multihead_blocks_with_value_encoding_follow_the_kernel_path(dev):
+    """Half-and-half blocks with Gaussian value bins: as on the reference's kernel path
+    (models/indexed_lattice_multi_head_attention_cuda.py:731-746) the real-space half carries a
+    value encoding and the reciprocal half zeros; checked against the CPU oracle restating that."""
+    cfg = default_params(num_layers=2, domain="multihead", value_pe_dist_real=16, adaptive_cutoff_sigma=0.0,
+                         lattice_range=2)
+    torch.manual_seed(2)
+    model = Latticeformer(cfg)
+    b = make_config_batch("cfg1_simplified_b32")
+    P = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    cap = {}
+    with torch.no_grad():
+        y_ref = om.latticeformer_forward(P, cfg, b, capture=cap, multihead_values=True)
+    model.to(dev).eval()
+    values = {}
+    for li, layer in enumerate(model.encoder.layers):
+        layer.self_attn.register_forward_hook(lambda m, i, o, li=li: values.__setitem__(li, o[1]))
+    with torch.no_grad():
+        y = model(b.to(dev))
+    H = cfg.head_num
+    for li in range(cfg.num_layers):
+        assert_close(values[li], cap[f"layer{li}.values"], f"layer {li} values")
+        assert float(values[li][:, H // 2:].abs().max()) == 0.0
+    assert_close(y, y_ref, "model output")

@@ -113,6 +113,8 @@ def test_backward_is_the_gradient_of_log_sum_only():
     z_full = torch.log(full_cube_sum(b, edges, ad2, 2)) + (1.5 * torch.log(-4 * math.pi * ad2))[edges[0]]
     (z_full * gz.double()).sum().backward()
     assert rel_err(full.float(), ad2.grad.float()) < 1e-6
+    ga_full = ks.reci_enc_bwd(a, kr, rec, b.batch, e_start, gz, se, 2, normalisation_grad=True)
+    assert rel_err(ga_full, ad2.grad.float()) < 5e-6
 
 
 def test_kr_base_is_the_phase_per_reciprocal_vector():
