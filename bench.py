@@ -57,6 +57,23 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
     elapsed = time.perf_counter() - t0
     ops.set_event_log(None)
     eager = {"value": round(B * args.steps / elapsed, 2), "ms_per_step": round(elapsed / args.steps * 1e3, 4)}
+    # Kernel durations: the encoding / attention launches of one step are re-issued back to back
+    # (queue kept full), each bracketed by a pair of HIP events on the launch stream.
+    calls = {"real_enc_fwd": [], "real_enc_bwd": [], "fused_dpa_fwd": [], "fused_dpa_bwd": []}
+    originals = {name: getattr(ops, name) for name in calls}
+    for name in calls:
+        setattr(ops, name, (lambda nm: lambda *a, **kw: (calls[nm].append((a, kw)), originals[nm](*a, **kw))[1])(name))
+    training_step(model, data, opt, sch)
+    for name in calls:
+        setattr(ops, name, originals[name])
+    log = []
+    ops.set_event_log(log)
+    for name in calls:
+        for _ in range(max(args.steps // 4, 5)):
+            for a, kw in calls[name]:
+                originals[name](*a, **kw)
+    torch.cuda.synchronize()
+    ops.set_event_log(None)
     submission = "eager launches"
     if not args.no_graph:
         # the same step (device-side schedule, capturable AdamW) as one HIP graph replay
@@ -79,13 +96,19 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
     # backward work per eval: the forward's accumulation twice (S and Q) + geometry and weights
     flop_bwd = evals * (23 + 4 * H + 2 + 2 * K + 4 * H * K) + float(E) * H * 3 * 2 * D * K
     bwd_ms = avg("real_enc_bwd")
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(f"{args.config}:{args.rule}:bwd")
     roofline = {
         "kernel": "real_enc_bwd_pair_kernel + reductions (periodic encoding backward)",
         "bound": "mfma", "achieved": round(flop_bwd / (bwd_ms * 1e-3) / 1e12, 3) if bwd_ms > 0 else 0.0,
         "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
         "frac": round(flop_bwd / (bwd_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4) if bwd_ms > 0 else 0.0,
-        "traffic": None, "avg_launch_ms": bwd_ms,
-        "note": "event pairs recorded in the eager training loop (include launch gaps)",
+        "traffic": traffic, "avg_launch_ms": bwd_ms,
+        "note": "HIP event pairs around cf_real_enc_bwd (pair kernel + its two fixed-order reductions), the "
+                "step's four launches re-issued back to back",
         "real_enc_fwd_avg_ms": avg("real_enc_fwd"), "fused_dpa_fwd_avg_ms": avg("fused_dpa_fwd"),
         "fused_dpa_bwd_avg_ms": avg("fused_dpa_bwd"),
     }
@@ -151,7 +174,8 @@ def main() -> int:
                     help="time full training steps (forward + backward + AdamW) instead of forwards")
     ap.add_argument("--profile-kernel", action="store_true",
                     help="counter-collection helper: launch only a 256 MiB device copy (calibration) and the "
-                         "periodic-encoding kernel on the workload, 5 times each, and exit")
+                         "periodic-encoding kernel on the workload (with --train: its backward), 5 times each, "
+                         "and exit")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -190,7 +214,7 @@ def main() -> int:
 
     from crystalformer_amd.graphs import GraphedForward
 
-    if args.train:
+    if args.train and not args.profile_kernel:
         return train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N, E, H, K)
 
     def timed(step_fn, steps, warmup):
@@ -208,15 +232,21 @@ def main() -> int:
         src = torch.ones(64 << 20, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
         captured = {}
-        orig = ops.real_enc_fwd
+        which = "real_enc_bwd" if args.train else "real_enc_fwd"       # --train: the backward kernel
+        orig = getattr(ops, which)
 
         def spy(*a, **kw):
             captured.setdefault("args", (a, kw))
             return orig(*a, **kw)
-        ops.real_enc_fwd = spy
-        with torch.no_grad():
-            model(data)
-        ops.real_enc_fwd = orig
+        setattr(ops, which, spy)
+        if args.train:
+            model.train()
+            out = model(data)
+            torch.nn.functional.l1_loss(out[:, 0], data.y).backward()
+        else:
+            with torch.no_grad():
+                model(data)
+        setattr(ops, which, orig)
         a, kw = captured["args"]
         for _ in range(5):
             dst.copy_(src)
