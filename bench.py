@@ -61,8 +61,16 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
     # (queue kept full), each bracketed by a pair of HIP events on the launch stream.
     calls = {"real_enc_fwd": [], "real_enc_bwd": [], "fused_dpa_fwd": [], "fused_dpa_bwd": []}
     originals = {name: getattr(ops, name) for name in calls}
+    def detached(v):       # no autograd graph may outlive the step through the recorded arguments
+        return v.detach() if torch.is_tensor(v) else v
+
+    def spy_on(nm):
+        def spy(*a, **kw):
+            calls[nm].append((tuple(detached(v) for v in a), {k: detached(v) for k, v in kw.items()}))
+            return originals[nm](*a, **kw)
+        return spy
     for name in calls:
-        setattr(ops, name, (lambda nm: lambda *a, **kw: (calls[nm].append((a, kw)), originals[nm](*a, **kw))[1])(name))
+        setattr(ops, name, spy_on(name))
     training_step(model, data, opt, sch)
     for name in calls:
         setattr(ops, name, originals[name])
@@ -74,6 +82,7 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
                 originals[name](*a, **kw)
     torch.cuda.synchronize()
     ops.set_event_log(None)
+    calls.clear()
     submission = "eager launches"
     if not args.no_graph:
         # the same step (device-side schedule, capturable AdamW) as one HIP graph replay

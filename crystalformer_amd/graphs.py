@@ -69,6 +69,11 @@ class GraphedTrainStep:
     step counter that lives in the graph, so no host value is baked into it.
     ``batch`` fixes the layout; later calls may pass other positions, lattices,
     species and targets with identical ``sizes``.
+
+    Tensors that still hold the autograd graph of an earlier eager step of ``model`` (a
+    loss, an output, a non-detached view of a parameter) must be dropped first: their
+    gradient-accumulation nodes are bound to the stream of that step, and a backward pass
+    under capture that has to synchronise with it aborts the capture.
     """
 
     def __init__(self, model: torch.nn.Module, batch: CrystalBatch, lr: float = 5e-4, sch_decay: float = 4000.0,
