@@ -145,6 +145,20 @@ __device__ __forceinline__ int wave_max_i(int v)
     return __builtin_amdgcn_readlane(v, 63);
 }
 
+// Inclusive prefix sum over the 64 lanes (Hillis-Steele inside each row of 16 lanes on
+// row shifts, then the row totals carried across with the two broadcasts), 6 instructions.
+constexpr int DPP_ROW_SHR1 = 0x111, DPP_ROW_SHR2 = 0x112, DPP_ROW_SHR4 = 0x114, DPP_ROW_SHR8 = 0x118;
+__device__ __forceinline__ int wave_inclusive_scan_i(int v)
+{
+    v += dpp_i<DPP_ROW_SHR1, 0xF>(0, v);
+    v += dpp_i<DPP_ROW_SHR2, 0xF>(0, v);
+    v += dpp_i<DPP_ROW_SHR4, 0xF>(0, v);
+    v += dpp_i<DPP_ROW_SHR8, 0xF>(0, v);
+    v += dpp_i<DPP_ROW_BCAST15, 0xA>(0, v);
+    v += dpp_i<DPP_ROW_BCAST31, 0xC>(0, v);
+    return v;
+}
+
 // Orders this wave's earlier LDS/global writes before its later reads.
 __device__ __forceinline__ void wave_mem_sync()
 {
