@@ -43,13 +43,19 @@ constexpr int PROJ_INDEXED = 2;          // W per edge or per atom: read from gl
 
 
 // LDS per work-group: per wave three ring arrays of RING_SLOTS words (d^2, distance
-// argument, flag bits); for PROJ_SHARED also WPB x 16 staged columns of 16*NT+1 floats
-// and WPB x 2 edge ids.
+// argument, flag bits); for PROJ_SHARED also the exchange buffer of 4 NT planes of 552 floats
+// (layout at its declaration), WPB x 2 edge ids and WPB x 16 reciprocal column totals.
 template <int NT, bool UNIFORM, int PROJ, int DT>
 __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
 {
     extern __shared__ __align__(16) float lds[];
-    constexpr int SROW = 16 * NT + 1;     // floats per staged column, odd stride
+    // Exchange buffer of the shared-projection epilogue: element (bin = 16 m + 4 q + r, unit, column
+    // = 8 dir + head) lives at (4 m + r) * SPLANE + dir * SDIR + unit * SUNIT + 8 q + head.  A writer
+    // (one unit, lanes over q, dir, head) and a reader (one head, lanes over q, dir, unit) then both
+    // spread over all 32 banks, two lanes per bank (dir), the least 64 lanes can do; a plain
+    // [column][bin] array costs four lanes per bank on both sides, and the LDS port is shared by
+    // the 16 wavefronts of a CU.
+    constexpr int SUNIT = 33, SDIR = 288, SPLANE = 552;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform by construction
     const int q = lane >> 4;
@@ -64,8 +70,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
     float *ring_d2 = lds + wave * (3 * RING_SLOTS);
     float *ring_s = ring_d2 + RING_SLOTS;
     int *ring_bits = reinterpret_cast<int *>(ring_s + RING_SLOTS);
-    float *Sbuf = lds + WPB * 3 * RING_SLOTS;                        // [WPB][16][SROW]
-    int64_t *meta = reinterpret_cast<int64_t *>(Sbuf + WPB * 16 * SROW);   // [WPB][2]
+    float *Sbuf = lds + WPB * 3 * RING_SLOTS;                        // [4 NT][SPLANE]
+    int64_t *meta = reinterpret_cast<int64_t *>(Sbuf + 4 * NT * SPLANE);   // [WPB][2]
     float *invbuf = reinterpret_cast<float *>(meta + WPB * 2);             // [WPB][16]
 
     // Gaussian argument of bin 16m + c at distance 0
@@ -426,11 +432,11 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         } else if (PROJ == PROJ_SHARED) {
             // park the column sums (inactive columns hold zeros: their weights are masked) and the
             // reciprocal of the column totals, then project per head
-            float *col = Sbuf + (wave * 16 + c) * SROW;
+            float *col = Sbuf + (c >> 3) * SDIR + wave * SUNIT + 8 * q + (c & 7);
 #pragma unroll
             for (int m = 0; m < NT; m++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) col[16 * m + 4 * q + r] = acc[m][r];
+                for (int r = 0; r < 4; r++) col[(4 * m + r) * SPLANE] = acc[m][r];
             if (q == 0) invbuf[wave * 16 + c] = inv;
             if (lane == 0) {
                 meta[2 * wave + 0] = unit_on ? e_ij : -1;
@@ -441,7 +447,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 // this wave: head hw; column j of the product = direction j/8 of unit j%8
                 const int hw = hg * 8 + wave;
                 const int j = c, unit_j = j & 7, dir_j = j >> 3;
-                const float *src = Sbuf + (unit_j * 16 + dir_j * 8 + wave) * SROW;
+                const float *src = Sbuf + dir_j * SDIR + unit_j * SUNIT + 8 * q + wave;
                 float4_t out[DT];
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++) out[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -449,7 +455,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 for (int t4 = 0; t4 < NT; t4++) {
                     float sb[4];
 #pragma unroll
-                    for (int r = 0; r < 4; r++) sb[r] = src[16 * t4 + 4 * q + r];
+                    for (int r = 0; r < 4; r++) sb[r] = src[(4 * t4 + r) * SPLANE];
 #pragma unroll
                     for (int r = 0; r < 4; r++)
 #pragma unroll
@@ -606,7 +612,7 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     const int DT = (mode == PROJ_SHARED && D > 16) ? 2 : 1;
     size_t lds = sizeof(float) * (size_t)WPB * 3 * RING_SLOTS;
     if (mode == PROJ_SHARED)
-        lds += sizeof(float) * (size_t)WPB * 16 * (16 * NT + 1) + sizeof(int64_t) * WPB * 2 + sizeof(float) * WPB * 16 + 8;
+        lds += sizeof(float) * (size_t)4 * NT * 552 + sizeof(int64_t) * WPB * 2 + sizeof(float) * WPB * 16 + 8;
     const int64_t rounds = ((U + WPB - 1) / WPB) * p.head_groups;
     if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // round positions are 32-bit in the kernel
     int64_t blocks = rounds;
