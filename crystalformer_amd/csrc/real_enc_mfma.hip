@@ -43,19 +43,13 @@ constexpr int PROJ_INDEXED = 2;          // W per edge or per atom: read from gl
 
 
 // LDS per work-group: per wave three ring arrays of RING_SLOTS words (d^2, distance
-// argument, flag bits); for PROJ_SHARED also the exchange buffer of 4 NT planes of 552 floats
-// (layout at its declaration), WPB x 2 edge ids and WPB x 16 reciprocal column totals.
+// argument, flag bits); for PROJ_SHARED also the exchange buffer of 4 NT planes of XPLANE floats
+// (layout in real_enc_pair.h), WPB x 2 edge ids and WPB x 16 reciprocal column totals.
 template <int NT, bool UNIFORM, int PROJ, int DT>
 __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
 {
     extern __shared__ __align__(16) float lds[];
-    // Exchange buffer of the shared-projection epilogue: element (bin = 16 m + 4 q + r, unit, column
-    // = 8 dir + head) lives at (4 m + r) * SPLANE + dir * SDIR + unit * SUNIT + 8 q + head.  A writer
-    // (one unit, lanes over q, dir, head) and a reader (one head, lanes over q, dir, unit) then both
-    // spread over all 32 banks, two lanes per bank (dir), the least 64 lanes can do; a plain
-    // [column][bin] array costs four lanes per bank on both sides, and the LDS port is shared by
-    // the 16 wavefronts of a CU.
-    constexpr int SUNIT = 33, SDIR = 288, SPLANE = 552;
+    constexpr int SPLANE = XPLANE;      // exchange buffer of the shared-projection epilogue
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform by construction
     const int q = lane >> 4;
@@ -432,7 +426,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         } else if (PROJ == PROJ_SHARED) {
             // park the column sums (inactive columns hold zeros: their weights are masked) and the
             // reciprocal of the column totals, then project per head
-            float *col = Sbuf + (c >> 3) * SDIR + wave * SUNIT + 8 * q + (c & 7);
+            float *col = Sbuf + xch_base(q, c & 7, wave, c >> 3);
 #pragma unroll
             for (int m = 0; m < NT; m++)
 #pragma unroll
@@ -447,7 +441,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 // this wave: head hw; column j of the product = direction j/8 of unit j%8
                 const int hw = hg * 8 + wave;
                 const int j = c, unit_j = j & 7, dir_j = j >> 3;
-                const float *src = Sbuf + dir_j * SDIR + unit_j * SUNIT + 8 * q + wave;
+                const float *src = Sbuf + xch_base(q, wave, unit_j, dir_j);
                 float4_t out[DT];
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++) out[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -612,7 +606,7 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     const int DT = (mode == PROJ_SHARED && D > 16) ? 2 : 1;
     size_t lds = sizeof(float) * (size_t)WPB * 3 * RING_SLOTS;
     if (mode == PROJ_SHARED)
-        lds += sizeof(float) * (size_t)4 * NT * 552 + sizeof(int64_t) * WPB * 2 + sizeof(float) * WPB * 16 + 8;
+        lds += sizeof(float) * (size_t)4 * NT * XPLANE + sizeof(int64_t) * WPB * 2 + sizeof(float) * WPB * 16 + 8;
     const int64_t rounds = ((U + WPB - 1) / WPB) * p.head_groups;
     if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // round positions are 32-bit in the kernel
     int64_t blocks = rounds;

@@ -29,7 +29,6 @@ template <int NT, bool UNIFORM>
 __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 {
     extern __shared__ __align__(16) float lds[];
-    constexpr int SROW = 16 * NT + 1;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int q = lane >> 4;
@@ -46,8 +45,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     float *ring_d2 = lds + wave * (3 * BRING_SLOTS);
     float *ring_s = ring_d2 + BRING_SLOTS;
     int *ring_bits = reinterpret_cast<int *>(ring_s + BRING_SLOTS);
-    float *Sbuf = lds + WPB * 3 * BRING_SLOTS;                          // [8 heads][2 dirs][8 units][SROW]
-    float *PXbuf = Sbuf + WPB * 16 * SROW;                              // [8 units][16 cols]
+    float *Sbuf = lds + WPB * 3 * BRING_SLOTS;                          // exchange buffer, 4 NT planes (real_enc_pair.h)
+    float *PXbuf = Sbuf + 4 * NT * XPLANE;                              // [8 units][16 cols]
 
     float ck[NT];
 #pragma unroll
@@ -282,11 +281,10 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         px += __shfl_xor(px, 32, WAVE);
 
         // ---- exchange: column (dir, head) of unit `wave` -> row ((head*2 + dir)*8 + wave)
-        const int srow = ((c & 7) * 2 + (c >> 3)) * WPB + wave;
         if (q == 0) PXbuf[wave * 16 + c] = px;
         const int hw = hg * 8 + wave;
         const int jcol = c, unit_j = jcol & 7, dir_j = jcol >> 3;    // product column j = dir*8 + unit
-        const float *src = Sbuf + ((wave * 2 + dir_j) * WPB + unit_j) * SROW;
+        const float *src = Sbuf + xch_base(q, wave, unit_j, dir_j);
         float dotS = 0.f, dotQ = 0.f;
         // projection operands of this wave's head (W stays in cache across rounds)
         float Wa[4 * NT];
@@ -337,13 +335,13 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         for (int pass = 0; pass < 2; pass++) {
             // pass 0 exchanges S (also feeds gW), pass 1 exchanges Q
             {
-                float *col = Sbuf + srow * SROW;
+                float *col = Sbuf + xch_base(q, c & 7, wave, c >> 3);
 #pragma unroll
                 for (int m = 0; m < NT; m++)
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
                         // (inactive columns hold zeros: their weights are masked in the loop)
-                        col[16 * m + 4 * q + r] = pass == 0 ? accS[m][r] : accQ[m][r];
+                        col[(4 * m + r) * XPLANE] = pass == 0 ? accS[m][r] : accQ[m][r];
                     }
             }
             __syncthreads();
@@ -352,7 +350,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             for (int t4 = 0; t4 < NT; t4++) {
                 float sb[4];
 #pragma unroll
-                for (int r = 0; r < 4; r++) sb[r] = src[16 * t4 + 4 * q + r];
+                for (int r = 0; r < 4; r++) sb[r] = src[(4 * t4 + r) * XPLANE];
 #pragma unroll
                 for (int r = 0; r < 4; r++)
                     out = __builtin_amdgcn_mfma_f32_16x16x4f32(Wa[4 * t4 + r], sb[r], out, 0, 0, 0);
@@ -380,10 +378,11 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 for (int s4 = 0; s4 < 4; s4++) {
                     const int colk = 4 * s4 + q;                    // this lane's reduction index
                     const float av = gvk[s4];
-                    const float *srck = Sbuf + ((wave * 2 + (colk >> 3)) * WPB + (colk & 7)) * SROW;
+                    // bin 16 t + c of column colk: plane 4 t + c % 4, q index c / 4
+                    const float *srck = Sbuf + (c & 3) * XPLANE + xch_base(c >> 2, wave, colk & 7, colk >> 3);
 #pragma unroll
                     for (int t = 0; t < NT; t++)
-                        gWacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, srck[16 * t + c], gWacc[t], 0, 0, 0);
+                        gWacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, srck[4 * t * XPLANE], gWacc[t], 0, 0, 0);
                 }
 #pragma unroll
                 for (int t = 0; t < NT; t++) gw_slot[t * WAVE] = gWacc[t];
@@ -464,7 +463,7 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
     p.window = sqrtf(40.0f) / bin_step;
     const int NT = K <= 16 ? 1 : K <= 32 ? 2 : 4;
     const bool uniform = cutoff == 0.0f;
-    const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)WPB * 16 * (16 * NT + 1) + WPB * 16 +
+    const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)4 * NT * XPLANE + WPB * 16 +
                                         (size_t)WPB * NT * WAVE * 4) + 16;
     if (((U + WPB - 1) / WPB) * ((H + 7) / 8) >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // 32-bit round positions
     const int blocks = real_enc_bwd_pairs_blocks(U, H);

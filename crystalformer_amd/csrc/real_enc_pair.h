@@ -118,6 +118,21 @@ __device__ __forceinline__ int column_bits(const ColumnBoxes &cb, int n1, int n2
 constexpr int WPB = 8;                   // wavefronts per work-group = units per round
 constexpr int PAIR_FIELDS = 5;           // words per unit descriptor: e_ij, e_ji, i, j, crystal
 
+// Exchange buffer of the shared-projection epilogues (forward and backward): the column sums a
+// wavefront holds for its unit are parked in LDS and read back by the wavefront that owns a head.
+// Element (bin = 16 m + 4 q + r, unit, column = 8 dir + head) lives at
+//     (4 m + r) * XPLANE + dir * 256 + unit * 32 + ((8 q + head) ^ unit).
+// A writer (one unit; lanes over q, dir, head), a reader (one head; lanes over q, dir, unit) and
+// the reader of the weight-gradient update (one head; lanes over 16 consecutive bins and 4
+// consecutive columns) all spread over the 32 banks with two lanes per bank, the least 64
+// lanes can do; a plain [column][bin] array puts four lanes on a bank on both sides, and the LDS
+// port is shared by the 16 wavefronts of a CU.
+constexpr int XPLANE = 516;
+__device__ __forceinline__ int xch_base(int q, int head, int unit, int dir)
+{
+    return dir * 256 + unit * 32 + ((8 * q + head) ^ unit);
+}
+
 // Position of a round: head group and round index inside it.  32-bit; the launchers
 // refuse work with 2^30 rounds or more.  One head group (H <= 8) needs no division.
 struct RoundPos { int hg, r; };
