@@ -151,7 +151,10 @@ __global__ __launch_bounds__(256) void fused_dpa_fwd_stream_kernel(DpaArgs p, in
 
     float m = -1.0e30f, l = 0.f;
     float4_v acc = {0.f, 0.f, 0.f, 0.f};
-    auto step = [&](int64_t e, int64_t j) {
+    // Raw logits of the main loop are parked in prob[] and normalised by the closing sweep; those of
+    // the last (for most rows: the only) partial step stay in registers and are written once,
+    // normalised, so that a short row never reads its own stores back.
+    auto step = [&](int64_t e, int64_t j, bool park) -> float {
         const float4_v k4 = key4[j * HD4 + piece];
         float4_v v4 = val4[j * HD4 + piece];
         if (bij4) {
@@ -161,21 +164,25 @@ __global__ __launch_bounds__(256) void fused_dpa_fwd_stream_kernel(DpaArgs p, in
         float s = q4.x * k4.x + q4.y * k4.y + q4.z * k4.z + q4.w * k4.w;
         for (int off = DV4 >> 1; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
         if (p.aij) s += p.aij[e * H + h];
-        if (lead) p.prob[e * H + h] = s;
+        if (park && lead) p.prob[e * H + h] = s;
         const float m_new = fmaxf(m, s);
         const float sc = exp2_hw((m - m_new) * LOG2E);
         const float pe = exp2_hw((s - m_new) * LOG2E);
         l = l * sc + pe;
         acc = acc * sc + v4 * pe;
         m = m_new;
+        return s;
     };
     const int stride = DPA_WPQ * ES;
-    int64_t e = e0 + wave * ES + es;
+    // the main loop takes whole steps of 4 * stride edges (the same number in every lane), the
+    // rest of the row (fewer than 4 * stride edges) is the partial step
+    int64_t eb = e0;
+    int64_t e = eb + wave * ES + es;
     // key indices one step (4 edges per slot) ahead
     int64_t jn[4];
 #pragma unroll
     for (int u = 0; u < 4; u++) jn[u] = (e + u * stride < e1) ? dst[e + u * stride] : 0;
-    for (; e + 3 * stride < e1; e += 4 * stride) {
+    for (; eb + 4 * stride <= e1; eb += 4 * stride, e += 4 * stride) {
         int64_t jc[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) jc[u] = jn[u];
@@ -185,11 +192,16 @@ __global__ __launch_bounds__(256) void fused_dpa_fwd_stream_kernel(DpaArgs p, in
             jn[u] = (en < e1) ? dst[en] : 0;
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) step(e + u * stride, jc[u]);
+        for (int u = 0; u < 4; u++) step(e + u * stride, jc[u], true);
     }
+    const int64_t e_tail = e;                      // first edge of this lane's slot in the last step
+    const int64_t parked = (eb - e0) * H;          // logits parked by the main loop
+    float s_tail[4];
 #pragma unroll
-    for (int u = 0; u < 4; u++)
-        if (e + u * stride < e1) step(e + u * stride, jn[u]);
+    for (int u = 0; u < 4; u++) {
+        s_tail[u] = 0.f;
+        if (e_tail + u * stride < e1) s_tail[u] = step(e_tail + u * stride, jn[u], false);
+    }
     // merge the edge slots of this wavefront
     auto merge = [&](float mo, float lo, float4_v ao) {
         const float m_new = fmaxf(m, mo);
@@ -228,11 +240,17 @@ __global__ __launch_bounds__(256) void fused_dpa_fwd_stream_kernel(DpaArgs p, in
     }
     __syncthreads();
     // normalise the parked logits: element x of the row's (n,H) block belongs to head x % H
+    if (lead) {
+        const float mt = fin[0][h], it = fin[1][h];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (e_tail + u * stride < e1)
+                p.prob[(e_tail + u * stride) * H + h] = exp2_hw((s_tail[u] - mt) * LOG2E) * it;
+    }
     const int hx = threadIdx.x % H;
     const float mh = fin[0][hx], ih = fin[1][hx];
     float *row = p.prob + e0 * H;
-    const int64_t total = (e1 - e0) * H;
-    for (int64_t x = threadIdx.x; x < total; x += blockDim.x) row[x] = exp2_hw((row[x] - mh) * LOG2E) * ih;
+    for (int64_t x = threadIdx.x; x < parked; x += blockDim.x) row[x] = exp2_hw((row[x] - mh) * LOG2E) * ih;
 }
 
 // ------------------------------------------------- backward, streaming version
