@@ -150,81 +150,15 @@ __global__ __launch_bounds__(1024) void column_sum_kernel(const float *g, int64_
 }
 
 // Weight gradient of a linear layer, gW (C, K) = g^T x with g (N, C), x (N, K): a short, wide
-// product with a long reduction over the rows.  The rows are cut into slices; a work-group of
-// 4 wavefronts (2 x 2) computes the 32 x 32 block (c0.., k0..) of one slice, operands straight
-// from global memory (lane (q, c) reads g[n + q][c0 + c] and x[n + q][k0 + c], 4 rows per MFMA),
-// and writes it to part[slice]; a second kernel adds the slices in order.
-constexpr int WG_SLICE_STEPS = 8;      // MFMA steps (of 4 rows) whose loads are issued together
-
-__global__ __launch_bounds__(256) void weight_grad_slices_kernel(const float *g, const float *x, int64_t N,
-                                                                 int C, int K, int rows_per_slice, float *part,
-                                                                 float *part_b)
-{
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int q = lane >> 4, c = lane & 15;
-    const int c0 = blockIdx.x * 32 + 16 * (wave >> 1);
-    const int k0 = blockIdx.y * 32 + 16 * (wave & 1);
-    const int64_t n_begin = (int64_t)blockIdx.z * rows_per_slice;
-    const int64_t n_end = min(N, n_begin + rows_per_slice);
-    const int gc = min(c0 + c, C - 1), xk = min(k0 + c, K - 1);
-    float4_t acc = {0.f, 0.f, 0.f, 0.f};
-    float colsum = 0.f;                     // bias gradient: this lane's rows of column c0 + c
-    for (int64_t n0 = n_begin; n0 < n_end; n0 += 4 * WG_SLICE_STEPS) {
-        float a[WG_SLICE_STEPS], b[WG_SLICE_STEPS];
-#pragma unroll
-        for (int t = 0; t < WG_SLICE_STEPS; t++) {
-            const int64_t n = n0 + 4 * t + q;
-            const bool in = n < n_end;
-            a[t] = in ? g[n * C + gc] : 0.f;
-            b[t] = in ? x[n * K + xk] : 0.f;
-        }
-#pragma unroll
-        for (int t = 0; t < WG_SLICE_STEPS; t++) {
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t], b[t], acc, 0, 0, 0);
-            colsum += a[t];
-        }
-    }
-    if (part_b && blockIdx.y == 0 && (wave & 1) == 0) {
-        // rows n = 4 t + q: add the four row classes in ascending q
-        const float s = (colsum + __shfl_xor(colsum, 16, 64)) + (__shfl_xor(colsum, 32, 64) + __shfl_xor(colsum, 48, 64));
-        if (q == 0 && c0 + c < C) part_b[(int64_t)blockIdx.z * C + c0 + c] = s;
-    }
-    // lane (q, c) holds gW[c0 + 4 q + r][k0 + c]
-    float *dst = part + (int64_t)blockIdx.z * C * K;
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int cc = c0 + 4 * q + r, kk = k0 + c;
-        if (cc < C && kk < K) dst[(int64_t)cc * K + kk] = acc[r];
-    }
-}
-
-// out[x] = sum over slices of part[s][x]; with out_b, elements past `total` belong to a second
-// array of `total_b` elements per slice (the bias gradient) summed the same way.
-__global__ __launch_bounds__(256) void add_slices_kernel(const float *part, int slices, int64_t total, float *out,
-                                                         const float *part_b, int64_t total_b, float *out_b)
-{
-    int64_t x = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (x >= total) {
-        x -= total;
-        if (!out_b || x >= total_b) return;
-        part = part_b; total = total_b; out = out_b;
-    }
-    float a0 = 0.f, a1 = 0.f;
-    int s = 0;
-    for (; s + 1 < slices; s += 2) {
-        a0 += part[(int64_t)s * total + x];
-        a1 += part[(int64_t)(s + 1) * total + x];
-    }
-    if (s < slices) a0 += part[(int64_t)s * total + x];
-    out[x] = a0 + a1;
-}
+// product with a long reduction over the rows.  The rows are cut into slices whose partial
+// products are written out and added by a second kernel in a fixed order (no atomics).  The
+// slice kernel serves a group of layers at once (kernel further down); a single layer is a
+// group of one.
 
 // ---- grouped weight gradients -------------------------------------------------
 // The weight (and bias) gradients of several linear layers in two launches: the layers'
-// 32 x 32 output tiles are numbered consecutively and a work-group finds its layer by
-// scanning the group's tile prefix.  Per layer the arithmetic, slicing and summation order
-// are those of weight_grad_slices_kernel / add_slices_kernel, so results are identical.
+// 64 x 64 output tiles are numbered consecutively and a work-group finds its layer by
+// scanning the group's tile prefix.
 constexpr int WG_GROUP = 16;
 
 struct WeightGradGroup {
@@ -232,21 +166,33 @@ struct WeightGradGroup {
     float *gw[WG_GROUP], *gb[WG_GROUP];
     int64_t part_off[WG_GROUP];      // floats from the workspace start to this layer's slices
     int N[WG_GROUP], C[WG_GROUP], K[WG_GROUP], slices[WG_GROUP];
-    int tile0[WG_GROUP + 1];         // prefix over 32 x 32 tiles
+    int tile0[WG_GROUP + 1];         // prefix over 64 x 64 tiles
     int cell0[WG_GROUP + 1];         // prefix over 256-element blocks of C (K + 1) outputs
     int count;
     float *part;
 };
 
+constexpr int WGT = 64;            // output tile of a work-group: 64 x 64
+constexpr int WG_ROWS = 16;        // rows staged per step
+constexpr int WG_LD = WGT + 16;    // LDS row stride, 16 mod 32: the four rows of an operand read cover all banks twice
+
+// A work-group of 4 wavefronts (2 x 2, 32 x 32 outputs each) owns a 64 x 64 block of one
+// layer's gW for one slice of rows.  16 rows of g (64 columns) and of x (64 columns) are staged
+// in LDS per step with 16-byte global loads (one per thread and matrix) and read back as MFMA
+// operands: lane (q, c) takes g[row 4 s + q][column c] and x[row 4 s + q][column c], four rows
+// per v_mfma_f32_16x16x4_f32.  The bias gradient (column sums of g) comes from the operands of
+// the wavefronts in the first block column.
 __global__ __launch_bounds__(256) void weight_grad_group_slices_kernel(WeightGradGroup a)
 {
+    __shared__ __align__(16) float gs[WG_ROWS * WG_LD];
+    __shared__ __align__(16) float xs[WG_ROWS * WG_LD];
     int t = 0;
     while (t + 1 < a.count && a.tile0[t + 1] <= (int)blockIdx.x) t++;
     if ((int)blockIdx.y >= a.slices[t]) return;
     const int tile = blockIdx.x - a.tile0[t];
     const int C = a.C[t], K = a.K[t];
     const int64_t N = a.N[t];
-    const int tiles_k = (K + 31) / 32;
+    const int tiles_k = (K + WGT - 1) / WGT;
     const int tc = tile / tiles_k, tk = tile - tc * tiles_k;
     const int slices = a.slices[t];
     int rows = (int)(((N + slices - 1) / slices + 3) / 4 * 4);
@@ -258,38 +204,79 @@ __global__ __launch_bounds__(256) void weight_grad_group_slices_kernel(WeightGra
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int q = lane >> 4, c = lane & 15;
-    const int c0 = tc * 32 + 16 * (wave >> 1);
-    const int k0 = tk * 32 + 16 * (wave & 1);
+    const int wr = wave >> 1, wc = wave & 1;
+    const int c0 = tc * WGT, k0 = tk * WGT;
     const int64_t n_begin = (int64_t)blockIdx.y * rows;
     const int64_t n_end = min(N, n_begin + rows);
-    const int gc = min(c0 + c, C - 1), xk = min(k0 + c, K - 1);
-    float4_t acc = {0.f, 0.f, 0.f, 0.f};
-    float colsum = 0.f;
-    for (int64_t n0 = n_begin; n0 < n_end; n0 += 4 * WG_SLICE_STEPS) {
-        float av[WG_SLICE_STEPS], bv[WG_SLICE_STEPS];
+    // staging role: thread -> row t / 16, four columns from 4 (t % 16)
+    const int srow = threadIdx.x >> 4, scol = (threadIdx.x & 15) * 4;
+    const bool vec_g = (C & 3) == 0 && c0 + scol + 3 < C, vec_x = (K & 3) == 0 && k0 + scol + 3 < K;
+
+    float4_t acc[2][2];
 #pragma unroll
-        for (int u = 0; u < WG_SLICE_STEPS; u++) {
-            const int64_t n = n0 + 4 * u + q;
-            const bool in = n < n_end;
-            av[u] = in ? g[n * C + gc] : 0.f;
-            bv[u] = in ? x[n * K + xk] : 0.f;
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float colsum[2] = {0.f, 0.f};
+    auto fetch = [&](const float *src, int64_t n, int ld, int col0, int width, bool vec) -> float4_t {
+        float4_t v = {0.f, 0.f, 0.f, 0.f};
+        if (n < n_end) {
+            if (vec) {
+                v = *reinterpret_cast<const float4_t *>(src + n * ld + col0);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (col0 + r < width) v[r] = src[n * ld + col0 + r];
+            }
         }
+        return v;
+    };
+    float4_t gn = fetch(g, n_begin + srow, C, c0 + scol, C, vec_g);
+    float4_t xn = fetch(x, n_begin + srow, K, k0 + scol, K, vec_x);
+    for (int64_t n0 = n_begin; n0 < n_end; n0 += WG_ROWS) {
+        __syncthreads();                               // the previous step's operands have been read
+        *reinterpret_cast<float4_t *>(gs + srow * WG_LD + scol) = gn;
+        *reinterpret_cast<float4_t *>(xs + srow * WG_LD + scol) = xn;
+        __syncthreads();
+        gn = fetch(g, n0 + WG_ROWS + srow, C, c0 + scol, C, vec_g);
+        xn = fetch(x, n0 + WG_ROWS + srow, K, k0 + scol, K, vec_x);
 #pragma unroll
-        for (int u = 0; u < WG_SLICE_STEPS; u++) {
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u], acc, 0, 0, 0);
-            colsum += av[u];
+        for (int s4 = 0; s4 < WG_ROWS / 4; s4++) {
+            float av[2], bv[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) av[i] = gs[(4 * s4 + q) * WG_LD + 32 * wr + 16 * i + c];
+#pragma unroll
+            for (int j = 0; j < 2; j++) bv[j] = xs[(4 * s4 + q) * WG_LD + 32 * wc + 16 * j + c];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                colsum[i] += av[i];
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+            }
         }
     }
-    if (part_b && tk == 0 && (wave & 1) == 0) {
-        const float s = (colsum + __shfl_xor(colsum, 16, 64)) + (__shfl_xor(colsum, 32, 64) + __shfl_xor(colsum, 48, 64));
-        if (q == 0 && c0 + c < C) part_b[(int64_t)blockIdx.y * C + c0 + c] = s;
+    if (part_b && tk == 0 && wc == 0) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            // rows n = 4 s + q: add the four row classes in ascending q
+            const float s = (colsum[i] + __shfl_xor(colsum[i], 16, 64)) +
+                            (__shfl_xor(colsum[i], 32, 64) + __shfl_xor(colsum[i], 48, 64));
+            const int cc = c0 + 32 * wr + 16 * i + c;
+            if (q == 0 && cc < C) part_b[(int64_t)blockIdx.y * C + cc] = s;
+        }
     }
+    // lane (q, c) holds gW[c0 + 32 wr + 16 i + 4 q + r][k0 + 32 wc + 16 j + c]
     float *dst = part + (int64_t)blockIdx.y * C * K;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int cc = c0 + 4 * q + r, kk = k0 + c;
-        if (cc < C && kk < K) dst[(int64_t)cc * K + kk] = acc[r];
-    }
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int cc = c0 + 32 * wr + 16 * i + 4 * q + r, kk = k0 + 32 * wc + 16 * j + c;
+                if (cc < C && kk < K) dst[(int64_t)cc * K + kk] = acc[i][j][r];
+            }
 }
 
 __global__ __launch_bounds__(256) void weight_grad_group_add_kernel(WeightGradGroup a)
@@ -376,30 +363,16 @@ extern "C" int64_t cf_linear_weight_grad_workspace(int64_t N, int64_t C, int64_t
     return (int64_t)weight_grad_slices(N) * C * (K + 1) * (int64_t)sizeof(float);
 }
 
+extern "C" int cf_linear_weight_grad_grouped(int n_layers, const float *const *g, const float *const *x,
+                                             const int64_t *N, const int64_t *C, const int64_t *K,
+                                             float *const *gW, float *const *gb, void *workspace,
+                                             int64_t workspace_bytes, void *stream);
+
 extern "C" int cf_linear_weight_grad(const float *g, const float *x, int64_t N, int64_t C, int64_t K,
                                      void *workspace, int64_t workspace_bytes, float *gW, float *gb, void *stream)
 {
-    CF_REQUIRE(N >= 0 && C >= 1 && K >= 1 && C < (1 << 20) && K < (1 << 20), CF_ERR_INVALID_ARGUMENT,
-               "cf_linear_weight_grad: bad sizes");
-    CF_REQUIRE(gW && (N == 0 || (g && x)), CF_ERR_INVALID_ARGUMENT, "cf_linear_weight_grad: null pointer");
-    const int slices = weight_grad_slices(N);
-    CF_REQUIRE(workspace && workspace_bytes >= cf_linear_weight_grad_workspace(N, C, K), CF_ERR_INVALID_ARGUMENT,
-               "cf_linear_weight_grad: workspace of %lld bytes needed",
-               (long long)cf_linear_weight_grad_workspace(N, C, K));
-    hipStream_t st = (hipStream_t)stream;
-    const int rows = (int)(((N + slices - 1) / slices + 3) / 4 * 4);
-    dim3 grid((unsigned)((C + 31) / 32), (unsigned)((K + 31) / 32), (unsigned)slices);
-    CF_REQUIRE(grid.y < 65536, CF_ERR_UNSUPPORTED, "cf_linear_weight_grad: too wide");
-    const int64_t total = C * K;
-    float *part_b = gb ? (float *)workspace + (int64_t)slices * total : nullptr;
-    weight_grad_slices_kernel<<<grid, 256, 0, st>>>(g, x, N, (int)C, (int)K, rows < 4 ? 4 : rows,
-                                                    (float *)workspace, part_b);
-    CF_CHECK_LAUNCH("cf_linear_weight_grad: slices");
-    const int64_t cells = total + (gb ? C : 0);
-    add_slices_kernel<<<(int)((cells + 255) / 256), 256, 0, st>>>((const float *)workspace, slices, total, gW,
-                                                                  part_b, C, gb);
-    CF_CHECK_LAUNCH("cf_linear_weight_grad: sum");
-    return CF_OK;
+    // a group of one layer: same kernels, same slicing, same summation order
+    return cf_linear_weight_grad_grouped(1, &g, &x, &N, &C, &K, &gW, &gb, workspace, workspace_bytes, stream);
 }
 
 extern "C" int64_t cf_linear_weight_grad_grouped_workspace(int n_layers, const int64_t *N, const int64_t *C,
@@ -457,7 +430,7 @@ extern "C" int cf_linear_weight_grad_grouped(int n_layers, const float *const *g
             a.cell0[k] = (int)cells;
             if (live) {
                 off += cf_linear_weight_grad_workspace(N[t], C[t], K[t]) / (int64_t)sizeof(float);
-                tiles += ((C[t] + 31) / 32) * ((K[t] + 31) / 32);
+                tiles += ((C[t] + WGT - 1) / WGT) * ((K[t] + WGT - 1) / WGT);
                 cells += (C[t] * (K[t] + 1) + 255) / 256;
                 if (a.slices[k] > max_slices) max_slices = a.slices[k];
                 CF_REQUIRE(tiles < (1ll << 30) && cells < (1ll << 30), CF_ERR_UNSUPPORTED,
