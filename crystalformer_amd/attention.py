@@ -254,8 +254,13 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                                       self.in_proj_bias)
             q, k, v = q.view(n, H, kd // H), k.view(n, H, kd // H), v.view(n, H, vd // H)
         elif fused_train:
-            q, k, v = hip_funcs.FusedLinearHIP.apply(query, self.in_proj_bias, None, False, self.q_proj_weight,
-                                                     self.k_proj_weight, self.v_proj_weight)
+            # a residual that is the input itself rides through the projection node (see its docstring)
+            carry = residual is query and query.is_contiguous()
+            out = hip_funcs.FusedLinearHIP.apply(query, self.in_proj_bias, None, False, carry, self.q_proj_weight,
+                                                 self.k_proj_weight, self.v_proj_weight)
+            q, k, v = out[:3]
+            if carry:
+                residual = out[3]
             q, k, v = q.view(n, H, kd // H), k.view(n, H, kd // H), v.view(n, H, vd // H)
         else:
             q = linear_hip(query, self.q_proj_weight, b_q).contiguous().view(n, H, kd // H)
@@ -310,7 +315,8 @@ class CrystalformerMultiheadAttentionCUDA(Module):
         if fused_linear:
             attn, = ops.linear_rows(attn, (self.out_proj.weight,), self.out_proj.bias, residual=residual)
         elif fused_train and ops.linear_rows_supported(attn, self.out_proj.weight):
-            attn, = hip_funcs.FusedLinearHIP.apply(attn, self.out_proj.bias, residual, False, self.out_proj.weight)
+            attn, = hip_funcs.FusedLinearHIP.apply(attn, self.out_proj.bias, residual, False, False,
+                                                   self.out_proj.weight)
         else:
             attn = linear_hip(attn, self.out_proj.weight, self.out_proj.bias)
             if residual is not None:

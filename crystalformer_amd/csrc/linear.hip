@@ -122,6 +122,122 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(LinArgs p)
     }
 }
 
+// Input gradient of linear layers: Y (N, K) = mask(sum_i G_i W_i) + A with G_i (N, C), W_i (C, K)
+// row-major, up to three terms sharing the shapes (the query / key / value projections feed one
+// input), A an optional addend (the gradient arriving on a residual branch) and mask an optional
+// (N, K) tensor whose non-positive entries zero the product (the ReLU in front of the layer).
+// Same tiling as linear_rows_kernel (64 x 64 per work-group, 2 x 2 wavefronts), 64-wide chunks
+// of the reduction staged in LDS; here the reduction runs over the rows of W, so its tile is
+// staged as [reduction][column] and read four bytes at a time as the B operand.
+constexpr int NN_T = 64;
+constexpr int NN_KC = 64;          // reduction chunk: long enough for the next chunk's loads to land meanwhile
+constexpr int NN_GLD = NN_KC + 4;  // G tile row stride (floats): 16-byte aligned, staggers the banks
+constexpr int NN_WLD = NN_T + 4;   // 4 rows apart = 16 banks apart: the four rows of a B read cover all banks twice
+
+struct LinNNArgs {
+    const float *g[3];
+    const float *w[3];
+    const float *add, *mask;
+    float *y;
+    int64_t N;
+    int C, K, terms;
+};
+
+__global__ __launch_bounds__(256) void linear_rows_nn_kernel(LinNNArgs p)
+{
+    __shared__ __align__(16) float gs[NN_T * NN_GLD];
+    __shared__ __align__(16) float ws[NN_KC * NN_WLD];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int q = lane >> 4, c = lane & 15;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int64_t row0 = (int64_t)blockIdx.x * NN_T;
+    const int col0 = blockIdx.y * NN_T;
+    // staging role for both tiles (64 rows x 64 floats): thread -> row t / 16 (+16 u), piece t % 16
+    const int srow = threadIdx.x >> 4, spiece = threadIdx.x & 15;
+    int64_t grow[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) grow[u] = min(row0 + srow + 16 * u, p.N - 1) * p.C + 4 * spiece;
+    const int wcol = min(col0 + 4 * spiece, p.K - 4);            // K is a multiple of 4
+
+    float4_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const int chunks = p.C / NN_KC;                              // C is a multiple of 64
+    const int steps = p.terms * chunks;
+    // Two register sets, each fetched two chunks ahead: a work-group is alone on its CU for these
+    // shapes (one wavefront per SIMD), so nothing else hides the latency of the loads.
+    float4_t gr[2][4], wg[2][4];
+    auto fetch = [&](int step, float4_t *gdst, float4_t *wdst) {
+        if (step >= steps) return;
+        const int term = step / chunks, k0 = (step - term * chunks) * NN_KC;
+        const float *g = p.g[term] + k0, *w = p.w[term] + (int64_t)(k0 + srow) * p.K + wcol;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            gdst[u] = *reinterpret_cast<const float4_t *>(g + grow[u]);
+            wdst[u] = *reinterpret_cast<const float4_t *>(w + (int64_t)(16 * u) * p.K);
+        }
+    };
+    auto chunk = [&](int step, float4_t *gset, float4_t *wset) {
+        __syncthreads();                                         // previous chunk fully consumed
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            *reinterpret_cast<float4_t *>(gs + (srow + 16 * u) * NN_GLD + 4 * spiece) = gset[u];
+            *reinterpret_cast<float4_t *>(ws + (srow + 16 * u) * NN_WLD + 4 * spiece) = wset[u];
+        }
+        __syncthreads();
+        fetch(step + 2, gset, wset);                             // in flight during this and the next chunk
+        // all operands of the chunk first (one wait), then the 64 MFMAs: a wavefront is alone on
+        // its SIMD here, so a wait per read would be paid in full
+        float4_t a[NN_KC / 16][2];
+        float b[NN_KC / 16][4][2];
+#pragma unroll
+        for (int ss = 0; ss < NN_KC / 16; ss++) {
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                a[ss][i] = *reinterpret_cast<const float4_t *>(gs + ((wr * 2 + i) * 16 + c) * NN_GLD + 16 * ss + 4 * q);
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)   // step r reduces over the rows 16 ss + 4 q' + r of the W tile
+                    b[ss][r][j] = ws[(16 * ss + 4 * q + r) * NN_WLD + (wc * 2 + j) * 16 + c];
+        }
+#pragma unroll
+        for (int ss = 0; ss < NN_KC / 16; ss++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[ss][i][r], b[ss][r][j], acc[i][j], 0, 0, 0);
+    };
+    fetch(0, gr[0], wg[0]);
+    fetch(1, gr[1], wg[1]);
+    for (int step = 0; step < steps; step += 2) {
+        chunk(step, gr[0], wg[0]);
+        if (step + 1 < steps) chunk(step + 1, gr[1], wg[1]);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int col = col0 + (wc * 2 + j) * 16 + c;
+        if (col >= p.K) continue;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int64_t row = row0 + (wr * 2 + i) * 16 + 4 * q + r;
+                if (row >= p.N) continue;
+                float v = acc[i][j][r];
+                if (p.mask && !(p.mask[row * p.K + col] > 0.f)) v = 0.f;
+                if (p.add) v += p.add[row * p.K + col];
+                p.y[row * p.K + col] = v;
+            }
+    }
+}
+
 // Column sums of a row-major (N, C) matrix (the bias gradient of a linear layer): 16 columns x
 // 64 row groups per work-group of 1024 threads, each thread adds every 64th row into 4 running
 // sums, the 64 partial sums of a column are then added in order.  No atomics, no scratch.
@@ -343,6 +459,32 @@ extern "C" int cf_linear_rows(const float *x, int64_t N, int64_t K, const float 
     else
         linear_rows_kernel<64, 32, 4, 1><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
     CF_CHECK_LAUNCH("cf_linear_rows");
+    return CF_OK;
+}
+
+extern "C" int cf_linear_rows_nn(const float *g0, const float *g1, const float *g2, int n_terms, const float *w0,
+                                 const float *w1, const float *w2, int64_t N, int64_t C, int64_t K,
+                                 const float *add, const float *mask, float *y, void *stream)
+{
+    CF_REQUIRE(N >= 0 && C >= 1 && K >= 1 && n_terms >= 1 && n_terms <= 3 && C <= (1 << 20) && K <= (1 << 20),
+               CF_ERR_INVALID_ARGUMENT, "cf_linear_rows_nn: bad sizes N=%lld C=%lld K=%lld terms=%d", (long long)N,
+               (long long)C, (long long)K, n_terms);
+    if (N == 0) return CF_OK;
+    CF_REQUIRE(C % 64 == 0 && K % 4 == 0, CF_ERR_UNSUPPORTED,
+               "cf_linear_rows_nn: C must be a multiple of 64 and K of 4 (got %lld, %lld)", (long long)C,
+               (long long)K);
+    const float *g[3] = {g0, g1, g2}, *w[3] = {w0, w1, w2};
+    LinNNArgs p{};
+    for (int i = 0; i < n_terms; i++) {
+        CF_REQUIRE(g[i] && w[i], CF_ERR_INVALID_ARGUMENT, "cf_linear_rows_nn: null operand %d", i);
+        p.g[i] = g[i];
+        p.w[i] = w[i];
+    }
+    CF_REQUIRE(y, CF_ERR_INVALID_ARGUMENT, "cf_linear_rows_nn: null output");
+    p.add = add; p.mask = mask; p.y = y; p.N = N; p.C = (int)C; p.K = (int)K; p.terms = n_terms;
+    dim3 grid((unsigned)((N + NN_T - 1) / NN_T), (unsigned)((K + NN_T - 1) / NN_T));
+    linear_rows_nn_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(p);
+    CF_CHECK_LAUNCH("cf_linear_rows_nn");
     return CF_OK;
 }
 

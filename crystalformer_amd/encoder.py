@@ -129,12 +129,8 @@ class CrystalformerEncoderLayerCUDA(Module):
             # the same epilogues with autograd (graphed training step, no norm layers, no dropout)
             x = self.self_attn(x, x, x, batch, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell,
                                onehot, need_weights=False, residual=x)[0]
-            h, = hip_funcs.FusedLinearHIP.apply(x, self.linear1.bias, None, True, self.linear1.weight)
-            if self.linear2.weight.shape[1] <= 256:
-                x, = hip_funcs.FusedLinearHIP.apply(h, self.linear2.bias, x, False, self.linear2.weight)
-            else:
-                x = x + linear_hip(h, self.linear2.weight, self.linear2.bias)
-            return x
+            return hip_funcs.FusedFeedForwardHIP.apply(x, self.linear1.weight, self.linear1.bias,
+                                                       self.linear2.weight, self.linear2.bias)
         if self.norm_first:
             x = x + self._sa_block(self.norm1(x), batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot)
             x = x + self._ff_block(self.norm2(x))

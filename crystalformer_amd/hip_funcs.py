@@ -325,44 +325,109 @@ class LinearRowsHIP(torch.autograd.Function):
         return gx, gw, gb
 
 
+def input_gradient(gs, weights, add: Optional[Tensor], mask: Optional[Tensor], like: Tensor) -> Tensor:
+    """``mask(sum_i gs[i] @ weights[i]) + add``.  One row-block launch where that replaces
+    several (more than one term, or a mask); a single plain product is left to the library
+    GEMM, which is faster at these sizes (measured at 1774 rows: 5.7 us against 6.8 us for
+    128 -> 128, 8.9 + 4.8 us against 17 us for 512 -> 128 with an addend)."""
+    if not gs:
+        return add if add is not None else torch.zeros_like(like)
+    if (len(gs) > 1 or mask is not None) and ops.linear_rows_nn_supported(gs[0], weights[0]):
+        return ops.linear_rows_nn(gs, weights, add=add.contiguous() if add is not None else None, mask=mask)
+    gx = torch.mm(gs[0], weights[0])
+    for g, w in zip(gs[1:], weights[1:]):
+        gx.addmm_(g, w)
+    if mask is not None:
+        gx = torch.ops.aten.threshold_backward(gx, mask, 0)
+    return gx + add if add is not None else gx
+
+
+class FusedFeedForwardHIP(torch.autograd.Function):
+    """``y = x + W2 relu(W1 x + b1) + b2`` (the feed-forward half of a block without norm layers
+    and dropout): two row-block launches forward, two backward -- the ReLU mask rides in the
+    epilogue of the first input-gradient kernel, the residual gradient in that of the second --
+    and both layers' weight and bias gradients from the grouped fixed-order kernel (deferred
+    inside :class:`deferred_weight_grads`)."""
+
+    @staticmethod
+    def forward(ctx, x, w1, b1, w2, b2):
+        x = x.contiguous()
+        h, = ops.linear_rows(x, (w1,), b1, relu=True)
+        y, = ops.linear_rows(h, (w2,), b2, residual=x)
+        ctx.save_for_backward(x, h, w1, w2)
+        ctx.leaves = tuple(t if (t is not None and t.is_leaf) else None for t in (w1, b1, w2, b2))
+        ctx.has_bias = (b1 is not None, b2 is not None)
+        return y
+
+    @staticmethod
+    def backward(ctx, g):
+        x, h, w1, w2 = ctx.saved_tensors
+        g = g.contiguous()
+        gh = input_gradient([g], [w2], None, h, h)                 # (g W2) where the ReLU was open
+        gx = input_gradient([gh], [w1], g, None, x) if ctx.needs_input_grad[0] else None
+        w1_p, b1_p, w2_p, b2_p = ctx.leaves
+        need = ctx.needs_input_grad
+        layers = [(gh, x, w1, w1_p, b1_p, need[1], ctx.has_bias[0] and need[2]),
+                  (g, h, w2, w2_p, b2_p, need[3], ctx.has_bias[1] and need[4])]
+        out = [None, None, None, None]                             # gw1, gb1, gw2, gb2
+        immediate = []
+        for k, (gg, xx, w, w_p, b_p, want_w, want_b) in enumerate(layers):
+            if not want_w and not want_b:
+                continue
+            if _deferred is not None and want_w and w_p is not None and w_p.grad is None and \
+                    (not ctx.has_bias[k] or (want_b and b_p is not None and b_p.grad is None)):
+                _deferred.append((gg, xx, w_p, b_p if want_b else None, 0))
+            else:
+                gw = torch.empty_like(w, memory_format=torch.contiguous_format)
+                gb = torch.empty(w.shape[0], dtype=w.dtype, device=w.device) if want_b else None
+                immediate.append((gg, xx, gw, gb))
+                out[2 * k], out[2 * k + 1] = (gw if want_w else None), gb
+        if immediate:
+            ops.linear_weight_grad_grouped(immediate)
+        return (gx, *out)
+
+
 class FusedLinearHIP(torch.autograd.Function):
     """``(y_0, ..)`` with ``y_i = act(x W_i^T + b_i) (+ residual)`` for up to three equally
     shaped weights sharing the input (query / key / value projections) in one row-block
     launch, bias, ReLU and residual in its epilogue.  ``bias`` is one vector over all
-    outputs (n_weights * C).  Backward: the input gradient as library GEMMs accumulating
-    into one buffer, weight and bias gradients from the grouped fixed-order kernel (deferred
-    to the end of the backward pass inside :class:`deferred_weight_grads`)."""
+    outputs (n_weights * C).  With ``carry`` the input itself is returned as one more output
+    (an identity whose gradient this node adds to the input gradient in the epilogue of its
+    own kernel, where autograd would launch an addition for a residual branch that leaves the
+    input here).  Backward: the input gradient from the row-block kernel for all terms at
+    once, weight and bias gradients from the grouped fixed-order kernel (deferred to the end
+    of the backward pass inside :class:`deferred_weight_grads`)."""
 
     @staticmethod
-    def forward(ctx, x, bias, residual, relu, *weights):
+    def forward(ctx, x, bias, residual, relu, carry, *weights):
         if relu and (residual is not None or len(weights) != 1):
             raise ValueError("FusedLinearHIP: ReLU goes with a single weight and no residual")
-        x = x.contiguous()
-        ys = ops.linear_rows(x, weights, bias, residual=residual, relu=relu)
-        ctx.save_for_backward(x, *weights, *((ys[0],) if relu else ()))
-        ctx.relu, ctx.nw = relu, len(weights)
+        if carry and not x.is_contiguous():
+            raise ValueError("FusedLinearHIP: a carried input must be contiguous")
+        xc = x.contiguous()
+        ys = ops.linear_rows(xc, weights, bias, residual=residual, relu=relu)
+        ctx.save_for_backward(xc, *weights, *((ys[0],) if relu else ()))
+        ctx.relu, ctx.nw, ctx.carry = relu, len(weights), carry
         # the parameters themselves (leaves only: no cycle through the graph), for deferred gradients
         ctx.leaves = ([w if w.is_leaf else None for w in weights],
                       bias if (bias is not None and bias.is_leaf) else None, bias is not None)
-        return tuple(ys)
+        return (*ys, x) if carry else tuple(ys)
 
     @staticmethod
     def backward(ctx, *gs):
         saved = ctx.saved_tensors
         x, weights = saved[0], saved[1:1 + ctx.nw]
         C = weights[0].shape[0]
-        gs = [g.contiguous() if g is not None else None for g in gs]
+        g_carry = gs[ctx.nw] if ctx.carry else None
+        gs = [g.contiguous() if g is not None else None for g in gs[:ctx.nw]]
         if ctx.relu and gs[0] is not None:
             gs[0] = torch.ops.aten.threshold_backward(gs[0], saved[-1], 0)
         g_res = gs[0] if ctx.needs_input_grad[2] else None
         gx = None
         if ctx.needs_input_grad[0]:
-            for g, w in zip(gs, weights):
-                if g is not None:
-                    gx = torch.mm(g, w) if gx is None else gx.addmm_(g, w)
-            if gx is None:
-                gx = torch.zeros_like(x)
-        need_w = [ctx.needs_input_grad[4 + i] for i in range(ctx.nw)]
+            gx = input_gradient([g for g in gs if g is not None],
+                                [w for g, w in zip(gs, weights) if g is not None], g_carry, None, x)
+        need_w = [ctx.needs_input_grad[5 + i] for i in range(ctx.nw)]
         leaves_w, bias_p, has_bias = ctx.leaves
         want_b = has_bias and ctx.needs_input_grad[1]
         gws = [None] * ctx.nw
@@ -379,7 +444,7 @@ class FusedLinearHIP(torch.autograd.Function):
                 ops.linear_weight_grad_grouped([(gs[i], x, gws[i], gb[i * C:(i + 1) * C] if want_b else None)
                                                 for i in range(ctx.nw)])
                 gws = [gw if need else None for gw, need in zip(gws, need_w)]
-        return (gx, gb, g_res, None, *gws)
+        return (gx, gb, g_res, None, None, *gws)
 
 
 # A list while a training step defers its linear layers' weight gradients (see

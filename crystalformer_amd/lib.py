@@ -43,6 +43,7 @@ SIGNATURES = {
     "cf_edge_index": (_int, [_ptr, _ptr, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "cf_edge_pairs": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _ptr, _ptr]),
     "cf_linear_rows": (_int, [_ptr, _i64, _i64, _ptr, _ptr, _ptr, _int, _i64, _ptr, _ptr, _int, _ptr, _ptr, _ptr, _ptr]),
+    "cf_linear_rows_nn": (_int, [_ptr, _ptr, _ptr, _int, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "cf_linear_weight_grad_workspace": (_i64, [_i64, _i64, _i64]),
     "cf_linear_weight_grad": (_int, [_ptr, _ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),
     "cf_linear_weight_grad_grouped_workspace": (_i64, [_int, _ptr, _ptr, _ptr]),

@@ -705,6 +705,40 @@ def linear_rows(x: Tensor, weights, bias: Optional[Tensor] = None, residual: Opt
     return tuple(ys)
 
 
+def linear_rows_nn_supported(g: Tensor, w: Tensor) -> bool:
+    """True when :func:`linear_rows_nn` serves g (N,C) @ w (C,K): float32 on the GPU, C a
+    multiple of 64, K a multiple of 4."""
+    return (g.is_cuda and w.is_cuda and g.dtype == torch.float32 and w.dtype == torch.float32 and g.dim() == 2
+            and w.dim() == 2 and g.shape[1] == w.shape[0] and g.shape[1] % 64 == 0 and w.shape[1] % 4 == 0)
+
+
+def linear_rows_nn(gs, weights, add: Optional[Tensor] = None, mask: Optional[Tensor] = None) -> Tensor:
+    """``mask(sum_i gs[i] @ weights[i]) + add`` for up to three terms of equal shapes in one
+    launch: the input gradient of linear layers ``y = x W^T`` (``weights[i]`` is W as stored,
+    (C,K) = (out, in)).  ``mask`` zeroes the product where it is not positive."""
+    gs = [_f32(g, "g") for g in gs]
+    weights = [_f32(w, "weight") for w in weights]
+    dev = require_device(*gs, *weights, add, mask)
+    add, mask = _f32(add, "add"), _f32(mask, "mask")
+    if not 1 <= len(gs) <= 3 or len(gs) != len(weights):
+        raise _lib.CrystalformerHipError("linear_rows_nn: one to three (g, weight) pairs expected")
+    N, C = gs[0].shape
+    K = weights[0].shape[1]
+    if any(g.shape != (N, C) for g in gs) or any(w.shape != (C, K) for w in weights):
+        raise _lib.CrystalformerHipError("linear_rows_nn: g (N,C) and weight (C,K) of equal shapes expected")
+    for t, name in ((add, "add"), (mask, "mask")):
+        if t is not None and t.shape != (N, K):
+            raise _lib.CrystalformerHipError(f"linear_rows_nn: {name} must be (N,K)")
+    y = torch.empty((N, K), dtype=torch.float32, device=dev)
+    g3 = gs + [None] * (3 - len(gs))
+    w3 = weights + [None] * (3 - len(weights))
+    with device_guard(dev):
+        rc = _lib.load().cf_linear_rows_nn(ptr(g3[0]), ptr(g3[1]), ptr(g3[2]), len(gs), ptr(w3[0]), ptr(w3[1]),
+                                           ptr(w3[2]), N, C, K, ptr(add), ptr(mask), ptr(y), stream_handle(dev))
+    check(rc, "cf_linear_rows_nn")
+    return y
+
+
 def column_sum(g: Tensor) -> Tensor:
     """Sum over the rows of a (N,C) float32 matrix, fixed order, one launch."""
     dev = require_device(g)

@@ -300,6 +300,17 @@ int cf_linear_rows(const float *x, int64_t N, int64_t K, const float *w0, const 
                    const float *residual, int relu, float *y0, float *y1, float *y2, void *stream);
 
 /*
+ * Input gradient of linear layers (what autograd computes for the F.linear calls cited at
+ * cf_linear_rows): y (N,K) = mask(sum_i g_i W_i) + add, g_i (N,C), W_i (C,K) row-major, 1..3 terms
+ * of equal shapes (query / key / value projections share their input); add (N,K) or NULL (a
+ * gradient arriving on a residual branch); mask (N,K) or NULL: where mask <= 0 the product is
+ * zeroed (the ReLU in front of the layer).  C a multiple of 64, K of 4.
+ */
+int cf_linear_rows_nn(const float *g0, const float *g1, const float *g2, int n_terms, const float *w0,
+                      const float *w1, const float *w2, int64_t N, int64_t C, int64_t K, const float *add,
+                      const float *mask, float *y, void *stream);
+
+/*
  * Column sums of a row-major (N,C) matrix, out (C): the bias gradient of the linear layers
  * (what autograd computes for the F.linear calls cited at cf_linear_rows), in a fixed
  * order, one launch, no scratch.

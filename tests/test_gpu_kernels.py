@@ -724,9 +724,9 @@ def test_fused_linear_function_grads(dev, defer):
     leaves = [t.to(dev).requires_grad_() for t in (x0, *ws, b3, w1, b1, w2, b2)]
     x, a, b, c, bb, w1d, b1d, w2d, b2d = leaves
     loss = graph(x, (a, b, c), bb, w1d, b1d, w2d, b2d,
-                 lambda x, b3, ws: hip_funcs.FusedLinearHIP.apply(x, b3, None, False, *ws),
-                 lambda x, b, w: hip_funcs.FusedLinearHIP.apply(x, b, None, True, w)[0],
-                 lambda x, b, r, w: hip_funcs.FusedLinearHIP.apply(x, b, r, False, w)[0])
+                 lambda x, b3, ws: hip_funcs.FusedLinearHIP.apply(x, b3, None, False, False, *ws),
+                 lambda x, b, w: hip_funcs.FusedLinearHIP.apply(x, b, None, True, False, w)[0],
+                 lambda x, b, r, w: hip_funcs.FusedLinearHIP.apply(x, b, r, False, False, w)[0])
     if defer:
         with hip_funcs.deferred_weight_grads():
             loss.backward()
@@ -798,3 +798,56 @@ def test_reci_enc_clamp_and_function(dev):
     assert float((z.detach().cpu() - z_ref)[solid].abs().max()) < 1e-4
     ga_ref = ks.reci_enc_bwd(a, kr_ref, rec, b.batch, e_start, gz, se_ref, 2)
     assert_close(ad.grad, ga_ref, "ga", rtol=2e-4)
+
+
+@pytest.mark.parametrize("N,C,K,terms", [(1774, 128, 128, 3), (1774, 512, 128, 1), (1774, 128, 512, 1), (70, 64, 20, 2),
+                                         (3, 64, 4, 1), (130, 192, 72, 3)])
+def test_linear_rows_nn(dev, N, C, K, terms):
+    """Input-gradient kernel: mask(sum_i g_i W_i) + add against float64, with ragged row and
+    column tails, one to three terms, with and without addend and mask."""
+    gen = torch.Generator().manual_seed(N + C + K + terms)
+    gs = [torch.randn(N, C, generator=gen) for _ in range(terms)]
+    ws = [torch.randn(C, K, generator=gen) * 0.1 for _ in range(terms)]
+    add, mask = torch.randn(N, K, generator=gen), torch.randn(N, K, generator=gen)
+    base = sum(g.double() @ w.double() for g, w in zip(gs, ws))
+    dg, dw = [g.to(dev) for g in gs], [w.to(dev) for w in ws]
+    assert ops.linear_rows_nn_supported(dg[0], dw[0])
+    assert_close(ops.linear_rows_nn(dg, dw), base.float(), "plain", rtol=3e-6)
+    assert_close(ops.linear_rows_nn(dg, dw, add=add.to(dev)), (base + add.double()).float(), "add", rtol=3e-6)
+    want = torch.where(mask.double() > 0, base, torch.zeros_like(base)) + add.double()
+    assert_close(ops.linear_rows_nn(dg, dw, add=add.to(dev), mask=mask.to(dev)), want.float(), "mask + add", rtol=3e-6)
+    assert not ops.linear_rows_nn_supported(torch.randn(4, 30, device=dev), torch.randn(30, 8, device=dev))
+
+
+@pytest.mark.parametrize("defer", [False, True])
+def test_fused_feed_forward_and_carried_input(dev, defer):
+    """One block's dense path as the graphed training step runs it -- projections with the input
+    carried to the residual of the output projection, then FusedFeedForwardHIP -- against float64
+    autograd of the same expression: y = z + W2 relu(W1 z + b1) + b2, z = x + Wo (q * k + v) + bo."""
+    from crystalformer_amd import hip_funcs
+    gen = torch.Generator().manual_seed(29)
+    N, E, F = 210, 64, 128
+    shapes = dict(x=(N, E), wq=(E, E), wk=(E, E), wv=(E, E), b3=(3 * E,), wo=(E, E), bo=(E,), w1=(F, E), b1=(F,),
+                  w2=(E, F), b2=(E,))
+    vals = {k: torch.randn(*shp, generator=gen) * (0.2 if k.startswith("w") else 1.0) for k, shp in shapes.items()}
+    t = torch.randn(N, E, generator=gen)
+    lin = torch.nn.functional.linear
+    r = {k: v.double().requires_grad_() for k, v in vals.items()}
+    bq, bk, bv = r["b3"].split(E)
+    z = r["x"] + lin(lin(r["x"], r["wq"], bq) * lin(r["x"], r["wk"], bk) + lin(r["x"], r["wv"], bv), r["wo"], r["bo"])
+    y_ref = z + lin(torch.relu(lin(z, r["w1"], r["b1"])), r["w2"], r["b2"])
+    (y_ref * t.double()).sum().backward()
+    d = {k: v.to(dev).requires_grad_() for k, v in vals.items()}
+    q, k, v, xc = hip_funcs.FusedLinearHIP.apply(d["x"], d["b3"], None, False, True, d["wq"], d["wk"], d["wv"])
+    z, = hip_funcs.FusedLinearHIP.apply(q * k + v, d["bo"], xc, False, False, d["wo"])
+    y = hip_funcs.FusedFeedForwardHIP.apply(z, d["w1"], d["b1"], d["w2"], d["b2"])
+    assert_close(y, y_ref.detach().float(), "y", rtol=3e-6)
+    if defer:
+        with hip_funcs.deferred_weight_grads():
+            (y * t.to(dev)).sum().backward()
+            assert d["w1"].grad is None and d["b3"].grad is None
+    else:
+        (y * t.to(dev)).sum().backward()
+    for name in shapes:
+        assert d[name].grad is not None, name
+        assert_close(d[name].grad, r[name].grad.float(), name, rtol=1e-5)
