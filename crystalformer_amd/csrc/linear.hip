@@ -448,13 +448,19 @@ extern "C" int cf_linear_rows(const float *x, int64_t N, int64_t K, const float 
     }
     p.bias = bias; p.res = residual;
     p.N = N; p.K = (int)K; p.C = (int)C; p.nw = n_weights; p.relu = relu;
-    // wide outputs: 64 x 64 tiles (2 x 2 wavefronts); narrow ones: 64 x 32 (4 x 1), more work-groups
+    // wide outputs: 64-column tiles (2 x 2 wavefronts); narrow ones: 32-column tiles, more work-groups
     const int64_t total_cols = (int64_t)n_weights * C;
     const bool wide = total_cols >= 256;
-    const int64_t gx = (N + 63) / 64;
+    // few rows (a tile grid that leaves CUs idle): half-height tiles, twice the work-groups
+    const bool small = N <= 8192;
+    const int64_t gx = (N + (small ? 31 : 63)) / (small ? 32 : 64);
     const int64_t gy = (total_cols + (wide ? 63 : 31)) / (wide ? 64 : 32);
     CF_REQUIRE(gx < (1ll << 31) && gy < 65536, CF_ERR_UNSUPPORTED, "cf_linear_rows: too large");
-    if (wide)
+    if (small && wide)
+        linear_rows_kernel<32, 64, 2, 2><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
+    else if (small)
+        linear_rows_kernel<32, 32, 2, 2><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
+    else if (wide)
         linear_rows_kernel<64, 64, 2, 2><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
     else
         linear_rows_kernel<64, 32, 4, 1><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
