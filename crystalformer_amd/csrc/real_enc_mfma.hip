@@ -111,6 +111,27 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         geo = unit_geom(gv0, !UNIFORM);
         ids_next = unit_ids(dv1);
     }
+    // Fixed cube: the translation a lane evaluates in chunk ch is the same in every round; the
+    // first two chunks (128 translations, the default cube has 125) are decoded once.
+    constexpr int NPRE = 2;
+    float npre[UNIFORM ? NPRE : 1][3];
+    if (UNIFORM) {
+        BoxDims b0;
+        b0.U1 = b0.U2 = b0.U3 = p.lattice_range;
+        b0.S3 = b0.S2 = 2 * p.lattice_range + 1;
+        b0.plane = b0.S2 * b0.S3;
+        b0.T = b0.S2 * b0.plane;
+        b0.inv_plane = 1.0f / (float)b0.plane;
+        b0.inv_S3 = 1.0f / (float)b0.S3;
+#pragma unroll
+        for (int ch = 0; ch < NPRE; ch++) {
+            int n1, n2, n3;
+            decode(b0, min(ch * WAVE + lane, b0.T - 1), n1, n2, n3);
+            npre[ch][0] = (float)n1;
+            npre[ch][1] = (float)n2;
+            npre[ch][2] = (float)n3;
+        }
+    }
     int it = 0;
     for (int rd = blockIdx.x; rd < rounds; it++) {
         const int hg = pos.hg;
@@ -223,7 +244,13 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 d2c[ch] = 0.f;
                 if (ch < nchunk) {
                     int cb;
-                    geometry(ch * WAVE + lane, ch * WAVE + lane < T, d2c[ch], cb);
+                    if (UNIFORM && ch < NPRE) {
+                        d2c[ch] = dist2(cell, npre[UNIFORM ? ch : 0][0], npre[UNIFORM ? ch : 0][1],
+                                        npre[UNIFORM ? ch : 0][2]);
+                        cb = ch * WAVE + lane < T ? 0xFFFF : 0;
+                    } else {
+                        geometry(ch * WAVE + lane, ch * WAVE + lane < T, d2c[ch], cb);
+                    }
                     track_min(d2c[ch], cb, ch * WAVE + lane);
                     if (!UNIFORM) bitsc[ch] = cb;
                 }
@@ -407,7 +434,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         // column totals: the 4 lanes sharing c hold partial sums
         sum += __shfl_xor(sum, 16, WAVE);
         sum += __shfl_xor(sum, 32, WAVE);
-        const float inv = 1.0f / sum;
+        const float inv = __builtin_amdgcn_rcpf(sum);      // 1 ulp, one instruction
         const int64_t e_col = (c < 8) ? e_ij : e_ji;
         if (col_on && q == 0) p.z[e_col * H + h] = log2_hw(sum) * LN2 + d2min * a;
 
