@@ -84,6 +84,22 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
     ops.set_event_log(None)
     calls.clear()
     submission = "eager launches"
+    # the same step with the fused pieces (row-block linear Functions, grouped weight gradients, one
+    # device-side clip + AdamW update), still launched eagerly: what a loop over changing batches gets
+    from crystalformer_amd.training import FusedAdamW, fused_training_step
+    fopt = FusedAdamW(model)
+    for _ in range(max(args.warmup, 1)):
+        fused_training_step(model, data, fopt)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = fused_training_step(model, data, fopt)
+    torch.cuda.synchronize()
+    fused_elapsed = time.perf_counter() - t0
+    eager["fused_step"] = {"value": round(B * args.steps / fused_elapsed, 2),
+                           "ms_per_step": round(fused_elapsed / args.steps * 1e3, 4)}
+    del loss
+    fopt.zero_grad(set_to_none=True)
     if not args.no_graph:
         # the same step (device-side schedule, capturable AdamW) as one HIP graph replay
         from crystalformer_amd.graphs import GraphedTrainStep

@@ -108,23 +108,8 @@ class GraphedTrainStep:
             torch.cuda.synchronize()
 
     def _step(self) -> torch.Tensor:
-        from . import hip_funcs
-        previous = hip_funcs.USE_LINEAR_FUNCTION
-        hip_funcs.USE_LINEAR_FUNCTION = True
-        try:
-            return self._step_body()
-        finally:
-            hip_funcs.USE_LINEAR_FUNCTION = previous
-
-    def _step_body(self) -> torch.Tensor:
-        import torch.nn.functional as F
-        from . import hip_funcs
-        out = self.model(self.static)
-        loss = F.l1_loss(out[:, 0], self.static.y, reduction="none").mean()
-        with hip_funcs.deferred_weight_grads():           # all linear layers' weight gradients at the end
-            loss.backward()
-        self.opt.step()
-        return loss.detach()
+        from .training import fused_training_step
+        return fused_training_step(self.model, self.static, self.opt, zero_grad=False)
 
     def __call__(self, batch: Optional[CrystalBatch] = None) -> torch.Tensor:
         if batch is not None and batch is not self.static:

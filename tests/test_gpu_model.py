@@ -443,3 +443,22 @@ def test_multihead_blocks_with_value_encoding_follow_the_kernel_path(dev):
         assert_close(values[li], cap[f"layer{li}.values"], f"layer {li} values")
         assert float(values[li][:, H // 2:].abs().max()) == 0.0
     assert_close(y, y_ref, "model output")
+
+
+def test_fused_training_step_follows_plain_step_on_changing_batches(dev):
+    """fused_training_step (eager, any batch) against the plain training_step with
+    torch.optim.AdamW on a sequence of different batches: same losses to optimiser round-off."""
+    from crystalformer_amd.synthetic import make_batch
+    from crystalformer_amd.training import FusedAdamW, fused_training_step, make_optimizer, training_step
+    import copy
+    _, m_plain = build_model("cfg1_simplified_b32", num_layers=2, value_pe_dist_real=16)
+    m_plain.to(dev).train()
+    m_fused = copy.deepcopy(m_plain)
+    opt, sch = make_optimizer(m_plain)
+    fopt = FusedAdamW(m_fused)
+    for step in range(5):
+        b = make_batch(6 + step, (1, 9), False, (3.0, 7.0), (70.0, 110.0), seed=40 + step, with_targets=True).to(dev)
+        lp = float(training_step(m_plain, b, opt, sch))
+        lf = float(fused_training_step(m_fused, b, fopt))
+        assert abs(lp - lf) <= 2e-4 * max(1.0, abs(lp)), (step, lp, lf)
+    assert float(fopt.state[0]) == 5
