@@ -118,12 +118,7 @@ class CrystalformerEncoderLayerCUDA(Module):
             x = self.self_attn(x, x, x, batch, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell,
                                onehot, need_weights=False, residual=x)[0]
             h, = ops.linear_rows(x, (self.linear1.weight,), self.linear1.bias, relu=True)
-            if self.linear2.weight.shape[1] <= 256:
-                x, = ops.linear_rows(h, (self.linear2.weight,), self.linear2.bias, residual=x)
-            else:
-                # long reduction, narrow output: too few tiles for the row-block kernel (measured
-                # 11 us against 8 us for the library GEMM plus the add at 1774 x 512 -> 128)
-                x = x + F.linear(h, self.linear2.weight, self.linear2.bias)
+            x, = ops.linear_rows(h, (self.linear2.weight,), self.linear2.bias, residual=x)
             return x
         if self._fused_train(x):
             # the same epilogues with autograd (graphed training step, no norm layers, no dropout)
