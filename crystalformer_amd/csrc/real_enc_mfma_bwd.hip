@@ -156,8 +156,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         bx.S2 = 2 * bx.U2 + 1;
         bx.plane = bx.S2 * bx.S3;
         bx.T = (2 * bx.U1 + 1) * bx.plane;
-        bx.inv_plane = 1.0f / (float)bx.plane;
-        bx.inv_S3 = 1.0f / (float)bx.S3;
+        bx.inv_plane = __builtin_amdgcn_rcpf((float)bx.plane);
+        bx.inv_S3 = __builtin_amdgcn_rcpf((float)bx.S3);
         const int T = bx.T;
         ColumnBoxes cbox{0, 0, 0};
         if (!UNIFORM) cbox = column_boxes(R1, R2, R3, bx, lane);
