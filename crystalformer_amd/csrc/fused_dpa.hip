@@ -118,90 +118,122 @@ __global__ __launch_bounds__(256) void fused_dpa_fwd_kernel(DpaArgs p)
 // One work-group of 4 wavefronts per query atom, single pass over the edge row
 // with a running (max, sum, output) per head ("online" softmax).  Lane = (edge
 // slot, head, 4 components): the H*Dv/4 lanes of a slot read one edge's key row,
-// value row and b_ij row as consecutive 16-byte pieces (fully coalesced);
-// 4*ES = 4*64/(H*Dv/4) edges are in flight per step, the loop is unrolled 4x and
-// the key indices of the next step are fetched one step ahead.  The partial
+// value row and b_ij row as consecutive 16-byte pieces (fully coalesced).
+// A step covers 4 edges per slot (4*4*ES edges per work-group); all of its loads
+// are issued before the first is consumed, without branches: an edge past the end
+// of the row reads the row's last edge instead and is masked out of the sums, so
+// a row of up to one step costs one memory round trip after its key indices.
+// The key indices of the next step are fetched one step ahead.  The partial
 // (max, sum, output) of slots and wavefronts are merged through shuffles and LDS.
-// Raw logits are parked in prob[e,h] and normalised by a second, cheap sweep
-// (4*H bytes per edge).  Needs Dk == Dv, Dv/4 a power of two, H*Dv/4 <= 64.
+// Raw logits of whole steps are parked in prob[e,h] and normalised by a closing
+// sweep (4*H bytes per edge); those of the last, partial step stay in registers.
+// Needs Dk == Dv, Dv/4 a power of two, H*Dv/4 <= 64.
 typedef float float4_v __attribute__((ext_vector_type(4)));
 
 constexpr int DPA_WPQ = 4;     // wavefronts per query row
 
-__global__ __launch_bounds__(256) void fused_dpa_fwd_stream_kernel(DpaArgs p, int DV4, int LPE)
+// Sum over the DV4 adjacent lanes that hold one head's components; every lane of the
+// wavefront must be active.
+template <int DV4>
+__device__ __forceinline__ float head_sum(float s)
+{
+#pragma unroll
+    for (int off = DV4 >> 1; off >= 4; off >>= 1) s += __shfl_xor(s, off, WAVE);
+    if (DV4 >= 4) s += dpp_f<DPP_QUAD_2301, 0xF>(0.f, s);
+    if (DV4 >= 2) s += dpp_f<DPP_QUAD_1032, 0xF>(0.f, s);
+    return s;
+}
+
+// Loads and stores at a 32-bit byte offset from a wave-uniform base (scalar base + vector
+// offset addressing: no 64-bit address per lane).
+__device__ __forceinline__ float4_v ld4(const void *base, uint32_t byte_off)
+{
+    return *reinterpret_cast<const float4_v *>(static_cast<const char *>(base) + byte_off);
+}
+__device__ __forceinline__ float ld1(const void *base, uint32_t byte_off)
+{
+    return *reinterpret_cast<const float *>(static_cast<const char *>(base) + byte_off);
+}
+__device__ __forceinline__ void st1(void *base, uint32_t byte_off, float v)
+{
+    *reinterpret_cast<float *>(static_cast<char *>(base) + byte_off) = v;
+}
+
+// Every byte offset into prob / b_ij / key / value fits 32 bits (checked by the host).
+template <int DV4, bool HAS_A, bool HAS_B>
+__global__ __launch_bounds__(256, 7) void fused_dpa_fwd_stream_kernel(DpaArgs p, int LPE)
 {
     __shared__ float part[DPA_WPQ][WAVE][6];
     __shared__ float fin[2][MAXH];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int64_t i = blockIdx.x;
-    const int H = p.H;
-    const int HD4 = LPE;                       // float4 pieces per edge row
+    const uint32_t i = blockIdx.x;
+    const uint32_t H = p.H;
+    const uint32_t HD4 = LPE;                  // float4 pieces per edge row
     const int ES = WAVE / LPE;                 // edge slots per wavefront
     const int es = lane / LPE;
-    const int piece = lane - es * LPE;         // which float4 of the (H,Dv) row
-    const int h = piece / DV4;
-    const bool lead = (piece - h * DV4) == 0;  // first piece of its head: owns the logit
-    const int64_t e0 = p.e_start[i], e1 = p.e_start[i + 1];
+    const uint32_t piece = lane - es * LPE;    // which float4 of the (H,Dv) row
+    const uint32_t h = piece / DV4;
+    const bool lead = (piece % DV4) == 0;      // first piece of its head: owns the logit
+    const uint32_t e0 = (uint32_t)p.e_start[i], e1 = (uint32_t)p.e_start[i + 1];
+    if (e0 >= e1) {                            // an atom without edges yields zeros (whole work-group)
+        if (threadIdx.x < HD4)
+            reinterpret_cast<float4_v *>(p.out)[i * HD4 + threadIdx.x] = float4_v{0.f, 0.f, 0.f, 0.f};
+        return;
+    }
+    const uint32_t e_last = e1 - 1;
     const int64_t *dst = p.edges + p.E;
-    const float4_v *key4 = reinterpret_cast<const float4_v *>(p.key);
-    const float4_v *val4 = reinterpret_cast<const float4_v *>(p.val);
-    const float4_v *bij4 = reinterpret_cast<const float4_v *>(p.bij);
-    const float4_v q4 = reinterpret_cast<const float4_v *>(p.que)[i * HD4 + piece];
+    const float4_v q4 = ld4(p.que, (i * HD4 + piece) * 16u);
 
     float m = -1.0e30f, l = 0.f;
     float4_v acc = {0.f, 0.f, 0.f, 0.f};
-    // Raw logits of the main loop are parked in prob[] and normalised by the closing sweep; those of
-    // the last (for most rows: the only) partial step stay in registers and are written once,
-    // normalised, so that a short row never reads its own stores back.
-    auto step = [&](int64_t e, int64_t j, bool park) -> float {
-        const float4_v k4 = key4[j * HD4 + piece];
-        float4_v v4 = val4[j * HD4 + piece];
-        if (bij4) {
-            const float4_v b4 = bij4[e * HD4 + piece];
-            v4 += b4;
-        }
-        float s = q4.x * k4.x + q4.y * k4.y + q4.z * k4.z + q4.w * k4.w;
-        for (int off = DV4 >> 1; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
-        if (p.aij) s += p.aij[e * H + h];
-        if (park && lead) p.prob[e * H + h] = s;
-        const float m_new = fmaxf(m, s);
+    float4_v k4[4], v4[4], b4[4];
+    float av[4];
+    auto fetch = [&](int u, uint32_t e, uint32_t j) {
+        if (HAS_B) b4[u] = ld4(p.bij, (e * HD4 + piece) * 16u);      // independent of the key index: first
+        if (HAS_A) av[u] = ld1(p.aij, (e * H + h) * 4u);
+        k4[u] = ld4(p.key, (j * HD4 + piece) * 16u);
+        v4[u] = ld4(p.val, (j * HD4 + piece) * 16u);
+    };
+    auto fold = [&](int u, bool valid) -> float {
+        float4_v vv = v4[u];
+        if (HAS_B) vv += b4[u];
+        float s = q4.x * k4[u].x + q4.y * k4[u].y + q4.z * k4[u].z + q4.w * k4[u].w;
+        s = head_sum<DV4>(s);
+        if (HAS_A) s += av[u];
+        const float m_new = valid ? fmaxf(m, s) : m;
         const float sc = exp2_hw((m - m_new) * LOG2E);
-        const float pe = exp2_hw((s - m_new) * LOG2E);
+        const float pe = valid ? exp2_hw((s - m_new) * LOG2E) : 0.f;
         l = l * sc + pe;
-        acc = acc * sc + v4 * pe;
+        acc = acc * sc + vv * pe;
         m = m_new;
         return s;
     };
-    const int stride = DPA_WPQ * ES;
+    const uint32_t stride = DPA_WPQ * ES;
     // the main loop takes whole steps of 4 * stride edges (the same number in every lane), the
     // rest of the row (fewer than 4 * stride edges) is the partial step
-    int64_t eb = e0;
-    int64_t e = eb + wave * ES + es;
-    // key indices one step (4 edges per slot) ahead
-    int64_t jn[4];
-#pragma unroll
-    for (int u = 0; u < 4; u++) jn[u] = (e + u * stride < e1) ? dst[e + u * stride] : 0;
-    for (; eb + 4 * stride <= e1; eb += 4 * stride, e += 4 * stride) {
-        int64_t jc[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) jc[u] = jn[u];
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int64_t en = e + (4 + u) * stride;
-            jn[u] = (en < e1) ? dst[en] : 0;
-        }
-#pragma unroll
-        for (int u = 0; u < 4; u++) step(e + u * stride, jc[u], true);
-    }
-    const int64_t e_tail = e;                      // first edge of this lane's slot in the last step
-    const int64_t parked = (eb - e0) * H;          // logits parked by the main loop
+    uint32_t eb = e0;
+    uint32_t e = eb + wave * ES + es;
     float s_tail[4];
+    for (;;) {
+        const bool last = eb + 4 * stride >= e1;                    // uniform
+        uint32_t jn[4];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-        s_tail[u] = 0.f;
-        if (e_tail + u * stride < e1) s_tail[u] = step(e_tail + u * stride, jn[u], false);
+        for (int u = 0; u < 4; u++) jn[u] = (uint32_t)dst[min(e + u * stride, e_last)];
+#pragma unroll
+        for (int u = 0; u < 4; u++) fetch(u, min(e + u * stride, e_last), jn[u]);
+#pragma unroll
+        for (int u = 0; u < 4; u++) s_tail[u] = fold(u, e + u * stride < e1);
+        if (last) break;
+        if (lead) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) st1(p.prob, ((e + u * stride) * H + h) * 4u, s_tail[u]);
+        }
+        eb += 4 * stride;
+        e += 4 * stride;
     }
+    const uint32_t e_tail = e;                     // first edge of this lane's slot in the last step
+    const uint32_t parked = (eb - e0) * H;         // logits parked by the earlier steps
     // merge the edge slots of this wavefront
     auto merge = [&](float mo, float lo, float4_v ao) {
         const float m_new = fmaxf(m, mo);
@@ -226,77 +258,116 @@ __global__ __launch_bounds__(256) void fused_dpa_fwd_stream_kernel(DpaArgs p, in
         dstp[0] = m; dstp[1] = l; dstp[2] = acc.x; dstp[3] = acc.y; dstp[4] = acc.z; dstp[5] = acc.w;
     }
     __syncthreads();
-    if (wave == 0 && es == 0) {
+    const bool closer = wave == 0 && es == 0;
+    if (closer) {
         for (int w = 1; w < DPA_WPQ; w++) {
             const float *src = part[w][piece];
             merge(src[0], src[1], float4_v{src[2], src[3], src[4], src[5]});
         }
-        const float inv = l > 0.f ? 1.0f / l : 0.f;     // an atom without edges yields zeros
-        reinterpret_cast<float4_v *>(p.out)[i * HD4 + piece] = acc * inv;
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        acc = acc * inv;
         if (lead) {
             fin[0][h] = m;
             fin[1][h] = inv;
         }
     }
     __syncthreads();
-    // normalise the parked logits: element x of the row's (n,H) block belongs to head x % H
+    if (closer) reinterpret_cast<float4_v *>(p.out)[i * HD4 + piece] = acc;   // after the barrier: nothing waits for it
+    // normalise: the partial step from registers, the parked logits in place (element x of the
+    // row's (n,H) block belongs to head x % H)
     if (lead) {
         const float mt = fin[0][h], it = fin[1][h];
 #pragma unroll
         for (int u = 0; u < 4; u++)
             if (e_tail + u * stride < e1)
-                p.prob[(e_tail + u * stride) * H + h] = exp2_hw((s_tail[u] - mt) * LOG2E) * it;
+                st1(p.prob, ((e_tail + u * stride) * H + h) * 4u, exp2_hw((s_tail[u] - mt) * LOG2E) * it);
     }
-    const int hx = threadIdx.x % H;
-    const float mh = fin[0][hx], ih = fin[1][hx];
-    float *row = p.prob + e0 * H;
-    for (int64_t x = threadIdx.x; x < parked; x += blockDim.x) row[x] = exp2_hw((row[x] - mh) * LOG2E) * ih;
+    if (parked > 0) {
+        const uint32_t hx = threadIdx.x % H;
+        const float mh = fin[0][hx], ih = fin[1][hx];
+        float *row = p.prob + (size_t)e0 * H;
+        for (uint32_t x = threadIdx.x; x < parked; x += blockDim.x) row[x] = exp2_hw((row[x] - mh) * LOG2E) * ih;
+    }
 }
 
 // ------------------------------------------------- backward, streaming version
-// Same lane layout as the streaming forward (work-group of 4 wavefronts per atom,
-// lane = (edge slot, head, 4 components)), two kernels, fixed summation order:
+// Same lane layout and load batching as the streaming forward (work-group of 4
+// wavefronts per atom, lane = (edge slot, head, 4 components), 4 edges per slot and
+// step, loads of a step issued together, edges past the end clamped and masked),
+// two kernels, fixed summation order:
 //   query side  per query i over its edge row: gb_ij = go_i p_ij (stored),
 //               gs_ij = sum_d (v_j + b_ij - o_i) gb_ij (stored as gaij),
 //               gq_i = sum_j gs_ij k_j;
 //   key side    per key j over the column (i, j) of the crystal's dense block:
 //               gv_j = sum_i go_i p_ij, gk_j = sum_i gs_ij q_i.
-__global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs p, int DV4, int LPE)
+__device__ __forceinline__ void st4(void *base, uint32_t byte_off, float4_v v)
+{
+    *reinterpret_cast<float4_v *>(static_cast<char *>(base) + byte_off) = v;
+}
+
+template <int DV4, bool HAS_B, bool WANT_GB>
+__global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs p, int LPE)
 {
     __shared__ float part[DPA_WPQ][WAVE][4];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int64_t i = blockIdx.x;
-    const int H = p.H;
-    const int HD4 = LPE;
+    const uint32_t i = blockIdx.x;
+    const uint32_t H = p.H;
+    const uint32_t HD4 = LPE;
     const int ES = WAVE / LPE;
     const int es = lane / LPE;
-    const int piece = lane - es * LPE;
-    const int h = piece / DV4;
-    const bool lead = (piece - h * DV4) == 0;
-    const int64_t e0 = p.e_start[i], e1 = p.e_start[i + 1];
+    const uint32_t piece = lane - es * LPE;
+    const uint32_t h = piece / DV4;
+    const bool lead = (piece % DV4) == 0;
+    const uint32_t e0 = (uint32_t)p.e_start[i], e1 = (uint32_t)p.e_start[i + 1];
+    if (e0 >= e1) {                            // an atom without edges: no query gradient (whole work-group)
+        if (threadIdx.x < HD4) st4(p.gque, (i * HD4 + threadIdx.x) * 16u, float4_v{0.f, 0.f, 0.f, 0.f});
+        return;
+    }
+    const uint32_t e_last = e1 - 1;
     const int64_t *dst = p.edges + p.E;
-    const float4_v *key4 = reinterpret_cast<const float4_v *>(p.key);
-    const float4_v *val4 = reinterpret_cast<const float4_v *>(p.val);
-    const float4_v *bij4 = reinterpret_cast<const float4_v *>(p.bij);
-    float4_v *gb4 = reinterpret_cast<float4_v *>(p.gbij);
-    const float4_v go4 = reinterpret_cast<const float4_v *>(p.gout)[i * HD4 + piece];
-    const float4_v o4 = reinterpret_cast<const float4_v *>(p.out_in)[i * HD4 + piece];
+    const float4_v go4 = ld4(p.gout, (i * HD4 + piece) * 16u);
+    const float4_v o4 = ld4(p.out_in, (i * HD4 + piece) * 16u);
     float4_v gq = {0.f, 0.f, 0.f, 0.f};
-    const int stride = DPA_WPQ * ES;
-    for (int64_t e = e0 + wave * ES + es; e < e1; e += stride) {
-        const int64_t j = dst[e];
-        const float pr = p.prob_in[e * H + h];
-        const float4_v k4 = key4[j * HD4 + piece];
-        float4_v m4 = val4[j * HD4 + piece];
-        if (bij4) m4 += bij4[e * HD4 + piece];
-        const float4_v t4 = go4 * pr;
-        if (gb4) gb4[e * HD4 + piece] = t4;
-        m4 -= o4;
-        float gs = m4.x * t4.x + m4.y * t4.y + m4.z * t4.z + m4.w * t4.w;
-        for (int off = DV4 >> 1; off > 0; off >>= 1) gs += __shfl_xor(gs, off, WAVE);
-        if (lead) p.gaij[e * H + h] = gs;
-        gq += k4 * gs;
+    const uint32_t stride = DPA_WPQ * ES;
+    uint32_t e = e0 + wave * ES + es;
+    for (uint32_t eb = e0; eb < e1; eb += 4 * stride, e += 4 * stride) {
+        uint32_t ec[4], j[4];
+        float pr[4], gsv[4];
+        float4_v k4[4], m4[4], b4[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            ec[u] = min(e + u * stride, e_last);
+            j[u] = (uint32_t)dst[ec[u]];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            pr[u] = ld1(p.prob_in, (ec[u] * H + h) * 4u);
+            if (HAS_B) b4[u] = ld4(p.bij, (ec[u] * HD4 + piece) * 16u);
+            m4[u] = ld4(p.val, (j[u] * HD4 + piece) * 16u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const bool valid = e + u * stride < e1;
+            const float4_v t4 = go4 * pr[u];
+            float4_v d4 = m4[u];
+            if (HAS_B) d4 += b4[u];
+            d4 -= o4;
+            float gs = d4.x * t4.x + d4.y * t4.y + d4.z * t4.z + d4.w * t4.w;
+            gs = head_sum<DV4>(gs);
+            if (valid) {
+                if (WANT_GB) st4(p.gbij, (ec[u] * HD4 + piece) * 16u, t4);
+                if (lead) st1(p.gaij, (ec[u] * H + h) * 4u, gs);
+            }
+            gsv[u] = valid ? gs : 0.f;
+        }
+        // the key rows (cache hits: the value rows of the same atoms were just read) come second,
+        // into the registers the value and b_ij rows have left
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 4; u++) k4[u] = ld4(p.key, (j[u] * HD4 + piece) * 16u);
+#pragma unroll
+        for (int u = 0; u < 4; u++) gq += k4[u] * gsv[u];
     }
     for (int off = LPE; off < WAVE; off <<= 1) {
         gq.x += __shfl_xor(gq.x, off, WAVE);
@@ -314,36 +385,48 @@ __global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs
             const float *s = part[w][piece];
             gq += float4_v{s[0], s[1], s[2], s[3]};
         }
-        reinterpret_cast<float4_v *>(p.gque)[i * HD4 + piece] = gq;
+        st4(p.gque, (i * HD4 + piece) * 16u, gq);
     }
 }
 
-__global__ __launch_bounds__(256) void fused_dpa_bwd_key_stream_kernel(DpaArgs p, int DV4, int LPE)
+template <int DV4>
+__global__ __launch_bounds__(256) void fused_dpa_bwd_key_stream_kernel(DpaArgs p, int LPE)
 {
     __shared__ float part[DPA_WPQ][WAVE][8];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int64_t j = blockIdx.x;
-    const int H = p.H;
-    const int HD4 = LPE;
+    const uint32_t j = blockIdx.x;
+    const uint32_t H = p.H;
+    const uint32_t HD4 = LPE;
     const int ES = WAVE / LPE;
     const int es = lane / LPE;
-    const int piece = lane - es * LPE;
-    const int h = piece / DV4;
+    const uint32_t piece = lane - es * LPE;
+    const uint32_t h = piece / DV4;
     const int64_t b = p.batch[j];
-    const int64_t ab = p.atom_start[b];
-    const int64_t n = p.atom_start[b + 1] - ab;
-    const int64_t eb = p.edge_start[b] + (j - ab);
-    const float4_v *que4 = reinterpret_cast<const float4_v *>(p.que);
-    const float4_v *go4 = reinterpret_cast<const float4_v *>(p.gout);
+    const uint32_t ab = (uint32_t)p.atom_start[b];
+    const uint32_t n = (uint32_t)p.atom_start[b + 1] - ab;          // >= 1: atom j is one of them
+    const uint32_t ebase = (uint32_t)p.edge_start[b] + (j - ab);
     float4_v gv = {0.f, 0.f, 0.f, 0.f}, gk = {0.f, 0.f, 0.f, 0.f};
-    const int stride = DPA_WPQ * ES;
-    for (int64_t il = wave * ES + es; il < n; il += stride) {
-        const int64_t e = eb + il * n;
-        const float pr = p.prob_in[e * H + h];
-        const float gs = p.gaij[e * H + h];
-        gv += go4[(ab + il) * HD4 + piece] * pr;
-        gk += que4[(ab + il) * HD4 + piece] * gs;
+    const uint32_t stride = DPA_WPQ * ES;
+    uint32_t il = wave * ES + es;
+    for (uint32_t ib = 0; ib < n; ib += 4 * stride, il += 4 * stride) {
+        float pr[4], gs[4];
+        float4_v g4[4], q4[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint32_t ic = min(il + u * stride, n - 1);
+            const uint32_t e = ebase + ic * n;
+            pr[u] = ld1(p.prob_in, (e * H + h) * 4u);
+            gs[u] = ld1(p.gaij, (e * H + h) * 4u);
+            g4[u] = ld4(p.gout, ((ab + ic) * HD4 + piece) * 16u);
+            q4[u] = ld4(p.que, ((ab + ic) * HD4 + piece) * 16u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const bool valid = il + u * stride < n;
+            gv += g4[u] * (valid ? pr[u] : 0.f);
+            gk += q4[u] * (valid ? gs[u] : 0.f);
+        }
     }
     for (int off = LPE; off < WAVE; off <<= 1) {
         gv.x += __shfl_xor(gv.x, off, WAVE); gv.y += __shfl_xor(gv.y, off, WAVE);
@@ -363,8 +446,8 @@ __global__ __launch_bounds__(256) void fused_dpa_bwd_key_stream_kernel(DpaArgs p
             gv += float4_v{s[0], s[1], s[2], s[3]};
             gk += float4_v{s[4], s[5], s[6], s[7]};
         }
-        reinterpret_cast<float4_v *>(p.gval)[j * HD4 + piece] = gv;
-        reinterpret_cast<float4_v *>(p.gkey)[j * HD4 + piece] = gk;
+        st4(p.gval, (j * HD4 + piece) * 16u, gv);
+        st4(p.gkey, (j * HD4 + piece) * 16u, gk);
     }
 }
 
@@ -477,6 +560,49 @@ void launch_fwd(const DpaArgs &p, hipStream_t st)
     fused_dpa_fwd_kernel<H><<<(int)((p.N + wpb - 1) / wpb), wpb * WAVE, 0, st>>>(p);
 }
 
+template <int DV4>
+void launch_fwd_stream_dv(const DpaArgs &p, int lpe, hipStream_t st)
+{
+    const dim3 grid((unsigned)p.N), block(DPA_WPQ * WAVE);
+    if (p.aij && p.bij) fused_dpa_fwd_stream_kernel<DV4, true, true><<<grid, block, 0, st>>>(p, lpe);
+    else if (p.aij) fused_dpa_fwd_stream_kernel<DV4, true, false><<<grid, block, 0, st>>>(p, lpe);
+    else if (p.bij) fused_dpa_fwd_stream_kernel<DV4, false, true><<<grid, block, 0, st>>>(p, lpe);
+    else fused_dpa_fwd_stream_kernel<DV4, false, false><<<grid, block, 0, st>>>(p, lpe);
+}
+
+void launch_fwd_stream(const DpaArgs &p, int dv4, int lpe, hipStream_t st)
+{
+    switch (dv4) {
+        case 1: launch_fwd_stream_dv<1>(p, lpe, st); break;
+        case 2: launch_fwd_stream_dv<2>(p, lpe, st); break;
+        case 4: launch_fwd_stream_dv<4>(p, lpe, st); break;
+        case 8: launch_fwd_stream_dv<8>(p, lpe, st); break;
+        default: launch_fwd_stream_dv<16>(p, lpe, st); break;
+    }
+}
+
+template <int DV4>
+void launch_bwd_stream_dv(const DpaArgs &p, int lpe, hipStream_t st)
+{
+    const dim3 grid((unsigned)p.N), block(DPA_WPQ * WAVE);
+    if (p.bij && p.gbij) fused_dpa_bwd_query_stream_kernel<DV4, true, true><<<grid, block, 0, st>>>(p, lpe);
+    else if (p.bij) fused_dpa_bwd_query_stream_kernel<DV4, true, false><<<grid, block, 0, st>>>(p, lpe);
+    else if (p.gbij) fused_dpa_bwd_query_stream_kernel<DV4, false, true><<<grid, block, 0, st>>>(p, lpe);
+    else fused_dpa_bwd_query_stream_kernel<DV4, false, false><<<grid, block, 0, st>>>(p, lpe);
+    fused_dpa_bwd_key_stream_kernel<DV4><<<grid, block, 0, st>>>(p, lpe);
+}
+
+void launch_bwd_stream(const DpaArgs &p, int dv4, int lpe, hipStream_t st)
+{
+    switch (dv4) {
+        case 1: launch_bwd_stream_dv<1>(p, lpe, st); break;
+        case 2: launch_bwd_stream_dv<2>(p, lpe, st); break;
+        case 4: launch_bwd_stream_dv<4>(p, lpe, st); break;
+        case 8: launch_bwd_stream_dv<8>(p, lpe, st); break;
+        default: launch_bwd_stream_dv<16>(p, lpe, st); break;
+    }
+}
+
 }  // namespace
 
 extern "C" int cf_fused_dpa_fwd(const float *que, const float *key, const float *val,
@@ -498,8 +624,9 @@ extern "C" int cf_fused_dpa_fwd(const float *que, const float *key, const float 
     // streaming kernel when a head's components split into 16-byte pieces that tile a wavefront
     const int64_t dv4 = Dv / 4, lpe = H * dv4;
     const bool pow2 = (dv4 & (dv4 - 1)) == 0 && (H & (H - 1)) == 0;
-    if (Dk == Dv && Dv % 4 == 0 && pow2 && lpe >= 1 && lpe <= 64) {
-        fused_dpa_fwd_stream_kernel<<<(int)N, DPA_WPQ * WAVE, 0, st>>>(p, (int)dv4, (int)lpe);
+    const bool fits32 = (E + 1) * H * Dv * 4 < (1ll << 32) && (N + 1) * H * Dv * 4 < (1ll << 32);
+    if (Dk == Dv && Dv % 4 == 0 && pow2 && lpe >= 1 && lpe <= 64 && dv4 <= 16 && fits32) {
+        launch_fwd_stream(p, (int)dv4, (int)lpe, st);
         CF_CHECK_LAUNCH("cf_fused_dpa_fwd");
         return CF_OK;
     }
@@ -545,11 +672,10 @@ extern "C" int cf_fused_dpa_bwd(const float *que, const float *key, const float 
     {
         const int64_t dv4 = Dv / 4, lpe = H * dv4;
         const bool pow2 = (dv4 & (dv4 - 1)) == 0 && (H & (H - 1)) == 0;
-        if (Dk == Dv && Dv % 4 == 0 && pow2 && lpe >= 1 && lpe <= 64) {
-            fused_dpa_bwd_query_stream_kernel<<<(int)N, DPA_WPQ * WAVE, 0, st>>>(p, (int)dv4, (int)lpe);
-            CF_CHECK_LAUNCH("cf_fused_dpa_bwd: query side");
-            fused_dpa_bwd_key_stream_kernel<<<(int)N, DPA_WPQ * WAVE, 0, st>>>(p, (int)dv4, (int)lpe);
-            CF_CHECK_LAUNCH("cf_fused_dpa_bwd: key side");
+        const bool fits32 = (E + 1) * H * Dv * 4 < (1ll << 32) && (N + 1) * H * Dv * 4 < (1ll << 32);
+        if (Dk == Dv && Dv % 4 == 0 && pow2 && lpe >= 1 && lpe <= 64 && dv4 <= 16 && fits32) {
+            launch_bwd_stream(p, (int)dv4, (int)lpe, st);
+            CF_CHECK_LAUNCH("cf_fused_dpa_bwd: streaming kernels");
             return CF_OK;
         }
     }
