@@ -22,6 +22,9 @@ constexpr int MAX_RANGE = 64;
 void set_error(const char *fmt, ...);
 int hip_failed(hipError_t err, const char *what);
 int device_cu_count();
+// Work-groups a persistent kernel may launch at `per_cu` per CU, scaled by the calling
+// thread's launch share (cf_set_launch_share).
+int persistent_grid_cap(int per_cu);
 
 // real_enc_mfma.hip
 int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,

@@ -38,9 +38,27 @@ int device_cu_count()
     return cached_cus;
 }
 
+static thread_local double g_launch_share = 1.0;
+
+int persistent_grid_cap(int per_cu)
+{
+    const int64_t cap = (int64_t)((double)device_cu_count() * per_cu * g_launch_share);
+    return (int)(cap < 1 ? 1 : cap);
+}
+
 }  // namespace cf
 
 extern "C" int cf_version(void) { return 100; }
+
+extern "C" int cf_set_launch_share(double share)
+{
+    CF_REQUIRE(share > 0.0 && share <= 1.0, CF_ERR_INVALID_ARGUMENT,
+               "cf_set_launch_share: share %g outside (0, 1]", share);
+    cf::g_launch_share = share;
+    return CF_OK;
+}
+
+extern "C" double cf_get_launch_share(void) { return cf::g_launch_share; }
 
 extern "C" const char *cf_last_error(void) { return cf::g_error; }
 

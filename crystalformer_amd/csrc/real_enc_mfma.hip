@@ -637,7 +637,7 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     const int64_t rounds = ((U + WPB - 1) / WPB) * p.head_groups;
     if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // round positions are 32-bit in the kernel
     int64_t blocks = rounds;
-    int64_t cap = (int64_t)device_cu_count() * 2;      // 16 waves per CU
+    int64_t cap = persistent_grid_cap(2);              // 16 waves per CU, times the launch share
     if (blocks > cap) blocks = cap;
     if (blocks < 1) return CF_OK;
     // A ticket is drawn three rounds before it is executed (descriptor, then geometry, each

@@ -24,9 +24,15 @@ class GraphedForward:
 
     ``batch`` fixes the layout: later calls may pass a batch with different
     positions, lattices or species but identical ``sizes``.
+
+    ``launch_share`` (0 < share <= 1) is for several graphs replayed concurrently on
+    different streams: the periodic-encoding launches of this graph then take that share
+    of the GPU each (:class:`crystalformer_amd.ops.launch_share`), which lengthens one
+    replay on its own and shortens the steps when several are in flight.
     """
 
-    def __init__(self, model: torch.nn.Module, batch: CrystalBatch, warmup: int = 3):
+    def __init__(self, model: torch.nn.Module, batch: CrystalBatch, warmup: int = 3,
+                 launch_share: float = 1.0):
         if not batch.pos.is_cuda:
             raise ValueError("GraphedForward needs a batch on the GPU")
         self.model = model
@@ -42,7 +48,7 @@ class GraphedForward:
                 model(self.static)
         torch.cuda.current_stream().wait_stream(stream)
         torch.cuda.synchronize()
-        with torch.no_grad(), torch.cuda.graph(self.graph):
+        with torch.no_grad(), ops.launch_share(launch_share), torch.cuda.graph(self.graph):
             self.output = model(self.static)
         # the graph holds raw addresses of the cached index tensors of this layout
         self._keepalive = ops.index_cache_snapshot()

@@ -29,6 +29,8 @@ SIGNATURES = {
     "cf_version": (_int, []),
     "cf_last_error": (ctypes.c_char_p, []),
     "cf_max_translation_range": (_int, []),
+    "cf_set_launch_share": (_int, [_dbl]),
+    "cf_get_launch_share": (_dbl, []),
     "cf_real_enc_fwd": (_int, [_ptr] * 5 + [_i64] * 6 + [_dbl, _dbl, _ptr, _i64, _ptr, _dbl, _int, _int,
                                                          _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
     "cf_real_enc_bwd_workspace": (_i64, [_i64] * 6 + [_int]),

@@ -46,6 +46,27 @@ def count_translation_evals(a_ik: Tensor, rvlen_n: Optional[Tensor], batch_i: Te
     return float(T[edge_ij_e[0]].sum().item())
 
 
+class launch_share:
+    """Context manager: within it, forward launches of the periodic encoding made by this
+    thread occupy at most ``share`` of the GPU (``cf_set_launch_share``), so that kernels of
+    other streams run beside them.  For callers that keep several forwards in flight; a
+    graph captured inside keeps the share.  Results do not depend on it."""
+
+    def __init__(self, share: float):
+        self.share = float(share)
+        self.previous = 1.0
+
+    def __enter__(self):
+        lib = _lib.load()
+        self.previous = float(lib.cf_get_launch_share())
+        check(lib.cf_set_launch_share(self.share), "cf_set_launch_share")
+        return self
+
+    def __exit__(self, *exc):
+        check(_lib.load().cf_set_launch_share(self.previous), "cf_set_launch_share")
+        return False
+
+
 class _timed:
     def __init__(self, name: str, **info):
         self.name, self.info = name, info

@@ -40,6 +40,20 @@ const char *cf_last_error(void);
 int cf_max_translation_range(void);
 
 /*
+ * Share of the GPU that one forward launch of the periodic encoding may occupy, for the
+ * calling thread (default 1).  The forward pair kernel is persistent: it launches two
+ * work-groups per CU, which hold the CU's whole register file, so kernels of other streams
+ * wait for it to drain.  A caller that keeps several streams busy (several forwards in
+ * flight) sets a share below 1: the kernel launches that fraction of its work-groups, runs
+ * longer on its own, and leaves room beside it; results are bit-identical.  Read at launch
+ * (a captured graph keeps the share it was captured with).  The backward kernel ignores
+ * it.  No counterpart in the reference, whose launches are sized by the problem alone
+ * (models/cuda_funcs/real_space_enc_proj.py:75-96).
+ */
+int cf_set_launch_share(double share);
+double cf_get_launch_share(void);
+
+/*
  * Real-space periodic encoding, forward.
  * Replaces the launches of real_enc_fwd / real_enc_proj_fwd
  * (models/cuda_funcs/real_space_enc.py:96-113,

@@ -73,6 +73,30 @@ def test_argument_validation_needs_no_device():
     assert L.cf_real_enc_bwd_workspace(10, 8, 100, 64, 16, 1, 1) >= 100 * 8 * 4 + 100 * 8 * 64 * 4
 
 
+def test_launch_share_is_validated_and_per_thread():
+    import threading
+    from crystalformer_amd import ops
+    L = lib.load()
+    assert L.cf_get_launch_share() == 1.0
+    for bad in (0.0, -0.5, 1.5, float("nan")):
+        assert L.cf_set_launch_share(bad) == -1 and b"share" in L.cf_last_error()
+        assert L.cf_get_launch_share() == 1.0
+    seen = []
+    with ops.launch_share(0.25):
+        assert L.cf_get_launch_share() == 0.25
+        t = threading.Thread(target=lambda: seen.append(L.cf_get_launch_share()))
+        t.start()
+        t.join()
+        with ops.launch_share(0.5):
+            assert L.cf_get_launch_share() == 0.5
+        assert L.cf_get_launch_share() == 0.25
+    assert L.cf_get_launch_share() == 1.0 and seen == [1.0]
+    with pytest.raises(lib.CrystalformerHipError):
+        with ops.launch_share(2.0):
+            pass
+    assert L.cf_get_launch_share() == 1.0
+
+
 def test_operators_refuse_cpu_tensors():
     a = torch.zeros(2, 8)
     with pytest.raises(lib.CrystalformerHipError, match="no CPU fallback"):

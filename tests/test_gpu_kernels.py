@@ -529,6 +529,23 @@ def test_real_enc_fwd_ticket_rounds_are_bit_identical(dev, sizes, H):
     assert_close(v1.cpu()[sel], sub_v, "v sample")
 
 
+@pytest.mark.parametrize("share", [0.6875, 0.25, 1.0 / 512])
+def test_real_enc_fwd_launch_share_changes_no_bit(dev, share):
+    """A launch that takes part of the GPU (fewer work-groups, more rounds each) gives the same
+    bits, with the fixed stride and with the shared-counter scheduling; the share is restored."""
+    for sizes, K, D in (([40, 3, 64, 17], 64, 16), ([256, 256], 16, 8)):
+        p = Problem(sizes, H=8, K=K, D=D, seed=43)
+        a, rpos, tv, bt, ed, W, rv = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.W, p.rvlen)
+        for cutoff in (0.0, -3.5):
+            z0, v0 = ops.real_enc_fwd(a, rpos, tv, bt, ed, K, p.dist_max, 1.0, W, rv, cutoff, 1, 0)
+            with ops.launch_share(share):
+                z1, v1 = ops.real_enc_fwd(a, rpos, tv, bt, ed, K, p.dist_max, 1.0, W, rv, cutoff, 1, 0)
+            assert torch.equal(z0, z1) and torch.equal(v0, v1)
+            assert ops._scheduling_words(dev).tolist() == [0, 0]
+    from crystalformer_amd import lib
+    assert lib.load().cf_get_launch_share() == 1.0
+
+
 @pytest.mark.parametrize("N,C", [(1774, 128), (1774, 512), (5, 3), (100, 384), (0, 7)])
 def test_column_sum(dev, N, C):
     g = torch.randn(N, C, generator=torch.Generator().manual_seed(N + C))
