@@ -1,6 +1,6 @@
 """HIP-graph replay of a fixed-shape forward.
 
-The model's forward issues ~170 small launches per step; for a batch layout
+The model's forward issues about 40 launches per step; for a batch layout
 that repeats (same crystal sizes, hence same N and E) the whole step is
 captured once into a HIP graph and replayed with a single submission.  Inputs
 live in static buffers that :meth:`GraphedForward.__call__` refreshes in place.
