@@ -241,13 +241,34 @@ __global__ __launch_bounds__(GE_THREADS) void gauss_exponents_bwd_kernel(GaussBw
     const float *wr = p.w + h * p.D;
     for (int64_t d0 = 0; d0 < p.D; d0 += 16) {
         const int nd = (int)min((int64_t)16, p.D - d0);
-        for (int d = 0; d < nd; d++) {
-            const float qv = live ? qr[d0 + d] : 0.f;
-            prod[threadIdx.x][d] = g_alpha * qv;
-            if (live && p.gq) {
-                float g = g_alpha * wr[d0 + d];
-                if (p.gqs) g += p.gqs[t * p.D + d0 + d] * p.q_scale;
-                p.gq[t * p.D + d0 + d] = g;
+        if ((p.D & 3) == 0) {
+            // rows are 16-byte aligned: four components per load and store
+            typedef float float4_t __attribute__((ext_vector_type(4)));
+            const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+            float4_t qv[4], wv[4], sv[4];
+#pragma unroll
+            for (int c4 = 0; c4 < 4; c4++) {
+                const bool on = live && 4 * c4 < nd;
+                qv[c4] = on ? *reinterpret_cast<const float4_t *>(qr + d0 + 4 * c4) : zero4;
+                wv[c4] = on && p.gq ? *reinterpret_cast<const float4_t *>(wr + d0 + 4 * c4) : zero4;
+                sv[c4] = on && p.gq && p.gqs ? *reinterpret_cast<const float4_t *>(p.gqs + t * p.D + d0 + 4 * c4) : zero4;
+            }
+#pragma unroll
+            for (int c4 = 0; c4 < 4; c4++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) prod[threadIdx.x][4 * c4 + r] = g_alpha * qv[c4][r];
+                if (live && p.gq && 4 * c4 < nd)
+                    *reinterpret_cast<float4_t *>(p.gq + t * p.D + d0 + 4 * c4) = wv[c4] * g_alpha + sv[c4] * p.q_scale;
+            }
+        } else {
+            for (int d = 0; d < nd; d++) {
+                const float qv = live ? qr[d0 + d] : 0.f;
+                prod[threadIdx.x][d] = g_alpha * qv;
+                if (live && p.gq) {
+                    float g = g_alpha * wr[d0 + d];
+                    if (p.gqs) g += p.gqs[t * p.D + d0 + d] * p.q_scale;
+                    p.gq[t * p.D + d0 + d] = g;
+                }
             }
         }
         __syncthreads();

@@ -413,6 +413,17 @@ __global__ __launch_bounds__(256) void gw_blocks_reduce_kernel(const float *part
     float acc0 = 0.f, acc1 = 0.f;
     if (x < HDK) {
         int b = pt;
+        // 8 loads in flight per thread; the two running sums take alternate blocks as before
+        for (; b + 56 < blocks; b += 64) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = part[(int64_t)(b + 8 * u) * HDK + x];
+#pragma unroll
+            for (int u = 0; u < 8; u += 2) {
+                acc0 += v[u];
+                acc1 += v[u + 1];
+            }
+        }
         for (; b + 8 < blocks; b += 16) {
             acc0 += part[(int64_t)b * HDK + x];
             acc1 += part[(int64_t)(b + 8) * HDK + x];
