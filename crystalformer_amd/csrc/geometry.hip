@@ -296,6 +296,17 @@ __global__ __launch_bounds__(256) void gauss_exponents_bwd_reduce_kernel(const f
     if (x >= hd) return;
     float s0 = 0.f, s1 = 0.f;
     int b = 0;
+    // 8 loads in flight; even blocks go to one running sum, odd blocks to the other
+    for (; b + 7 < blocks; b += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = part[(int64_t)(b + u) * hd + x];
+#pragma unroll
+        for (int u = 0; u < 8; u += 2) {
+            s0 += v[u];
+            s1 += v[u + 1];
+        }
+    }
     for (; b + 1 < blocks; b += 2) {
         s0 += part[(int64_t)b * hd + x];
         s1 += part[(int64_t)(b + 1) * hd + x];

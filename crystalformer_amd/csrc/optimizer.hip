@@ -6,18 +6,19 @@
 //
 // Tensors are handed over by value in the kernel arguments, ADAM_GROUP at a time; a
 // work-group owns one ADAM_CHUNK-element chunk of one tensor and finds it by scanning the
-// group's chunk prefix (a scalar loop over at most ADAM_GROUP entries).
+// group's chunk prefix (a scalar loop over at most ADAM_GROUP entries).  The model of the
+// benchmark has 58 parameter tensors: one launch of each kind.
 #include "cf_common.h"
 
 namespace {
 
 using namespace cf;
 
-constexpr int ADAM_GROUP = 24;      // tensors per launch (kernel-argument table)
+constexpr int ADAM_GROUP = 64;      // tensors per launch (kernel-argument table: 44 bytes each of the 4 KB)
 constexpr int ADAM_CHUNK = 2048;    // elements per work-group: 256 threads x 8
 constexpr int ADAM_THREADS = 256;
 
-struct AdamGroup {
+struct AdamGroup {                    // passed by value: has to fit the 4 KB of kernel arguments
     float *p[ADAM_GROUP];
     const float *g[ADAM_GROUP];
     float *m[ADAM_GROUP];
@@ -33,6 +34,7 @@ struct AdamGroup {
     float *state;                    // [0] steps taken (counted as float), [1] gradient norm, [2] lr used
     float lr0, sch_decay, beta1, beta2, eps, clip_norm;
 };
+static_assert(sizeof(AdamGroup) <= 4096, "AdamGroup must fit the kernel-argument segment");
 
 __device__ __forceinline__ float block_sum(float v, float *lds)
 {

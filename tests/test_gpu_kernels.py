@@ -589,11 +589,11 @@ def test_linear_weight_grad(dev, N, C, K):
 def test_fused_adamw_follows_torch(dev, clip):
     """clip + AdamW + inverse square-root schedule in one device-side update against
     torch.nn.utils.clip_grad_norm_ + torch.optim.AdamW + LambdaLR (the reference's training
-    step, models/regression.py:106-135, :254-269) on 30 tensors of ragged sizes (more than
-    one kernel-argument group, chunks with tails, a single-element tensor)."""
+    step, models/regression.py:106-135, :254-269) on 70 tensors of ragged sizes (more than
+    one kernel-argument group of 64, chunks with tails, a single-element tensor)."""
     from crystalformer_amd.training import FusedAdamW, make_optimizer
     gen = torch.Generator().manual_seed(11)
-    sizes = [1, 7, 128, 2048, 2049, 5000, 128 * 128, 512 * 128] + [100 + 37 * k for k in range(22)]
+    sizes = [1, 7, 128, 2048, 2049, 5000, 128 * 128, 512 * 128] + [100 + 37 * k for k in range(62)]
 
     class Bag(torch.nn.Module):
         def __init__(self):
