@@ -108,7 +108,10 @@ class Latticeformer(nn.Module):
         self.mlp = nn.Sequential(*layers)
 
     def forward(self, data):
-        x = self.input_embeddings(data.x)
+        # (inside a fused training step the embedding's and the head's weight gradients join the
+        # grouped weight-gradient launch; otherwise these are the stock linear ops)
+        from . import hip_funcs
+        x = hip_funcs.linear(data.x, self.input_embeddings.weight, self.input_embeddings.bias)
         x = self.encoder(x, data.pos, data.batch, data.trans_vec, data.sizes, data.x)
         x = self.proj_before_pooling(x)
         x = self.pooling_layer(x, data.batch, data.sizes)
@@ -122,7 +125,10 @@ class Latticeformer(nn.Module):
         mods = list(self.mlp)
         plain = all(isinstance(m, (nn.Linear, nn.ReLU, nn.Identity)) for m in mods)
         if not (plain and x.is_cuda and inference_only(x, self.mlp.parameters)):
-            return self.mlp(x)
+            from . import hip_funcs
+            for m in mods:
+                x = hip_funcs.linear(x, m.weight, m.bias) if isinstance(m, nn.Linear) else m(x)
+            return x
         i = 0
         while i < len(mods):
             m = mods[i]
