@@ -123,6 +123,24 @@ __global__ __launch_bounds__(ADAM_THREADS) void adamw_update_kernel(AdamGroup a)
 
 int64_t chunks_of(int64_t n) { return (n + ADAM_CHUNK - 1) / ADAM_CHUNK; }
 
+// Mean absolute error over the batch, summed over the targets, and its gradient, in one
+// work-group: loss = (1/B) sum_b sum_i |pred[b,i] - target[b,i]|, grad = sign(pred - target) / B.
+// Each thread adds its elements in ascending order, the threads are added in a fixed order.
+__global__ __launch_bounds__(ADAM_THREADS) void l1_mean_loss_kernel(const float *pred, const float *target, int64_t B,
+                                                                    int64_t total, float *loss, float *grad)
+{
+    __shared__ float lds[4];
+    const float inv = 1.0f / (float)B;
+    float s = 0.f;
+    for (int64_t x = threadIdx.x; x < total; x += ADAM_THREADS) {
+        const float d = pred[x] - target[x];
+        s += fabsf(d);
+        if (grad) grad[x] = d > 0.f ? inv : (d < 0.f ? -inv : 0.f);
+    }
+    s = block_sum(s, lds);
+    if (threadIdx.x == 0) loss[0] = s * inv;
+}
+
 }  // namespace
 
 extern "C" int64_t cf_adamw_step_workspace(int n_tensors, const int64_t *numel)
@@ -200,5 +218,16 @@ extern "C" int cf_adamw_step(int n_tensors, float *const *params, const float *c
             advance = false;
         }
     }
+    return CF_OK;
+}
+
+extern "C" int cf_l1_mean_loss(const float *pred, const float *target, int64_t B, int64_t T, float *loss, float *grad,
+                               void *stream)
+{
+    CF_REQUIRE(B >= 1 && T >= 1 && B * T < (1ll << 40), CF_ERR_INVALID_ARGUMENT, "cf_l1_mean_loss: bad sizes B=%lld T=%lld",
+               (long long)B, (long long)T);
+    CF_REQUIRE(pred && target && loss, CF_ERR_INVALID_ARGUMENT, "cf_l1_mean_loss: null pointer");
+    l1_mean_loss_kernel<<<1, ADAM_THREADS, 0, (hipStream_t)stream>>>(pred, target, B, B * T, loss, grad);
+    CF_CHECK_LAUNCH("cf_l1_mean_loss");
     return CF_OK;
 }

@@ -507,6 +507,24 @@ def linear(x: Tensor, weight: Tensor, bias: Optional[Tensor]) -> Tensor:
     return torch.nn.functional.linear(x, weight, bias)
 
 
+class L1MeanLossHIP(torch.autograd.Function):
+    """Scalar training loss ``mean_b sum_i |pred[b,i] - target[b,i]|`` (the reference's
+    ``regression_loss(..., "l1").mean()``, losses/regression_loss.py:10-20 and
+    models/regression.py:117-118) with its gradient computed by the same launch, where the
+    stock ops take about ten launches forward and backward."""
+
+    @staticmethod
+    def forward(ctx, pred: Tensor, target: Tensor):
+        loss, grad = ops.l1_mean_loss(pred.detach(), target.detach(), with_grad=ctx.needs_input_grad[0])
+        ctx.save_for_backward(grad)
+        return loss.reshape(())
+
+    @staticmethod
+    def backward(ctx, gloss):
+        grad, = ctx.saved_tensors
+        return (grad * gloss if grad is not None else None), None
+
+
 class IrregularMeanCUDA(torch.autograd.Function):
     """Per-crystal mean over atoms with a fixed summation order."""
 

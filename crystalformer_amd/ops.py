@@ -874,3 +874,20 @@ def adamw_step(plan: AdamWPlan, grads, lr0: float, sch_decay: float, beta1: floa
                                        beta1, beta2, eps, clip_norm, ptr(state), ptr(plan.ws), plan.ws_bytes,
                                        stream_handle(dev))
     check(rc, "cf_adamw_step")
+
+
+def l1_mean_loss(pred: Tensor, target: Tensor, with_grad: bool = True):
+    """``(loss, grad)``: the L1 losses of a batch summed over the targets and averaged over the
+    batch (one float on the device), and ``sign(pred - target) / B`` (None without
+    ``with_grad``), in one launch.  ``pred`` and ``target`` are (B, T)."""
+    dev = require_device(pred, target)
+    pred, target = _f32(pred, "pred"), _f32(target, "target")
+    if pred.dim() != 2 or target.shape != pred.shape or pred.shape[0] < 1 or pred.shape[1] < 1:
+        raise _lib.CrystalformerHipError("l1_mean_loss: pred and target must both be (B, T), B and T at least 1")
+    B, T = pred.shape
+    loss = torch.empty(1, dtype=torch.float32, device=dev)
+    grad = torch.empty_like(pred) if with_grad else None
+    with device_guard(dev):
+        rc = _lib.load().cf_l1_mean_loss(ptr(pred), ptr(target), B, T, ptr(loss), ptr(grad), stream_handle(dev))
+    check(rc, "cf_l1_mean_loss")
+    return loss, grad

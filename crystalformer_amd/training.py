@@ -119,7 +119,10 @@ def fused_training_step(model: nn.Module, batch, opt: "FusedAdamW", zero_grad: b
     hip_funcs.USE_LINEAR_FUNCTION = True
     try:
         out = model(batch)
-        loss = F.l1_loss(out[:, 0], batch.y, reduction="none").mean()
+        if out.shape[1] == 1:
+            loss = hip_funcs.L1MeanLossHIP.apply(out, batch.y.reshape(-1, 1))   # loss and its gradient in one launch
+        else:
+            loss = F.l1_loss(out[:, 0], batch.y, reduction="none").mean()
         with hip_funcs.deferred_weight_grads():           # all linear layers' weight gradients at the end
             loss.backward()
     finally:

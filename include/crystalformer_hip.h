@@ -383,7 +383,7 @@ int cf_linear_weight_grad_grouped(int n_layers, const float *const *g, const flo
  * gradient-norm clip (nn.utils.clip_grad_norm_, models/regression.py:122), AdamW
  * (optim.AdamW, models/regression.py:254; decoupled weight decay per tensor, betas, eps)
  * and the schedule lr0 * sqrt(sch_decay / (sch_decay + t)) of models/regression.py:269
- * (sch_decay <= 0: constant lr0), in 2 * ceil(n_tensors / 24) launches.
+ * (sch_decay <= 0: constant lr0), in 2 * ceil(n_tensors / 64) launches.
  *   params, grads, exp_avg, exp_avg_sq: HOST arrays of n_tensors device pointers (read at
  *       call time and passed to the kernels by value; the device memory they name is read
  *       and written when the kernels run)
@@ -399,6 +399,16 @@ int cf_adamw_step(int n_tensors, float *const *params, const float *const *grads
                   float *const *exp_avg_sq, const int64_t *numel, const float *weight_decay, float lr0,
                   float sch_decay, float beta1, float beta2, float eps, float clip_norm, float *state_3,
                   void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * Training loss of the regression module and its gradient in one launch: the per-sample
+ * L1 losses summed over the targets (losses/regression_loss.py:10-20 with loss_fn "l1"),
+ * averaged over the batch (models/regression.py:117-118).
+ *   pred, target: (B, T) row-major; loss: (1); grad: (B, T) = sign(pred - target) / B, or NULL
+ * One work-group, fixed summation order.
+ */
+int cf_l1_mean_loss(const float *pred, const float *target, int64_t B, int64_t T, float *loss, float *grad,
+                    void *stream);
 
 #ifdef __cplusplus
 }

@@ -348,3 +348,13 @@ def avr_pool(x: Tensor, sizes: Sequence[int]) -> Tensor:
     if torch.is_tensor(sizes):
         sizes = sizes.tolist()
     return torch.stack([torch.mean(c, dim=0) for c in torch.split_with_sizes(x, sizes, 0)])
+
+
+def l1_training_loss(pred: Tensor, target: Tensor) -> Tensor:
+    """Scalar training loss: per-sample L1 losses summed over the target columns
+    (losses/regression_loss.py:17-20, loss_fn "l1"), then the mean over the batch
+    (models/regression.py:117-118).  ``pred`` and ``target`` are (B, T)."""
+    loss = 0
+    for i in range(pred.shape[1]):
+        loss = loss + F.l1_loss(pred[:, i], target[:, i], reduction="none")
+    return loss.mean()

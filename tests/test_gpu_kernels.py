@@ -6,7 +6,7 @@ import math
 import pytest
 import torch
 
-from crystalformer_amd import lib, ops
+from crystalformer_amd import hip_funcs, lib, ops
 from oracle import kernel_semantics as ks
 from oracle import torch_path as tp
 from tests.helpers import Problem, assert_close, make_sized_batch, rel_err, to_dev
@@ -627,6 +627,31 @@ def test_fused_adamw_follows_torch(dev, clip):
     with pytest.raises(Exception):
         next(iter(mine.parameters())).grad = None
         fused.step()
+
+
+@pytest.mark.parametrize("B,T", [(128, 1), (1, 1), (1000, 3), (257, 2)])
+def test_l1_mean_loss_and_its_gradient(dev, B, T):
+    """Loss and gradient of one launch against the reference's loss (restated in the oracle) and
+    autograd; exact ties get a zero gradient, like torch's sign."""
+    from oracle import torch_path as tp
+    gen = torch.Generator().manual_seed(17)
+    pred = torch.randn(B, T, generator=gen)
+    target = torch.randn(B, T, generator=gen)
+    target[::7] = pred[::7]                                   # ties
+    ref_in = pred.clone().requires_grad_()
+    ref = tp.l1_training_loss(ref_in, target)
+    (ref * 3.0).backward()
+    loss, grad = ops.l1_mean_loss(pred.to(dev), target.to(dev))
+    ref_value = float(ref.detach())
+    assert abs(float(loss) - ref_value) <= 2e-6 * abs(ref_value) + 1e-12
+    assert torch.equal(grad.cpu() * 3.0, ref_in.grad) or float((grad.cpu() * 3.0 - ref_in.grad).abs().max()) < 1e-9
+    mine_in = pred.to(dev).requires_grad_()
+    out = hip_funcs.L1MeanLossHIP.apply(mine_in, target.to(dev))
+    assert out.dim() == 0
+    (out * 3.0).backward()
+    assert float((mine_in.grad.cpu() - ref_in.grad).abs().max()) < 1e-9
+    loss_only, none = ops.l1_mean_loss(pred.to(dev), target.to(dev), with_grad=False)
+    assert none is None and float(loss_only) == float(loss)
 
 
 @pytest.mark.parametrize("func", ["elu", "abs", "exp"])
