@@ -7,7 +7,7 @@
 // Tensors are handed over by value in the kernel arguments, ADAM_GROUP at a time; a
 // work-group owns one ADAM_CHUNK-element chunk of one tensor and finds it by scanning the
 // group's chunk prefix (a scalar loop over at most ADAM_GROUP entries).  The model of the
-// benchmark has 58 parameter tensors: one launch of each kind.
+// benchmark has 53 parameter tensors: one launch of each kind.
 #include "cf_common.h"
 
 namespace {
