@@ -40,7 +40,7 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
                               const float *gz, const float *gv, int64_t N, int64_t H, int64_t E, int64_t K,
                               int64_t D, float bin_step, float s_scale, const float *W, const float *rvlen,
                               float cutoff, int lattice_range, int min_range, float *ga_edge,
-                              float *gW_part, float *gW, hipStream_t st);
+                              float *gW_part, float *gW, const int64_t *e_start, float *ga_ik, hipStream_t st);
 
 #define CF_REQUIRE(cond, code, ...)            \
     do {                                       \

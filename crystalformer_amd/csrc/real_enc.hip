@@ -938,12 +938,9 @@ extern "C" int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const 
         }
         rc = launch_real_enc_bwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, z_ek, gz_ek,
                                        gv_ekd, N, H, E, K, D, p.bin_step, p.s_scale, W_k, rvlen_n, p.cutoff,
-                                       lattice_range, minimum_range, ga_edge, gW_part, gW_k, st);
+                                       lattice_range, minimum_range, ga_edge, gW_part, gW_k, e_start_i, ga_ik, st);
         if (rc == CF_OK) {
-            CF_CHECK_LAUNCH("cf_real_enc_bwd (pairs)");
-            int64_t total = N * H;
-            reduce_ga_kernel<<<(int)((total + 255) / 256), 256, 0, st>>>(ga_edge, e_start_i, N, (int)H, ga_ik);
-            CF_CHECK_LAUNCH("cf_real_enc_bwd: reduce_ga");
+            CF_CHECK_LAUNCH("cf_real_enc_bwd (pairs)");     // the pair kernel and its two reductions
             return CF_OK;
         }
         if (rc != CF_ERR_UNSUPPORTED) return rc;

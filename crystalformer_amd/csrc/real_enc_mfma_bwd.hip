@@ -401,19 +401,42 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     if (wa_hg >= 0) flush_gW(wa_hg);
 }
 
+// The two reductions behind the pair kernel in one launch (they are independent, and a launch
+// costs more than either): work-groups below gw_groups fold the per-work-group partial weight
+// gradients, the others fold the per-edge exponent gradients into per-atom ones.
+//
 // gW[x] = sum over work-groups of part[b][x], fixed order.  A work-group of 256 threads takes
 // 32 consecutive elements; 8 groups of threads each sum every 8th block (two running sums),
 // and the 8 partial results are added in order through LDS.
-__global__ __launch_bounds__(256) void gw_blocks_reduce_kernel(const float *part, int blocks, int64_t HDK,
-                                                               float *gW)
+//
+// ga[i,h] = sum over the edge row of atom i of ga_edge[e,h]: one thread per (i,h), eight
+// running sums over the row in order.
+__global__ __launch_bounds__(256) void bwd_reductions_kernel(const float *part, int blocks, int64_t HDK, float *gW,
+                                                             int gw_groups, const float *ga_edge,
+                                                             const int64_t *e_start, int64_t N, int H, float *ga)
 {
     __shared__ float red[8][32];
+    if ((int)blockIdx.x >= gw_groups) {
+        const int64_t tid = (int64_t)(blockIdx.x - gw_groups) * 256 + threadIdx.x;
+        if (tid >= N * H) return;
+        const int64_t i = tid / H;
+        const int h = (int)(tid - i * H);
+        const int64_t e0 = e_start[i], e1 = e_start[i + 1];
+        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        int64_t e = e0;
+        for (; e + 8 <= e1; e += 8)
+#pragma unroll
+            for (int u = 0; u < 8; u++) acc[u] += ga_edge[(e + u) * H + h];
+        for (int u = 0; e < e1; e++, u++) acc[u] += ga_edge[e * H + h];
+        ga[tid] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+        return;
+    }
     const int ex = threadIdx.x & 31, pt = threadIdx.x >> 5;
     const int64_t x = (int64_t)blockIdx.x * 32 + ex;
     float acc0 = 0.f, acc1 = 0.f;
     if (x < HDK) {
         int b = pt;
-        // 8 loads in flight per thread; the two running sums take alternate blocks as before
+        // 8 loads in flight per thread; the two running sums take alternate blocks
         for (; b + 56 < blocks; b += 64) {
             float v[8];
 #pragma unroll
@@ -459,7 +482,7 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
                               const float *gz, const float *gv, int64_t N, int64_t H, int64_t E, int64_t K,
                               int64_t D, float bin_step, float s_scale, const float *W, const float *rvlen,
                               float cutoff, int lattice_range, int min_range, float *ga_edge,
-                              float *gW_part, float *gW, hipStream_t st)
+                              float *gW_part, float *gW, const int64_t *e_start, float *ga_ik, hipStream_t st)
 {
     if (K < 1 || K > 64 || !W || D < 1 || D > 16) return CF_ERR_UNSUPPORTED;
     PairArgs p{};
@@ -489,9 +512,12 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
         default: CF_BPAIR(4); break;
     }
 #undef CF_BPAIR
-    if (gW_part && gW) {
-        const int64_t HDK = H * D * K;
-        gw_blocks_reduce_kernel<<<(int)((HDK + 31) / 32), 256, 0, st>>>(gW_part, blocks, HDK, gW);
+    {
+        const int64_t HDK = (gW_part && gW) ? H * D * K : 0;
+        const int gw_groups = (int)((HDK + 31) / 32);
+        const int64_t ga_groups = (N * H + 255) / 256;
+        bwd_reductions_kernel<<<(int)(gw_groups + ga_groups), 256, 0, st>>>(gW_part, blocks, HDK, gW, gw_groups, ga_edge,
+                                                                            e_start, N, (int)H, ga_ik);
     }
     return CF_OK;
 }
