@@ -143,75 +143,83 @@ struct LinNNArgs {
     int C, K, terms;
 };
 
+// TM x TN outputs per work-group (64 or 32 each), 2 x 2 wavefronts of TM/2 x TN/2.
+template <int TM, int TN>
 __global__ __launch_bounds__(256) void linear_rows_nn_kernel(LinNNArgs p)
 {
-    __shared__ __align__(16) float gs[NN_T * NN_GLD];
-    __shared__ __align__(16) float ws[NN_KC * NN_WLD];
+    constexpr int MT = TM / 32, NTL = TN / 32;                  // 16 x 16 tiles per wavefront
+    constexpr int WLD = TN + 4;                                  // as NN_WLD for the 64-wide tile
+    constexpr int GP = TM / 16;                                  // staging passes of the G tile (16 rows each)
+    constexpr int WPR = TN / 4, WROWS = 256 / WPR, WP = NN_KC / WROWS;   // W tile: pieces per row, rows per pass, passes
+    __shared__ __align__(16) float gs[TM * NN_GLD];
+    __shared__ __align__(16) float ws[NN_KC * WLD];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int q = lane >> 4, c = lane & 15;
     const int wr = wave >> 1, wc = wave & 1;
-    const int64_t row0 = (int64_t)blockIdx.x * NN_T;
-    const int col0 = blockIdx.y * NN_T;
-    // staging role for both tiles (64 rows x 64 floats): thread -> row t / 16 (+16 u), piece t % 16
+    const int64_t row0 = (int64_t)blockIdx.x * TM;
+    const int col0 = blockIdx.y * TN;
+    // staging roles: G tile (TM rows x 64 floats): row t / 16 (+16 u), piece t % 16;
+    // W tile (64 rows x TN floats): row t / WPR (+WROWS u), piece t % WPR
     const int srow = threadIdx.x >> 4, spiece = threadIdx.x & 15;
-    int64_t grow[4];
+    const int wrow = threadIdx.x / WPR, wpiece = threadIdx.x % WPR;
+    int64_t grow[GP];
 #pragma unroll
-    for (int u = 0; u < 4; u++) grow[u] = min(row0 + srow + 16 * u, p.N - 1) * p.C + 4 * spiece;
-    const int wcol = min(col0 + 4 * spiece, p.K - 4);            // K is a multiple of 4
+    for (int u = 0; u < GP; u++) grow[u] = min(row0 + srow + 16 * u, p.N - 1) * p.C + 4 * spiece;
+    const int wcol = min(col0 + 4 * wpiece, p.K - 4);           // K is a multiple of 4
 
-    float4_t acc[2][2];
+    float4_t acc[MT][NTL];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MT; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < NTL; j++) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
     const int chunks = p.C / NN_KC;                              // C is a multiple of 64
     const int steps = p.terms * chunks;
-    // Two register sets, each fetched two chunks ahead: a work-group is alone on its CU for these
-    // shapes (one wavefront per SIMD), so nothing else hides the latency of the loads.
-    float4_t gr[2][4], wg[2][4];
+    // Two register sets, each fetched two chunks ahead: few wavefronts share a SIMD for these
+    // shapes, so nothing else hides the latency of the loads.
+    float4_t gr[2][GP], wg[2][WP];
     auto fetch = [&](int step, float4_t *gdst, float4_t *wdst) {
         if (step >= steps) return;
         const int term = step / chunks, k0 = (step - term * chunks) * NN_KC;
-        const float *g = p.g[term] + k0, *w = p.w[term] + (int64_t)(k0 + srow) * p.K + wcol;
+        const float *g = p.g[term] + k0, *w = p.w[term] + (int64_t)(k0 + wrow) * p.K + wcol;
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            gdst[u] = *reinterpret_cast<const float4_t *>(g + grow[u]);
-            wdst[u] = *reinterpret_cast<const float4_t *>(w + (int64_t)(16 * u) * p.K);
-        }
+        for (int u = 0; u < GP; u++) gdst[u] = *reinterpret_cast<const float4_t *>(g + grow[u]);
+#pragma unroll
+        for (int u = 0; u < WP; u++) wdst[u] = *reinterpret_cast<const float4_t *>(w + (int64_t)(WROWS * u) * p.K);
     };
     auto chunk = [&](int step, float4_t *gset, float4_t *wset) {
         __syncthreads();                                         // previous chunk fully consumed
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < GP; u++)
             *reinterpret_cast<float4_t *>(gs + (srow + 16 * u) * NN_GLD + 4 * spiece) = gset[u];
-            *reinterpret_cast<float4_t *>(ws + (srow + 16 * u) * NN_WLD + 4 * spiece) = wset[u];
-        }
+#pragma unroll
+        for (int u = 0; u < WP; u++)
+            *reinterpret_cast<float4_t *>(ws + (wrow + WROWS * u) * WLD + 4 * wpiece) = wset[u];
         __syncthreads();
         fetch(step + 2, gset, wset);                             // in flight during this and the next chunk
-        // all operands of the chunk first (one wait), then the 64 MFMAs: a wavefront is alone on
-        // its SIMD here, so a wait per read would be paid in full
-        float4_t a[NN_KC / 16][2];
-        float b[NN_KC / 16][4][2];
+        // all operands of the chunk first (one wait), then the MFMAs: with one wavefront per SIMD a
+        // wait per read would be paid in full
+        float4_t a[NN_KC / 16][MT];
+        float b[NN_KC / 16][4][NTL];
 #pragma unroll
         for (int ss = 0; ss < NN_KC / 16; ss++) {
 #pragma unroll
-            for (int i = 0; i < 2; i++)
-                a[ss][i] = *reinterpret_cast<const float4_t *>(gs + ((wr * 2 + i) * 16 + c) * NN_GLD + 16 * ss + 4 * q);
+            for (int i = 0; i < MT; i++)
+                a[ss][i] = *reinterpret_cast<const float4_t *>(gs + ((wr * MT + i) * 16 + c) * NN_GLD + 16 * ss + 4 * q);
 #pragma unroll
             for (int r = 0; r < 4; r++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)   // step r reduces over the rows 16 ss + 4 q' + r of the W tile
-                    b[ss][r][j] = ws[(16 * ss + 4 * q + r) * NN_WLD + (wc * 2 + j) * 16 + c];
+                for (int j = 0; j < NTL; j++)   // step r reduces over the rows 16 ss + 4 q' + r of the W tile
+                    b[ss][r][j] = ws[(16 * ss + 4 * q + r) * WLD + (wc * NTL + j) * 16 + c];
         }
 #pragma unroll
         for (int ss = 0; ss < NN_KC / 16; ss++)
 #pragma unroll
             for (int r = 0; r < 4; r++)
 #pragma unroll
-                for (int i = 0; i < 2; i++)
+                for (int i = 0; i < MT; i++)
 #pragma unroll
-                    for (int j = 0; j < 2; j++)
+                    for (int j = 0; j < NTL; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[ss][i][r], b[ss][r][j], acc[i][j], 0, 0, 0);
     };
     fetch(0, gr[0], wg[0]);
@@ -221,14 +229,14 @@ __global__ __launch_bounds__(256) void linear_rows_nn_kernel(LinNNArgs p)
         if (step + 1 < steps) chunk(step + 1, gr[1], wg[1]);
     }
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int col = col0 + (wc * 2 + j) * 16 + c;
+    for (int j = 0; j < NTL; j++) {
+        const int col = col0 + (wc * NTL + j) * 16 + c;
         if (col >= p.K) continue;
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < MT; i++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const int64_t row = row0 + (wr * 2 + i) * 16 + 4 * q + r;
+                const int64_t row = row0 + (wr * MT + i) * 16 + 4 * q + r;
                 if (row >= p.N) continue;
                 float v = acc[i][j][r];
                 if (p.mask && !(p.mask[row * p.K + col] > 0.f)) v = 0.f;
@@ -488,8 +496,14 @@ extern "C" int cf_linear_rows_nn(const float *g0, const float *g1, const float *
     }
     CF_REQUIRE(y, CF_ERR_INVALID_ARGUMENT, "cf_linear_rows_nn: null output");
     p.add = add; p.mask = mask; p.y = y; p.N = N; p.C = (int)C; p.K = (int)K; p.terms = n_terms;
-    dim3 grid((unsigned)((N + NN_T - 1) / NN_T), (unsigned)((K + NN_T - 1) / NN_T));
-    linear_rows_nn_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(p);
+    // quarter tiles while full ones would leave most CUs without a work-group
+    if (((N + 63) / 64) * ((K + 63) / 64) < 128) {
+        dim3 grid((unsigned)((N + 31) / 32), (unsigned)((K + 31) / 32));
+        linear_rows_nn_kernel<32, 32><<<grid, 256, 0, (hipStream_t)stream>>>(p);
+    } else {
+        dim3 grid((unsigned)((N + NN_T - 1) / NN_T), (unsigned)((K + NN_T - 1) / NN_T));
+        linear_rows_nn_kernel<NN_T, NN_T><<<grid, 256, 0, (hipStream_t)stream>>>(p);
+    }
     CF_CHECK_LAUNCH("cf_linear_rows_nn");
     return CF_OK;
 }
