@@ -326,13 +326,13 @@ class LinearRowsHIP(torch.autograd.Function):
 
 
 def input_gradient(gs, weights, add: Optional[Tensor], mask: Optional[Tensor], like: Tensor) -> Tensor:
-    """``mask(sum_i gs[i] @ weights[i]) + add``.  One row-block launch where that replaces
-    several (more than one term, or a mask); a single plain product is left to the library
-    GEMM, which is faster at these sizes (measured at 1774 rows: 5.7 us against 6.8 us for
-    128 -> 128, 8.9 + 4.8 us against 17 us for 512 -> 128 with an addend)."""
+    """``mask(sum_i gs[i] @ weights[i]) + add``: one row-block launch for all terms, the mask and
+    the addend where the shapes allow it (at 1774 rows as fast as the library GEMM for a single
+    plain product -- 3.3 against 4.0 us for 128 -> 128, 6.8 against 6.5 us for 512 -> 128 -- and
+    ahead of it with an addend or several terms), else library GEMMs and element-wise launches."""
     if not gs:
         return add if add is not None else torch.zeros_like(like)
-    if (len(gs) > 1 or mask is not None) and ops.linear_rows_nn_supported(gs[0], weights[0]):
+    if ops.linear_rows_nn_supported(gs[0], weights[0]):
         return ops.linear_rows_nn(gs, weights, add=add.contiguous() if add is not None else None, mask=mask)
     gx = torch.mm(gs[0], weights[0])
     for g, w in zip(gs[1:], weights[1:]):
