@@ -22,21 +22,26 @@ struct LinArgs {
     int K, C, nw, relu;
 };
 
-constexpr int LIN_KC = 32;         // reduction chunk staged in LDS
-constexpr int LIN_LD = LIN_KC + 4; // LDS row stride (floats): 16-byte aligned, staggers the banks
-
-// LDS-tiled: a work-group of 4 wavefronts (WR x WC) owns TM rows x TN columns; every 32-wide
+// LDS-tiled: a work-group of 4 wavefronts (WR x WC) owns TM rows x TN columns; every KC-wide
 // chunk of the reduction is staged once in LDS (X tile and W tile, 16-byte global loads held
 // in registers while the previous chunk is multiplied) and read back as MFMA operands:
 // lane (q, c) = (lane / 16, lane % 16) reads 16 bytes of row c of a 16-row tile at
 // k = 16 s + 4 q, four MFMA steps per read, step r reducing over k = 16 s + 4 q' + r.
-template <int TM, int TN, int WR, int WC>
+// KC = 32 for large problems (many work-groups per CU hide the staging latency); KC = 64 for
+// the few thousand rows of a batch, where a work-group is nearly alone on its CU and every
+// chunk costs a full memory round trip (a 128-wide layer is then two chunks; one chunk of 128
+// is no faster and its 50 KB of LDS keep it from running beside the encoding kernel).
+// The LDS row stride KC + 4 floats keeps the rows 16-byte aligned and staggers the banks.
+template <int TM, int TN, int WR, int WC, int KC>
 __global__ __launch_bounds__(256) void linear_rows_kernel(LinArgs p)
 {
+    constexpr int LD = KC + 4;
     constexpr int MT = TM / (16 * WR), NT = TN / (16 * WC);     // 16 x 16 tiles per wavefront
-    constexpr int XL = TM / 32, WL = TN / 32;                   // 16-byte loads per thread and chunk
-    __shared__ __align__(16) float xs[TM * LIN_LD];
-    __shared__ __align__(16) float ws[TN * LIN_LD];
+    constexpr int PPR = KC / 4, RPP = 256 / PPR;                // 16-byte pieces per tile row, rows per staging pass
+    constexpr int XL = TM / RPP, WL = TN / RPP;                 // 16-byte loads per thread and chunk
+    static_assert(XL >= 1 && WL >= 1, "tile too small for the staging pattern");
+    __shared__ __align__(16) float xs[TM * LD];
+    __shared__ __align__(16) float ws[TN * LD];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int q = lane >> 4, c = lane & 15;
@@ -44,15 +49,15 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(LinArgs p)
     const int64_t row0 = (int64_t)blockIdx.x * TM;
     const int col0 = blockIdx.y * TN;                           // column over all weights
     const int total_cols = p.nw * p.C;
-    // staging role: thread -> (row t/8 (+32 u), 16-byte piece t%8) of a tile
-    const int srow = threadIdx.x >> 3, spiece = threadIdx.x & 7;
+    // staging role: thread -> (row t / PPR (+RPP u), 16-byte piece t % PPR) of a tile
+    const int srow = threadIdx.x / PPR, spiece = threadIdx.x % PPR;
     const float *xg[XL];
     const float *wg[WL];
 #pragma unroll
-    for (int u = 0; u < XL; u++) xg[u] = p.x + min(row0 + srow + 32 * u, p.N - 1) * p.K + 4 * spiece;
+    for (int u = 0; u < XL; u++) xg[u] = p.x + min(row0 + srow + RPP * u, p.N - 1) * p.K + 4 * spiece;
 #pragma unroll
     for (int u = 0; u < WL; u++) {
-        const int col = min(col0 + srow + 32 * u, total_cols - 1);
+        const int col = min(col0 + srow + RPP * u, total_cols - 1);
         const int wi = col / p.C;
         wg[u] = p.w[wi] + (int64_t)(col - wi * p.C) * p.K + 4 * spiece;
     }
@@ -71,25 +76,25 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(LinArgs p)
         for (int u = 0; u < WL; u++) wrg[u] = in ? *reinterpret_cast<const float4_t *>(wg[u] + k0) : zero4;
     };
     fetch(0);
-    for (int k0 = 0; k0 < p.K; k0 += LIN_KC) {
+    for (int k0 = 0; k0 < p.K; k0 += KC) {
         __syncthreads();                                        // previous chunk fully consumed
 #pragma unroll
         for (int u = 0; u < XL; u++)
-            *reinterpret_cast<float4_t *>(xs + (srow + 32 * u) * LIN_LD + 4 * spiece) = xr[u];
+            *reinterpret_cast<float4_t *>(xs + (srow + RPP * u) * LD + 4 * spiece) = xr[u];
 #pragma unroll
         for (int u = 0; u < WL; u++)
-            *reinterpret_cast<float4_t *>(ws + (srow + 32 * u) * LIN_LD + 4 * spiece) = wrg[u];
+            *reinterpret_cast<float4_t *>(ws + (srow + RPP * u) * LD + 4 * spiece) = wrg[u];
         __syncthreads();
-        if (k0 + LIN_KC < p.K) fetch(k0 + LIN_KC);              // in flight during the MFMAs below
+        if (k0 + KC < p.K) fetch(k0 + KC);                      // in flight during the MFMAs below
 #pragma unroll
-        for (int ss = 0; ss < LIN_KC / 16; ss++) {
+        for (int ss = 0; ss < KC / 16; ss++) {
             float4_t a[MT], b[NT];
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
-                a[mt] = *reinterpret_cast<const float4_t *>(xs + ((wr * MT + mt) * 16 + c) * LIN_LD + 16 * ss + 4 * q);
+                a[mt] = *reinterpret_cast<const float4_t *>(xs + ((wr * MT + mt) * 16 + c) * LD + 16 * ss + 4 * q);
 #pragma unroll
             for (int nt = 0; nt < NT; nt++)
-                b[nt] = *reinterpret_cast<const float4_t *>(ws + ((wc * NT + nt) * 16 + c) * LIN_LD + 16 * ss + 4 * q);
+                b[nt] = *reinterpret_cast<const float4_t *>(ws + ((wc * NT + nt) * 16 + c) * LD + 16 * ss + 4 * q);
 #pragma unroll
             for (int r = 0; r < 4; r++)
 #pragma unroll
@@ -464,14 +469,20 @@ extern "C" int cf_linear_rows(const float *x, int64_t N, int64_t K, const float 
     const int64_t gx = (N + (small ? 31 : 63)) / (small ? 32 : 64);
     const int64_t gy = (total_cols + (wide ? 63 : 31)) / (wide ? 64 : 32);
     CF_REQUIRE(gx < (1ll << 31) && gy < 65536, CF_ERR_UNSUPPORTED, "cf_linear_rows: too large");
-    if (small && wide)
-        linear_rows_kernel<32, 64, 2, 2><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
+    const dim3 grid((unsigned)gx, (unsigned)gy);
+    hipStream_t st = (hipStream_t)stream;
+    if (small && wide && K >= 64)
+        linear_rows_kernel<32, 64, 2, 2, 64><<<grid, 256, 0, st>>>(p);
+    else if (small && K >= 64)
+        linear_rows_kernel<32, 32, 2, 2, 64><<<grid, 256, 0, st>>>(p);
+    else if (small && wide)
+        linear_rows_kernel<32, 64, 2, 2, 32><<<grid, 256, 0, st>>>(p);
     else if (small)
-        linear_rows_kernel<32, 32, 2, 2><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
+        linear_rows_kernel<32, 32, 2, 2, 32><<<grid, 256, 0, st>>>(p);
     else if (wide)
-        linear_rows_kernel<64, 64, 2, 2><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
+        linear_rows_kernel<64, 64, 2, 2, 32><<<grid, 256, 0, st>>>(p);
     else
-        linear_rows_kernel<64, 32, 4, 1><<<dim3((unsigned)gx, (unsigned)gy), 256, 0, (hipStream_t)stream>>>(p);
+        linear_rows_kernel<64, 32, 4, 1, 32><<<grid, 256, 0, st>>>(p);
     CF_CHECK_LAUNCH("cf_linear_rows");
     return CF_OK;
 }
