@@ -110,8 +110,8 @@ def fused_training_step(model: nn.Module, batch, opt: "FusedAdamW", zero_grad: b
     """:func:`training_step` with the fused pieces, on any batch, launched eagerly: row-block
     linear Functions in the blocks, all linear layers' weight gradients from one grouped
     launch pair after the backward pass, clip + AdamW + schedule as one device-side update
-    (``opt`` carries the clip norm and the schedule).  About half the time of the plain step,
-    which is bound by the host side of some four hundred launches."""
+    (``opt`` carries the clip norm and the schedule).  About a third of the time of the plain
+    step, which is bound by the host side of some four hundred launches."""
     from . import hip_funcs
     if zero_grad:
         opt.zero_grad(set_to_none=True)
