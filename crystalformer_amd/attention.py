@@ -278,9 +278,10 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             spec = fused_exponents_spec(P) if q.is_cuda else None
             if spec is not None:
                 # alpha, its normalisation, the positive map and the query scaling in two launches
-                a, qs = GaussianExponentsHIP.apply(
-                    q, self.lattice_pos_weights, self.gauss_scale, P.normalize_gauss, self.training, spec[0],
-                    spec[1], P.gauss_lb_real, -0.5 * P.scale_real ** -2, 1.0 / math.sqrt(q.shape[-1]))
+                a, qs = hip_funcs.call(
+                    GaussianExponentsHIP, q, self.lattice_pos_weights, self.gauss_scale, P.normalize_gauss,
+                    self.training, spec[0], spec[1], P.gauss_lb_real, -0.5 * P.scale_real ** -2,
+                    1.0 / math.sqrt(q.shape[-1]))
             else:
                 a = gaussian_exponents(q, query, self.lattice_pos_weights, self.gauss_scale, P, self.training)
             dist_max = P.value_pe_dist_max
@@ -296,8 +297,8 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             if proj is not None and not P.value_pe_headed:
                 proj = proj.expand(proj.shape[0], H, proj.shape[2], proj.shape[3])
             enc = RealPeriodicEncodingWithProjFuncCUDA if P.use_low_memory else RealPeriodicEncodingFuncCUDA
-            out = enc.apply(a, points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real, dist_max,
-                            P.value_pe_width_scale, proj, *adaptive)
+            out = hip_funcs.call(enc, a, points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real, dist_max,
+                                 P.value_pe_width_scale, proj, *adaptive)
             bias = out[0]
             values = out[1] if len(out) >= 2 else None
 
@@ -308,7 +309,7 @@ class CrystalformerMultiheadAttentionCUDA(Module):
         if qs is None:
             qs = q / math.sqrt(q.shape[-1])
         if config.REPRODUCIBLITY_STATE >= 2 and batch_q is batch_kv:
-            attn = FusedDotProductAttentionCUDA.apply(qs, k, v, bias, values, batch_q, edges)
+            attn = hip_funcs.call(FusedDotProductAttentionCUDA, qs, k, v, bias, values, batch_q, edges)
         else:
             attn = loop_attention(qs, k, v, batch_q, edges, bias, values)
         attn = attn.contiguous().view(n, vd)

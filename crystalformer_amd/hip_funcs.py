@@ -103,6 +103,23 @@ def _w_leading(W_k: Optional[Tensor]) -> int:
     return 1 if W_k.dim() == 3 else W_k.shape[0]
 
 
+class _NoGradCtx:
+    """Stand-in for the autograd context when a Function's forward is called directly."""
+    needs_input_grad = (False,) * 16
+
+    def save_for_backward(self, *tensors):
+        pass
+
+
+def call(function, *args):
+    """``function.apply(*args)``; with autograd switched off the forward is called directly,
+    which spares the dispatch through the autograd machinery (several microseconds a call,
+    thirteen calls in a forward of the four-block model)."""
+    if torch.is_grad_enabled():
+        return function.apply(*args)
+    return function.forward(_NoGradCtx(), *args)
+
+
 def _enc_backward_tail(ga_ik, gW_k, has_adaptive_args: bool):
     base = (ga_ik, None, None, None, None, None, None, None, None, gW_k)
     return base + (None, None) if has_adaptive_args else base

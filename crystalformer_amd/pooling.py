@@ -16,6 +16,6 @@ def avr_pool(x, batch, sizes):
     """Mean over the atoms of each crystal; the irregular-mean kernel when the
     numerics switch is >= 1, otherwise the per-crystal torch loop."""
     if config.REPRODUCIBLITY_STATE >= 1 and x.is_cuda:
-        return hip_funcs.IrregularMeanCUDA.apply(x, batch, sizes)
+        return hip_funcs.call(hip_funcs.IrregularMeanCUDA, x, batch, sizes)
     parts = torch.split_with_sizes(x, sizes.tolist(), 0)
     return torch.stack([torch.mean(p, dim=0) for p in parts])
