@@ -70,6 +70,68 @@ __global__ void edge_index_kernel(const int64_t *atom_start, const int64_t *edge
     }
 }
 
+// Leading-zero cumulative sums of the crystal sizes, their squares and n (n + 1) / 2, in one
+// work-group: each thread sums a contiguous run of crystals, the run totals are scanned in
+// LDS, each thread then writes the prefixes of its run.
+constexpr int SCAN_THREADS = 256;
+__global__ __launch_bounds__(SCAN_THREADS) void layout_scan_kernel(const int64_t *sizes, int64_t B, int64_t *atom_start,
+                                                                   int64_t *edge_start, int64_t *unit_start)
+{
+    __shared__ int64_t tot[3][SCAN_THREADS];
+    const int t = threadIdx.x;
+    const int64_t run = (B + SCAN_THREADS - 1) / SCAN_THREADS;
+    const int64_t b0 = min((int64_t)t * run, B), b1 = min(b0 + run, B);
+    int64_t a = 0, e = 0, u = 0;
+    for (int64_t b = b0; b < b1; b++) {
+        const int64_t n = sizes[b];
+        a += n;
+        e += n * n;
+        u += n * (n + 1) / 2;
+    }
+    tot[0][t] = a; tot[1][t] = e; tot[2][t] = u;
+    __syncthreads();
+    if (t < 3) {                                     // exclusive scan of one row per thread
+        int64_t acc = 0;
+        for (int x = 0; x < SCAN_THREADS; x++) {
+            const int64_t v = tot[t][x];
+            tot[t][x] = acc;
+            acc += v;
+        }
+    }
+    __syncthreads();
+    a = tot[0][t]; e = tot[1][t]; u = tot[2][t];
+    if (t == 0) atom_start[0] = edge_start[0] = unit_start[0] = 0;
+    for (int64_t b = b0; b < b1; b++) {
+        const int64_t n = sizes[b];
+        a += n;
+        e += n * n;
+        u += n * (n + 1) / 2;
+        atom_start[b + 1] = a;
+        edge_start[b + 1] = e;
+        unit_start[b + 1] = u;
+    }
+}
+
+// CSR offsets of the atoms' edge rows in the dense blocks: atom i of crystal b (found by
+// bisection) starts at edge_start[b] + (i - atom_start[b]) n_b; entry N is the edge count.
+__global__ void layout_rows_kernel(const int64_t *atom_start, const int64_t *edge_start, int64_t B, int64_t N,
+                                   int64_t *e_start)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i > N) return;
+    if (i == N) {
+        e_start[N] = edge_start[B];
+        return;
+    }
+    int64_t lo = 0, hi = B;   // invariant: atom_start[lo] <= i < atom_start[hi]
+    while (hi - lo > 1) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (atom_start[mid] <= i) lo = mid; else hi = mid;
+    }
+    const int64_t a0 = atom_start[lo];
+    e_start[i] = edge_start[lo] + (i - a0) * (atom_start[lo + 1] - a0);
+}
+
 }  // namespace
 
 extern "C" int cf_irregular_mean_fwd(const float *src, const int64_t *start_n, int64_t B, int64_t D,
@@ -109,4 +171,23 @@ extern "C" int cf_edge_index(const int64_t *atom_start_n, const int64_t *edge_st
                                                                               pos, edge_ij_e, rpos_ij_e);
     CF_CHECK_LAUNCH("cf_edge_index");
     return CF_OK;
+}
+
+extern "C" int cf_batch_layout(const int64_t *sizes_n, int64_t B, int64_t N, int64_t E, int64_t *atom_start_n,
+                               int64_t *edge_start_n, int64_t *unit_start_n, int64_t *e_start_i, int64_t *edge_ij_e,
+                               int64_t *pairs_u, void *stream)
+{
+    CF_REQUIRE(B >= 1 && N >= 1 && E >= 1, CF_ERR_INVALID_ARGUMENT, "cf_batch_layout: B, N and E must be positive");
+    CF_REQUIRE(sizes_n && atom_start_n && edge_start_n && unit_start_n && e_start_i && edge_ij_e,
+               CF_ERR_INVALID_ARGUMENT, "cf_batch_layout: null pointer");
+    CF_REQUIRE(N < (1ll << 31) * 256, CF_ERR_UNSUPPORTED, "cf_batch_layout: too many atoms");
+    hipStream_t st = (hipStream_t)stream;
+    layout_scan_kernel<<<1, SCAN_THREADS, 0, st>>>(sizes_n, B, atom_start_n, edge_start_n, unit_start_n);
+    CF_CHECK_LAUNCH("cf_batch_layout: scan");
+    layout_rows_kernel<<<(int)((N + 1 + 255) / 256), 256, 0, st>>>(atom_start_n, edge_start_n, B, N, e_start_i);
+    CF_CHECK_LAUNCH("cf_batch_layout: rows");
+    int rc = cf_edge_index(atom_start_n, edge_start_n, B, E, nullptr, edge_ij_e, nullptr, stream);
+    if (rc) return rc;
+    if (pairs_u) rc = cf_edge_pairs(atom_start_n, edge_start_n, unit_start_n, B, E, pairs_u, stream);
+    return rc;
 }

@@ -61,6 +61,7 @@ SIGNATURES = {
     "cf_adamw_step": (_int, [_int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _f32, _f32, _f32, _f32, _f32, _f32, _ptr,
                              _ptr, _i64, _ptr]),
     "cf_l1_mean_loss": (_int, [_ptr, _ptr, _i64, _i64, _ptr, _ptr, _ptr]),
+    "cf_batch_layout": (_int, [_ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "cf_lattice_geometry": (_int, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
     "cf_gauss_exponents_workspace": (_i64, [_i64, _i64]),
     "cf_gauss_exponents": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _int, _int, _f32, _f32, _f32, _f32,

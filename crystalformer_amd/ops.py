@@ -491,16 +491,32 @@ def batch_layout(sizes: Tensor, batch_i: Tensor) -> BatchLayout:
     lay = BatchLayout()
     lay.sizes = sizes
     lay.batch = (batch_i - batch_i[0]) if batch_i.numel() else batch_i
-    lay.atom_start = F.pad(sizes.cumsum(0), (1, 0))
-    lay.edge_start = F.pad((sizes * sizes).cumsum(0), (1, 0))
-    tail = torch.stack([lay.atom_start[-1], lay.edge_start[-1]]).tolist() if sizes.numel() else [0, 0]
-    lay.num_atoms, lay.num_edges = int(tail[0]), int(tail[1])
+    # the one host read per distinct batch: the atom and edge counts size everything below
+    sizes_host = sizes.tolist()
+    B = len(sizes_host)
+    lay.num_atoms = sum(sizes_host)
+    lay.num_edges = sum(n * n for n in sizes_host)
     if lay.num_atoms != batch_i.numel():
         raise _lib.CrystalformerHipError(
             f"sizes sum to {lay.num_atoms} atoms but batch has {batch_i.numel()} entries")
-    lay.edges, _ = edge_index(sizes, None, lay.num_edges)
-    lay.e_start = edge_row_offsets(lay.edges, lay.num_atoms)
-    lay.pairs = edge_pairs(sizes, lay.num_atoms, lay.num_edges) if lay.num_edges else None
+    if B == 0 or lay.num_edges == 0 or min(sizes_host) < 0:
+        lay.atom_start = F.pad(sizes.cumsum(0), (1, 0))
+        lay.edge_start = F.pad((sizes * sizes).cumsum(0), (1, 0))
+        lay.edges, _ = edge_index(sizes, None, lay.num_edges)
+        lay.e_start = edge_row_offsets(lay.edges, lay.num_atoms)
+        lay.pairs = edge_pairs(sizes, lay.num_atoms, lay.num_edges) if lay.num_edges else None
+    else:
+        # prefix sums, row offsets, edge list and pair list in four launches
+        N, E = lay.num_atoms, lay.num_edges
+        starts = torch.empty((3, B + 1), dtype=torch.int64, device=dev)
+        lay.atom_start, lay.edge_start = starts[0], starts[1]
+        lay.e_start = torch.empty(N + 1, dtype=torch.int64, device=dev)
+        lay.edges = torch.empty((2, E), dtype=torch.int64, device=dev)
+        lay.pairs = torch.empty(((E + N) // 2, PAIR_FIELDS), dtype=torch.int64, device=dev)
+        with device_guard(dev):
+            rc = _lib.load().cf_batch_layout(ptr(sizes), B, N, E, ptr(starts[0]), ptr(starts[1]), ptr(starts[2]),
+                                             ptr(lay.e_start), ptr(lay.edges), ptr(lay.pairs), stream_handle(dev))
+        check(rc, "cf_batch_layout")
     s_, _ = _cache_lookup("e_start", lay.edges)
     _cache_store(s_, (lay.edges,), lay.e_start)
     if lay.pairs is not None:

@@ -401,6 +401,22 @@ int cf_adamw_step(int n_tensors, float *const *params, const float *const *grads
                   void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Every index structure of a batch of crystals with dense intra-crystal edges from the crystal
+ * sizes, in four launches and without a host round trip: what get_edge_index
+ * (models/indexed_latticeformer_encoder.py:15-32), the CSR offsets of
+ * models/cuda_funcs/fused_dpa.py:24-26 and cf_edge_pairs compute one by one.
+ *   sizes_n (B) atoms per crystal; N = sum n, E = sum n^2 (the caller knows them: it sized
+ *   the outputs)
+ * Outputs
+ *   atom_start_n, edge_start_n, unit_start_n (B+1): leading-zero cumulative sums of n, n^2,
+ *       n (n + 1) / 2
+ *   e_start_i (N+1), edge_ij_e (2,E), pairs_u ((E+N)/2, 5) or NULL
+ */
+int cf_batch_layout(const int64_t *sizes_n, int64_t B, int64_t N, int64_t E, int64_t *atom_start_n,
+                    int64_t *edge_start_n, int64_t *unit_start_n, int64_t *e_start_i, int64_t *edge_ij_e,
+                    int64_t *pairs_u, void *stream);
+
+/*
  * Training loss of the regression module and its gradient in one launch: the per-sample
  * L1 losses summed over the targets (losses/regression_loss.py:10-20 with loss_fn "l1"),
  * averaged over the batch (models/regression.py:117-118).

@@ -482,6 +482,25 @@ def test_batch_layout_bit_exact_and_cached(dev):
         ops.batch_layout(torch.tensor([2, 2], device=dev), torch.tensor([0, 0, 1], device=dev))
 
 
+@pytest.mark.parametrize("B,hi", [(1, 7), (128, 64), (300, 40), (1000, 9)])
+def test_batch_layout_structures_bit_exact(dev, B, hi):
+    """Prefix sums, row offsets, edge list and pair list of the one-call layout against the
+    oracle's loops and against the operators that build them one by one (more crystals than
+    the scan has threads included)."""
+    gen = torch.Generator().manual_seed(B)
+    sizes = torch.randint(1, hi + 1, (B,), generator=gen)
+    batch = torch.repeat_interleave(torch.arange(B), sizes)
+    lay = ops.batch_layout(sizes.to(dev), batch.to(dev))
+    zero = torch.zeros(1, dtype=torch.long)
+    assert torch.equal(lay.atom_start.cpu(), torch.cat([zero, sizes.cumsum(0)]))
+    assert torch.equal(lay.edge_start.cpu(), torch.cat([zero, (sizes * sizes).cumsum(0)]))
+    edges = tp.get_edge_index(sizes.tolist())
+    assert torch.equal(lay.edges.cpu(), edges)
+    assert torch.equal(lay.e_start.cpu(), tp.edge_row_offsets(edges, int(sizes.sum())))
+    assert torch.equal(lay.pairs, ops.edge_pairs(sizes.to(dev)))
+    assert torch.equal(lay.e_start, ops.edge_row_offsets(lay.edges, lay.num_atoms))
+
+
 @pytest.mark.parametrize("N,K,C,nw", [(1774, 128, 128, 3), (1774, 128, 512, 1), (1774, 512, 128, 1), (5, 16, 7, 2),
                                       (33, 48, 100, 1), (64, 64, 64, 3)])
 def test_linear_rows(dev, N, K, C, nw):
