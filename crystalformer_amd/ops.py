@@ -715,31 +715,53 @@ def linear_rows_supported(x: Tensor, *weights: Tensor) -> bool:
                and w.shape[1] == x.shape[1] for w in weights) and 1 <= len(weights) <= 3
 
 
+def _plain_f32(t: Tensor, dev: torch.device) -> bool:
+    return t.dtype is torch.float32 and t.device == dev and t.is_contiguous()
+
+
 def linear_rows(x: Tensor, weights, bias: Optional[Tensor] = None, residual: Optional[Tensor] = None,
                 relu: bool = False):
     """``act(x @ w.T + b) (+ residual)`` for up to three equally shaped weights in one
     launch; returns a tuple of outputs, one per weight.  No autograd."""
-    weights = [_f32(w, "weight") for w in weights]
-    dev = require_device(x, *weights, bias, residual)
-    x = _f32(x, "x")
-    bias = _f32(bias, "bias")
-    residual = _f32(residual, "residual")
+    dev = x.device
+    nw = len(weights)
+    # operands that need no conversion and no message (the hot case: this wrapper runs 18 times
+    # in a forward of the four-block model) skip the general checks below
+    lean = (dev.type == "cuda" and x.dim() == 2 and 1 <= nw <= 3 and _plain_f32(x, dev)
+            and (bias is None or _plain_f32(bias, dev)) and (residual is None or _plain_f32(residual, dev)))
+    if lean:
+        for w in weights:
+            if not (_plain_f32(w, dev) and w.dim() == 2):
+                lean = False
+                break
+    if not lean:
+        weights = [_f32(w, "weight") for w in weights]
+        dev = require_device(x, *weights, bias, residual)
+        x = _f32(x, "x")
+        bias = _f32(bias, "bias")
+        residual = _f32(residual, "residual")
+        if x.dim() != 2 or not 1 <= nw <= 3 or any(w.dim() != 2 for w in weights):
+            raise _lib.CrystalformerHipError("linear_rows: x (N, K) and one to three weights (C, K) expected")
     N, K = x.shape
     C = weights[0].shape[0]
-    if any(w.shape != (C, K) for w in weights):
-        raise _lib.CrystalformerHipError("linear_rows: weights must all be (C, K) with K = x.shape[1]")
-    if bias is not None and bias.numel() != len(weights) * C:
+    for w in weights:
+        if w.shape[0] != C or w.shape[1] != K:
+            raise _lib.CrystalformerHipError("linear_rows: weights must all be (C, K) with K = x.shape[1]")
+    if bias is not None and bias.numel() != nw * C:
         raise _lib.CrystalformerHipError("linear_rows: bias must have one entry per output column")
-    if residual is not None and (len(weights) != 1 or residual.shape != (N, C)):
+    if residual is not None and (nw != 1 or residual.shape != (N, C)):
         raise _lib.CrystalformerHipError("linear_rows: residual must be (N, C) with a single weight")
-    ys = [torch.empty((N, C), dtype=torch.float32, device=dev) for _ in weights]
-    pw = [ptr(w) for w in weights] + [None] * (3 - len(weights))
-    py = [ptr(y) for y in ys] + [None] * (3 - len(weights))
+    y0 = torch.empty((N, C), dtype=torch.float32, device=dev)
+    y1 = torch.empty((N, C), dtype=torch.float32, device=dev) if nw > 1 else None
+    y2 = torch.empty((N, C), dtype=torch.float32, device=dev) if nw > 2 else None
     with device_guard(dev):
-        rc = _lib.load().cf_linear_rows(ptr(x), N, K, pw[0], pw[1], pw[2], len(weights), C, ptr(bias),
-                                        ptr(residual), int(bool(relu)), py[0], py[1], py[2], stream_handle(dev))
-    check(rc, "cf_linear_rows")
-    return tuple(ys)
+        rc = _lib.load().cf_linear_rows(
+            x.data_ptr(), N, K, weights[0].data_ptr(), weights[1].data_ptr() if nw > 1 else None,
+            weights[2].data_ptr() if nw > 2 else None, nw, C, ptr(bias), ptr(residual), 1 if relu else 0,
+            y0.data_ptr(), ptr(y1), ptr(y2), stream_handle(dev))
+    if rc:
+        check(rc, "cf_linear_rows")
+    return (y0,) if nw == 1 else ((y0, y1) if nw == 2 else (y0, y1, y2))
 
 
 def linear_rows_nn_supported(g: Tensor, w: Tensor) -> bool:
