@@ -160,8 +160,14 @@ __device__ __forceinline__ void st1(void *base, uint32_t byte_off, float v)
 }
 
 // Every byte offset into prob / b_ij / key / value fits 32 bits (checked by the host).
-template <int DV4, bool HAS_A, bool HAS_B>
-__global__ __launch_bounds__(256, 7) void fused_dpa_fwd_stream_kernel(DpaArgs p, int LPE)
+// PREFETCH (long rows): the key indices of the next step are fetched one step ahead and every
+// load of a step is in flight together (one memory round trip per step, 80 registers).
+// Otherwise (rows of about one step): the indices are read at the top of the step and the
+// register budget is that of 8 resident wavefronts per SIMD, which the compiler meets by
+// fetching the value rows after the key rows have been used: one more round trip, and all
+// rows of a small batch resident at once.
+template <int DV4, bool HAS_A, bool HAS_B, bool PREFETCH>
+__global__ __launch_bounds__(256, (PREFETCH ? 6 : 7)) void fused_dpa_fwd_stream_kernel(DpaArgs p, int LPE)
 {
     __shared__ float part[DPA_WPQ][WAVE][6];
     __shared__ float fin[2][MAXH];
@@ -215,13 +221,23 @@ __global__ __launch_bounds__(256, 7) void fused_dpa_fwd_stream_kernel(DpaArgs p,
     uint32_t eb = e0;
     uint32_t e = eb + wave * ES + es;
     float s_tail[4];
-    for (;;) {
-        const bool last = eb + 4 * stride >= e1;                    // uniform
-        uint32_t jn[4];
+    uint32_t jn[4];
+    if (PREFETCH) {
 #pragma unroll
         for (int u = 0; u < 4; u++) jn[u] = (uint32_t)dst[min(e + u * stride, e_last)];
+    }
+    for (;;) {
+        const bool last = eb + 4 * stride >= e1;                    // uniform
+        if (!PREFETCH) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) jn[u] = (uint32_t)dst[min(e + u * stride, e_last)];
+        }
 #pragma unroll
         for (int u = 0; u < 4; u++) fetch(u, min(e + u * stride, e_last), jn[u]);
+        if (PREFETCH && !last) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) jn[u] = (uint32_t)dst[min(e + (4 + u) * stride, e_last)];
+        }
 #pragma unroll
         for (int u = 0; u < 4; u++) s_tail[u] = fold(u, e + u * stride < e1);
         if (last) break;
@@ -560,25 +576,31 @@ void launch_fwd(const DpaArgs &p, hipStream_t st)
     fused_dpa_fwd_kernel<H><<<(int)((p.N + wpb - 1) / wpb), wpb * WAVE, 0, st>>>(p);
 }
 
-template <int DV4>
+template <int DV4, bool PREFETCH>
 void launch_fwd_stream_dv(const DpaArgs &p, int lpe, hipStream_t st)
 {
     const dim3 grid((unsigned)p.N), block(DPA_WPQ * WAVE);
-    if (p.aij && p.bij) fused_dpa_fwd_stream_kernel<DV4, true, true><<<grid, block, 0, st>>>(p, lpe);
-    else if (p.aij) fused_dpa_fwd_stream_kernel<DV4, true, false><<<grid, block, 0, st>>>(p, lpe);
-    else if (p.bij) fused_dpa_fwd_stream_kernel<DV4, false, true><<<grid, block, 0, st>>>(p, lpe);
-    else fused_dpa_fwd_stream_kernel<DV4, false, false><<<grid, block, 0, st>>>(p, lpe);
+    if (p.aij && p.bij) fused_dpa_fwd_stream_kernel<DV4, true, true, PREFETCH><<<grid, block, 0, st>>>(p, lpe);
+    else if (p.aij) fused_dpa_fwd_stream_kernel<DV4, true, false, PREFETCH><<<grid, block, 0, st>>>(p, lpe);
+    else if (p.bij) fused_dpa_fwd_stream_kernel<DV4, false, true, PREFETCH><<<grid, block, 0, st>>>(p, lpe);
+    else fused_dpa_fwd_stream_kernel<DV4, false, false, PREFETCH><<<grid, block, 0, st>>>(p, lpe);
 }
 
 void launch_fwd_stream(const DpaArgs &p, int dv4, int lpe, hipStream_t st)
 {
+    // mean row length beyond two steps of the work-group: the variant that keeps one round trip per step
+    const int64_t step_edges = 4 * DPA_WPQ * (WAVE / lpe);
+    const bool long_rows = p.E > 2 * step_edges * p.N;
+#define CF_DPA_FWD(DV) \
+    do { if (long_rows) launch_fwd_stream_dv<DV, true>(p, lpe, st); else launch_fwd_stream_dv<DV, false>(p, lpe, st); } while (0)
     switch (dv4) {
-        case 1: launch_fwd_stream_dv<1>(p, lpe, st); break;
-        case 2: launch_fwd_stream_dv<2>(p, lpe, st); break;
-        case 4: launch_fwd_stream_dv<4>(p, lpe, st); break;
-        case 8: launch_fwd_stream_dv<8>(p, lpe, st); break;
-        default: launch_fwd_stream_dv<16>(p, lpe, st); break;
+        case 1: CF_DPA_FWD(1); break;
+        case 2: CF_DPA_FWD(2); break;
+        case 4: CF_DPA_FWD(4); break;
+        case 8: CF_DPA_FWD(8); break;
+        default: CF_DPA_FWD(16); break;
     }
+#undef CF_DPA_FWD
 }
 
 template <int DV4>

@@ -299,7 +299,9 @@ def dpa_problem(sizes, H, Dk, Dv, seed, bias=True, vals=True):
 @pytest.mark.parametrize("H,Dk,Dv,sizes", [(8, 16, 16, [1, 5, 70, 2, 33]), (4, 8, 32, [3, 65]), (1, 5, 4, [7, 2]),
                                            (16, 16, 16, [9, 1]), (2, 64, 64, [4]),
                                            (8, 16, 16, [32, 64, 31, 8]),      # rows of exactly one and two whole steps
-                                           (4, 8, 8, [17, 40]), (2, 4, 4, [130]), (1, 32, 32, [12])])
+                                           (4, 8, 8, [17, 40]), (2, 4, 4, [130]), (1, 32, 32, [12]),
+                                           (8, 16, 16, [200, 150, 97]),       # long rows: the prefetching variant
+                                           (8, 16, 16, [70, 66, 65])])
 def test_fused_dpa_fwd_bwd(dev, H, Dk, Dv, sizes, bias, vals):
     p, q, k, v, a, b = dpa_problem(sizes, H, Dk, Dv, 31, bias, vals)
     out, prob = ops.fused_dpa_fwd(*to_dev(dev, q, k, v, a, b, p.edges, p.e_start))
