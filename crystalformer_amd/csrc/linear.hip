@@ -508,7 +508,7 @@ extern "C" int cf_linear_rows_nn(const float *g0, const float *g1, const float *
     CF_REQUIRE(y, CF_ERR_INVALID_ARGUMENT, "cf_linear_rows_nn: null output");
     p.add = add; p.mask = mask; p.y = y; p.N = N; p.C = (int)C; p.K = (int)K; p.terms = n_terms;
     // quarter tiles while full ones would leave most CUs without a work-group
-    if (((N + 63) / 64) * ((K + 63) / 64) < 128) {
+    if (((N + 63) / 64) * ((K + 63) / 64) < 256) {
         dim3 grid((unsigned)((N + 31) / 32), (unsigned)((K + 31) / 32));
         linear_rows_nn_kernel<32, 32><<<grid, 256, 0, (hipStream_t)stream>>>(p);
     } else {
