@@ -461,22 +461,18 @@ extern "C" int cf_linear_rows(const float *x, int64_t N, int64_t K, const float 
     }
     p.bias = bias; p.res = residual;
     p.N = N; p.K = (int)K; p.C = (int)C; p.nw = n_weights; p.relu = relu;
-    // wide outputs: 64-column tiles (2 x 2 wavefronts); narrow ones: 32-column tiles, more work-groups
+    // few rows (a tile grid that leaves CUs idle): 32 x 32 tiles, four to eight times the work-groups;
+    // otherwise wide outputs take 64-column tiles (2 x 2 wavefronts), narrow ones 32-column tiles
     const int64_t total_cols = (int64_t)n_weights * C;
-    const bool wide = total_cols >= 256;
-    // few rows (a tile grid that leaves CUs idle): half-height tiles, twice the work-groups
     const bool small = N <= 8192;
+    const bool wide = !small && total_cols >= 256;
     const int64_t gx = (N + (small ? 31 : 63)) / (small ? 32 : 64);
     const int64_t gy = (total_cols + (wide ? 63 : 31)) / (wide ? 64 : 32);
     CF_REQUIRE(gx < (1ll << 31) && gy < 65536, CF_ERR_UNSUPPORTED, "cf_linear_rows: too large");
     const dim3 grid((unsigned)gx, (unsigned)gy);
     hipStream_t st = (hipStream_t)stream;
-    if (small && wide && K >= 64)
-        linear_rows_kernel<32, 64, 2, 2, 64><<<grid, 256, 0, st>>>(p);
-    else if (small && K >= 64)
+    if (small && K >= 64)
         linear_rows_kernel<32, 32, 2, 2, 64><<<grid, 256, 0, st>>>(p);
-    else if (small && wide)
-        linear_rows_kernel<32, 64, 2, 2, 32><<<grid, 256, 0, st>>>(p);
     else if (small)
         linear_rows_kernel<32, 32, 2, 2, 32><<<grid, 256, 0, st>>>(p);
     else if (wide)
