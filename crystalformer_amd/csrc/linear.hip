@@ -288,7 +288,7 @@ __global__ __launch_bounds__(1024) void column_sum_kernel(const float *g, int64_
 // The weight (and bias) gradients of several linear layers in two launches: the layers'
 // 64 x 64 output tiles are numbered consecutively and a work-group finds its layer by
 // scanning the group's tile prefix.
-constexpr int WG_GROUP = 16;
+constexpr int WG_GROUP = 32;       // layers per launch pair (64 bytes each of the 4 KB of kernel arguments)
 
 struct WeightGradGroup {
     const float *g[WG_GROUP], *x[WG_GROUP];
@@ -300,6 +300,7 @@ struct WeightGradGroup {
     int count;
     float *part;
 };
+static_assert(sizeof(WeightGradGroup) <= 4096, "WeightGradGroup must fit the kernel-argument segment");
 
 constexpr int WGT = 64;            // output tile of a work-group: 64 x 64
 constexpr int WG_ROWS = 16;        // rows staged per step

@@ -367,7 +367,7 @@ int cf_reci_enc_bwd(const float *a_ik, const float *kr_base_e, const float *rvec
                     int64_t E, int lattice_range, int normalisation_grad, float *ga_ik, void *stream);
 
 /*
- * cf_linear_weight_grad for n_layers linear layers at once (2 * ceil(n_layers / 16)
+ * cf_linear_weight_grad for n_layers linear layers at once (2 * ceil(n_layers / 32)
  * launches instead of 2 * n_layers); per layer the result is bit-identical to the single
  * call.  g, x, gW, gb: HOST arrays of device pointers (gb[t] may be NULL); N, C, K: HOST
  * arrays.  workspace: cf_linear_weight_grad_grouped_workspace(n_layers, N, C, K) bytes.

@@ -713,11 +713,11 @@ def test_gauss_exponents_bwd_kernel(dev, func, N, H, D, scaled):
 
 
 def test_linear_weight_grad_grouped_equals_single_calls(dev):
-    """Twenty layers of ragged shapes (two kernel-argument groups, with and without bias,
+    """Thirty-eight layers of ragged shapes (two kernel-argument groups of 32, with and without bias,
     different row counts and slice counts) in one grouped call: bit-identical to one call each."""
     gen = torch.Generator().manual_seed(21)
     shapes = [(1774, 128, 128), (1774, 512, 128), (1774, 128, 512), (70, 48, 32), (3, 5, 7), (600, 33, 100)]
-    shapes = shapes * 3 + [(1774, 128, 128), (40, 16, 16)]
+    shapes = shapes * 6 + [(1774, 128, 128), (40, 16, 16)]
     layers, expect = [], []
     for k, (N, C, K) in enumerate(shapes):
         g, x = torch.randn(N, C, generator=gen).to(dev), torch.randn(N, K, generator=gen).to(dev)
