@@ -25,8 +25,6 @@ int device_cu_count();
 // Work-groups a persistent kernel may launch at `per_cu` per CU, scaled by the calling
 // thread's launch share (cf_set_launch_share).
 int persistent_grid_cap(int per_cu);
-// True when the calling thread has set a launch share below 1 (other streams are expected to be busy).
-bool launch_is_shared();
 
 // real_enc_mfma.hip
 int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,

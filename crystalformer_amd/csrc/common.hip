@@ -46,8 +46,6 @@ int persistent_grid_cap(int per_cu)
     return (int)(cap < 1 ? 1 : cap);
 }
 
-bool launch_is_shared() { return g_launch_share < 1.0; }
-
 }  // namespace cf
 
 extern "C" int cf_version(void) { return 100; }

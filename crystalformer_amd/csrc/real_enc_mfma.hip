@@ -33,7 +33,7 @@ using namespace cf;
 using namespace cfpair;
 
 constexpr int RING_CAP = 256;            // translations staged per pass
-constexpr int RING_CAP_SMALL = 128;      // the same where the exchange buffer is double (see the kernel)
+constexpr int RING_CAP_SMALL = 128;      // the same for a fixed cube that fits (see SHORT_RING in the kernel)
 constexpr int RING_SLOTS = RING_CAP + 16; // + neutral padding (last groups, look-ahead) between the two blocks
 
 
@@ -45,9 +45,8 @@ constexpr int PROJ_INDEXED = 2;          // W per edge or per atom: read from gl
 
 // LDS per work-group: per wave three ring arrays of ring capacity + 16 words (d^2, distance
 // argument, flag bits); for PROJ_SHARED also the exchange buffer of 4 NT planes of XPLANE floats
-// (layout in real_enc_pair.h), WPB x 2 edge ids and WPB x 16 reciprocal column totals -- twice
-// each for the fixed cube (see DB in the kernel).
-template <int NT, bool UNIFORM, int PROJ, int DT, bool TWIN>
+// (layout in real_enc_pair.h), WPB x 2 edge ids and WPB x 16 reciprocal column totals.
+template <int NT, bool UNIFORM, int PROJ, int DT, bool SHORT_RING>
 __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
 {
     extern __shared__ __align__(16) float lds[];
@@ -63,24 +62,19 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
     const float *__restrict__ g_tvecs = p.tvecs;
     const float *__restrict__ g_a = p.a_ik;
     const float *__restrict__ g_rvlen = p.rvlen;
-    // TWIN (fixed cube with the shared projection, a launch that has the GPU to itself): the
-    // exchange buffer and its side arrays exist twice and rounds alternate between the copies, so
-    // that a wavefront may park round r + 1 while another still projects round r: one barrier
-    // per round instead of two (56.0 against 57.8 us at 56 440 edges).  The ring then holds 128
-    // translations per pass (the default cube has 125), which is what makes the second copy fit
-    // beside a second work-group on the CU.  Launches that share the GPU with other streams keep
-    // the single buffer: with several forwards in flight the lighter work-group did better.
-    static_assert(!TWIN || (UNIFORM && PROJ == PROJ_SHARED && NT <= 4), "no such variant");
-    constexpr bool DB = TWIN;
-    constexpr int RCAP = DB ? RING_CAP_SMALL : RING_CAP;
+    // SHORT_RING (a fixed cube of at most 128 translations, the default cube has 125): the ring
+    // holds 128 instead of 256 translations per pass.  Half the distances cached in registers
+    // across the staging passes and 12 KB less LDS per work-group: 56.0 against 57.8 us at
+    // 56 440 edges, and more room for the kernels of other streams beside it.
+    static_assert(!SHORT_RING || UNIFORM, "the short ring is for the fixed cube");
+    constexpr int RCAP = SHORT_RING ? RING_CAP_SMALL : RING_CAP;
     constexpr int RSLOTS = RCAP + 16;
-    constexpr int XB = 4 * NT * SPLANE;                              // floats of one exchange buffer
     float *ring_d2 = lds + wave * (3 * RSLOTS);
     float *ring_s = ring_d2 + RSLOTS;
     int *ring_bits = reinterpret_cast<int *>(ring_s + RSLOTS);
-    float *Sbuf0 = lds + WPB * 3 * RSLOTS;                           // (copies x) [4 NT][SPLANE]
-    int64_t *meta0 = reinterpret_cast<int64_t *>(Sbuf0 + (DB ? 2 : 1) * XB);      // (copies x) [WPB][2]
-    float *invbuf0 = reinterpret_cast<float *>(meta0 + (DB ? 2 : 1) * WPB * 2);   // (copies x) [WPB][16]
+    float *Sbuf = lds + WPB * 3 * RSLOTS;                            // [4 NT][SPLANE]
+    int64_t *meta = reinterpret_cast<int64_t *>(Sbuf + 4 * NT * SPLANE);   // [WPB][2]
+    float *invbuf = reinterpret_cast<float *>(meta + WPB * 2);             // [WPB][16]
 
     // Gaussian argument of bin 16m + c at distance 0
     float ck[NT];
@@ -467,9 +461,6 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         } else if (PROJ == PROJ_SHARED) {
             // park the column sums (inactive columns hold zeros: their weights are masked) and the
             // reciprocal of the column totals, then project per head
-            float *Sbuf = Sbuf0 + (DB ? (it & 1) * XB : 0);
-            int64_t *meta = meta0 + (DB ? (it & 1) * WPB * 2 : 0);
-            float *invbuf = invbuf0 + (DB ? (it & 1) * WPB * 16 : 0);
             float *col = Sbuf + xch_base(q, c & 7, wave, c >> 3);
 #pragma unroll
             for (int m = 0; m < NT; m++)
@@ -520,7 +511,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                     }
                 }
             }
-            if (!DB) __syncthreads();      // single buffer: nobody parks the next round before all have read this one
+            __syncthreads();
         } else {
             int64_t w_ind = 0;
             if (p.W_num == p.E) w_ind = e_col;
@@ -648,14 +639,12 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     if (W) mode = (W_num == 1) ? PROJ_SHARED : PROJ_INDEXED;
     if (mode == PROJ_SHARED && D > 32) return CF_ERR_UNSUPPORTED;
     const int DT = (mode == PROJ_SHARED && D > 16) ? 2 : 1;
-    // double exchange buffer with the short ring: a launch on its own whose cube fits one pass of
-    // that ring (so that both variants stage the translations in the same order, bit for bit)
+    // a fixed cube that fits one pass of the short ring
     const int64_t cube = (int64_t)(2 * lattice_range + 1) * (2 * lattice_range + 1) * (2 * lattice_range + 1);
-    const bool twin = uniform && mode == PROJ_SHARED && NT <= 4 && cube <= RING_CAP_SMALL && !launch_is_shared();
-    size_t lds = sizeof(float) * (size_t)WPB * 3 * ((twin ? RING_CAP_SMALL : RING_CAP) + 16);
+    const bool short_ring = uniform && cube <= RING_CAP_SMALL;
+    size_t lds = sizeof(float) * (size_t)WPB * 3 * ((short_ring ? RING_CAP_SMALL : RING_CAP) + 16);
     if (mode == PROJ_SHARED)
-        lds += (twin ? 2 : 1) * (sizeof(float) * (size_t)4 * NT * XPLANE + sizeof(int64_t) * WPB * 2 +
-                                 sizeof(float) * WPB * 16) + 8;
+        lds += sizeof(float) * (size_t)4 * NT * XPLANE + sizeof(int64_t) * WPB * 2 + sizeof(float) * WPB * 16 + 8;
     const int64_t rounds = ((U + WPB - 1) / WPB) * p.head_groups;
     if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // round positions are 32-bit in the kernel
     int64_t blocks = rounds;
@@ -667,46 +656,21 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     // and the fixed stride, which costs nothing, does better (measured: 64.5 against 70 us at
     // 7 rounds per work-group; 1.66 against 1.81 ms at 217).
     if (rounds < 16 * blocks) p.sched = nullptr;
-    // (more than 64 KB of dynamic LDS is asked for once per kernel and device)
-    int dev_ = 0;
-    if (lds > 65536 && hipGetDevice(&dev_) != hipSuccess) dev_ = 0;
-#define CF_PAIR(NTV, UNI, PRJ, DTV, TW)                                                                       \
-    do {                                                                                                      \
-        static bool lds_raised[64] = {};                                                                      \
-        if (lds > 65536 && !lds_raised[dev_ & 63]) {                                                          \
-            const hipError_t e_ = hipFuncSetAttribute(                                                        \
-                reinterpret_cast<const void *>(&real_enc_fwd_pair_kernel<NTV, UNI, PRJ, DTV, TW>),            \
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                        \
-            if (e_ != hipSuccess) return hip_failed(e_, "cf_real_enc_fwd: raising the dynamic LDS limit");    \
-            lds_raised[dev_ & 63] = true;                                                                     \
-        }                                                                                                     \
-        real_enc_fwd_pair_kernel<NTV, UNI, PRJ, DTV, TW><<<(int)blocks, WPB * WAVE, lds, st>>>(p);           \
+#define CF_PAIR(NTV, UNI, PRJ, DTV, SR) \
+    real_enc_fwd_pair_kernel<NTV, UNI, PRJ, DTV, SR><<<(int)blocks, WPB * WAVE, lds, st>>>(p)
+#define CF_PAIR_MODE(NTV, UNI, SR)                                            \
+    do {                                                                      \
+        if (mode == PROJ_NONE) CF_PAIR(NTV, UNI, PROJ_NONE, 1, SR);           \
+        else if (mode == PROJ_INDEXED) CF_PAIR(NTV, UNI, PROJ_INDEXED, 1, SR); \
+        else if (DT == 1) CF_PAIR(NTV, UNI, PROJ_SHARED, 1, SR);              \
+        else CF_PAIR(NTV, UNI, PROJ_SHARED, 2, SR);                           \
     } while (0)
-#define CF_PAIR_MODE(NTV, UNI)                                               \
-    do {                                                                     \
-        if (mode == PROJ_NONE) CF_PAIR(NTV, UNI, PROJ_NONE, 1, false);       \
-        else if (mode == PROJ_INDEXED) CF_PAIR(NTV, UNI, PROJ_INDEXED, 1, false); \
-        else if (DT == 1) CF_PAIR(NTV, UNI, PROJ_SHARED, 1, false);          \
-        else CF_PAIR(NTV, UNI, PROJ_SHARED, 2, false);                       \
+#define CF_PAIR_NT(NTV)                                     \
+    do {                                                    \
+        if (short_ring) CF_PAIR_MODE(NTV, true, true);      \
+        else if (uniform) CF_PAIR_MODE(NTV, true, false);   \
+        else CF_PAIR_MODE(NTV, false, false);               \
     } while (0)
-#define CF_PAIR_TWIN(NTV)                                     \
-    do {                                                      \
-        if (DT == 1) CF_PAIR(NTV, true, PROJ_SHARED, 1, true); \
-        else CF_PAIR(NTV, true, PROJ_SHARED, 2, true);        \
-    } while (0)
-#define CF_PAIR_NT(NTV)                       \
-    do {                                      \
-        if (uniform) CF_PAIR_MODE(NTV, true); \
-        else CF_PAIR_MODE(NTV, false);        \
-    } while (0)
-    if (twin) {
-        switch (NT) {
-            case 1: CF_PAIR_TWIN(1); break;
-            case 2: CF_PAIR_TWIN(2); break;
-            default: CF_PAIR_TWIN(4); break;
-        }
-        return CF_OK;
-    }
     switch (NT) {
         case 1: CF_PAIR_NT(1); break;
         case 2: CF_PAIR_NT(2); break;
@@ -714,7 +678,6 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
         default: CF_PAIR_NT(8); break;
     }
 #undef CF_PAIR_NT
-#undef CF_PAIR_TWIN
 #undef CF_PAIR_MODE
 #undef CF_PAIR
     return CF_OK;
