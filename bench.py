@@ -194,9 +194,9 @@ def main() -> int:
     ap.add_argument("--inflight", type=int, default=4,
                     help="batches in flight: the step's HIP graph is replayed round robin on this many "
                          "streams (default priority), each with its own copy of the batch; 1 = one after the other")
-    ap.add_argument("--launch-share", type=float, default=0.6875,
+    ap.add_argument("--launch-share", type=float, default=0.75,
                     help="with several steps in flight: share of the GPU one periodic-encoding launch "
-                         "occupies (352 of its 512 work-groups by default)")
+                         "occupies (384 of its 512 work-groups by default)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--train", action="store_true",
                     help="time full training steps (forward + backward + AdamW) instead of forwards")
