@@ -43,7 +43,8 @@ def test_real_enc_fwd(dev, H, K, D, cutoff, lr, mr):
             assert v is None
 
 
-@pytest.mark.parametrize("cutoff,lr,mr", RULES + [(-3.5, 3, 3)])
+# (fixed cubes of 27 and 125 translations take the short ring of the kernel, 343 the long one)
+@pytest.mark.parametrize("cutoff,lr,mr", RULES + [(-3.5, 3, 3), (0.0, 3, 0), (0.0, 1, 0)])
 @pytest.mark.parametrize("H,K,D", [(8, 64, 16), (4, 16, 8), (1, 7, 3), (2, 100, 4), (16, 32, 8), (8, 64, 32),
                                    (8, 48, 20), (8, 64, 64), (8, 0, 16), (2, 0, 4)])
 def test_real_enc_fwd_pair_kernel(dev, H, K, D, cutoff, lr, mr):
@@ -118,7 +119,7 @@ def test_real_enc_pair_kernel_atoms_outside_the_home_cell(dev, cutoff, mr):
         assert_close(gW, gW_ref.reshape(gW.shape), "gW", rtol=1e-4)
 
 
-@pytest.mark.parametrize("cutoff,lr,mr", RULES[:3])
+@pytest.mark.parametrize("cutoff,lr,mr", RULES[:3] + [(0.0, 3, 0)])
 @pytest.mark.parametrize("H,K,D", [(8, 64, 16), (4, 16, 8), (16, 32, 16), (1, 7, 12), (8, 64, 32)])
 def test_real_enc_bwd_pair_kernel(dev, H, K, D, cutoff, lr, mr):
     p = Problem([1, 3, 9, 2, 14, 1, 1, 1, 1, 20], H=H, K=K, D=D, seed=30)
