@@ -63,9 +63,9 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
     const float *__restrict__ g_a = p.a_ik;
     const float *__restrict__ g_rvlen = p.rvlen;
     // SHORT_RING (a fixed cube of at most 128 translations, the default cube has 125): the ring
-    // holds 128 instead of 192 translations per pass.  Half the distances cached in registers
-    // across the staging passes and 12 KB less LDS per work-group: 56.0 against 57.8 us at
-    // 56 440 edges, and more room for the kernels of other streams beside it.
+    // holds 128 translations per pass, no more than the cube needs.  Fewer distances cached in
+    // registers across the staging passes and less LDS per work-group than with a ring of 256:
+    // 56.0 against 57.8 us at 56 440 edges, and more room for the kernels of other streams.
     static_assert(!SHORT_RING || UNIFORM, "the short ring is for the fixed cube");
     constexpr int RCAP = SHORT_RING ? RING_CAP_SMALL : RING_CAP;
     constexpr int RSLOTS = RCAP + 16;
