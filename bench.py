@@ -384,6 +384,16 @@ def main() -> int:
                 tr = json.load(f).get(f"{args.config}:{args.rule}")
             if tr:
                 roofline["traffic"] = tr
+            with open(traffic_file) as f:
+                ins = json.load(f).get(f"{args.config}:{args.rule}:insts")
+            if ins and enc_avg_ms > 0:
+                # the kernel's own bound, from its rocprofv3 instruction counters: a wave64 vector
+                # instruction occupies its SIMD for 4 cycles, an fp32 16x16x4 MFMA for 32, and the
+                # two do not overlap in this kernel; 4 SIMDs per CU at the peak engine clock
+                cycles = (ins["valu"] - ins["mfma"]) * 4.0 + ins["mfma"] * 32.0
+                issue_ms = cycles / (ins["cus"] * 4 * ins["clock_ghz"] * 1e9) * 1e3
+                roofline["issue"] = {"valu_insts": ins["valu"], "mfma_insts": ins["mfma"],
+                                     "issue_ms": round(issue_ms, 4), "frac": round(issue_ms / enc_avg_ms, 4)}
         except Exception:
             pass
 
