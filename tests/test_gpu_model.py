@@ -273,6 +273,31 @@ def test_graph_replay_matches_eager(dev):
     assert torch.equal(graphed(b), y_eager)
 
 
+def test_graphs_in_flight_with_a_launch_share(dev):
+    """Four graphs of the same model captured with a launch share below 1 and replayed round robin
+    on four streams (the benchmark's throughput mode): every replay equals the eager result bit
+    for bit, and the share is back at 1 afterwards."""
+    from crystalformer_amd import lib
+    from crystalformer_amd.graphs import GraphedForward
+    cfg, model = build_model("cfg2_default_b128", num_layers=2, adaptive_cutoff_sigma=0.0)
+    model.to(dev).eval()
+    b = make_config_batch("cfg2_default_b128").to(dev)
+    with torch.no_grad():
+        y_eager = model(b).clone()
+    lanes = [(torch.cuda.Stream(), GraphedForward(model, b, warmup=1, launch_share=0.75)) for _ in range(4)]
+    assert lib.load().cf_get_launch_share() == 1.0
+    for st, _ in lanes:
+        st.wait_stream(torch.cuda.current_stream())
+    outs = []
+    for k in range(12):
+        st, g = lanes[k % 4]
+        with torch.cuda.stream(st):
+            outs.append((k % 4, g().clone()))
+    torch.cuda.synchronize()
+    for lane, y in outs:
+        assert torch.equal(y, y_eager), lane
+
+
 def test_graphed_training_step_matches_eager(dev):
     """Whole training step as one HIP graph.  (1) Replays equal, bit for bit, the same step
     launched eagerly (eager work and synchronisations between replays); (2) both follow the
