@@ -319,6 +319,29 @@ def test_fused_dpa_fwd_bwd(dev, H, Dk, Dv, sizes, bias, vals):
             assert_close(x, y, name)
 
 
+@pytest.mark.parametrize("H,D", [(8, 16), (1, 5)])
+def test_fused_dpa_fwd_on_an_arbitrary_edge_list(dev, H, D):
+    """The forward takes any edge list sorted by source atom: a random third of the dense edges
+    removed, one atom left without any edge (its output row is zero)."""
+    p, q, k, v, a, b = dpa_problem([5, 40, 70, 3], H, D, D, 35)
+    gen = torch.Generator().manual_seed(3)
+    keep = torch.rand(p.E, generator=gen) > 0.33
+    keep &= p.edges[0] != 17                                   # atom 17 loses every edge
+    edges = p.edges[:, keep].contiguous()
+    e_start = tp.edge_row_offsets(edges, p.N)
+    a, b = a[keep].contiguous(), b[keep].contiguous()
+    out, prob = ops.fused_dpa_fwd(*to_dev(dev, q, k, v, a, b, edges, e_start))
+    out_ref, prob_ref = ks.fused_dpa_fwd(q, k, v, a, b, edges, e_start)
+    assert_close(out, out_ref, "out")
+    assert_close(prob, prob_ref, "prob")
+    assert float(out[17].abs().max()) == 0.0
+    rows = torch.zeros(p.N, H).index_add_(0, edges[0], prob.cpu())
+    has = (e_start[1:] - e_start[:-1]) > 0
+    assert not bool(has[17]) and int(has.sum()) > p.N // 2
+    assert float((rows[has] - 1.0).abs().max()) < 1e-5         # each row's weights sum to one
+    assert float(out.cpu()[~has].abs().max()) == 0.0
+
+
 def test_fused_dpa_beyond_the_reference_size_limit(dev):
     """The reference's kernels stop at 320 atoms per crystal; these do not."""
     p, q, k, v, a, b = dpa_problem([444, 3], 8, 16, 16, 32)
