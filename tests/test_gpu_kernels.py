@@ -528,7 +528,8 @@ def test_batch_layout_structures_bit_exact(dev, B, hi):
 
 
 @pytest.mark.parametrize("N,K,C,nw", [(1774, 128, 128, 3), (1774, 128, 512, 1), (1774, 512, 128, 1), (5, 16, 7, 2),
-                                      (33, 48, 100, 1), (64, 64, 64, 3)])
+                                      (33, 48, 100, 1), (64, 64, 64, 3),
+                                      (9000, 128, 128, 3), (9001, 48, 96, 1)])     # beyond 8192 rows: the full-height tiles
 def test_linear_rows(dev, N, K, C, nw):
     g = torch.Generator().manual_seed(N + C)
     x = torch.randn(N, K, generator=g)
@@ -890,7 +891,8 @@ def test_reci_enc_clamp_and_function(dev):
 
 
 @pytest.mark.parametrize("N,C,K,terms", [(1774, 128, 128, 3), (1774, 512, 128, 1), (1774, 128, 512, 1), (70, 64, 20, 2),
-                                         (3, 64, 4, 1), (130, 192, 72, 3)])
+                                         (3, 64, 4, 1), (130, 192, 72, 3),
+                                         (16500, 128, 128, 2)])                    # enough work-groups for full tiles
 def test_linear_rows_nn(dev, N, C, K, terms):
     """Input-gradient kernel: mask(sum_i g_i W_i) + add against float64, with ragged row and
     column tails, one to three terms, with and without addend and mask."""
