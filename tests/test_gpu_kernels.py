@@ -702,7 +702,8 @@ def test_l1_mean_loss_and_its_gradient(dev, B, T):
 
 @pytest.mark.parametrize("func", ["elu", "abs", "exp"])
 @pytest.mark.parametrize("N,H,D,scaled", [(1774, 8, 16, True), (301, 3, 20, False), (5, 1, 4, True),
-                                          (700, 16, 8, True)])
+                                          (700, 16, 8, True),
+                                          (40, 2, 6, True), (33, 3, 19, False)])   # widths off the 16-byte path
 def test_gauss_exponents_bwd_kernel(dev, func, N, H, D, scaled):
     """Backward kernel against float64 autograd of a = coef * rho((alpha + shift) * scale),
     q_scaled = q * q_scale, with (scale, shift) constants; several blocks, ragged tails,
