@@ -28,8 +28,158 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 # published MI355X peaks
-PEAK_FP32_TFLOPS = 157.3
+PEAK_FP32_TFLOPS = 157.3          # fp32 on the matrix cores (and packed vector FMA, which this build compiles off)
+PEAK_FP32_VALU_TFLOPS = 78.6      # one fp32 FMA per lane and cycle: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz x 2
 PEAK_HBM_GBS = 8000.0
+PROFILE_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+KERNEL_SOURCES = ("real_enc_mfma.hip", "real_enc_mfma_bwd.hip", "real_enc_pair.h", "cf_common.h")
+
+
+def kernel_fingerprint() -> str:
+    """SHA-256 (first 16 hex digits) of the sources of the periodic-encoding pair kernels: stored
+    beside hardware counters when they are taken, compared when they are used."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "crystalformer_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def stored_counters(key: str, required: bool):
+    """Counters of one kernel launch from a ``rocprofv3 --pmc`` run (``--ingest-counters`` wrote
+    them).  They are NOT measured in this run: the entry carries the commit, the date and the
+    fingerprint of the kernel sources it was taken with, and ``current`` says whether that
+    fingerprint is still the one of the sources in the tree."""
+    if not os.path.exists(PROFILE_FILE):
+        if required:
+            raise SystemExit(f"bench.py: {PROFILE_FILE} is missing; collect counters (see --ingest-counters)")
+        return None
+    with open(PROFILE_FILE) as f:
+        entry = json.load(f).get(key)
+    if entry is None:
+        if required:
+            raise SystemExit(f"bench.py: no stored counters for '{key}' in {PROFILE_FILE}: run the kernel under "
+                             f"rocprofv3 --pmc (bench.py --profile-kernel) and ingest them with --ingest-counters, "
+                             f"or pass --no-counters to report the roofline without executed work")
+        return None
+    entry = dict(entry)
+    entry["current"] = entry.get("kernel_sha16") == kernel_fingerprint()
+    if not entry["current"]:
+        print(f"bench.py: WARNING: counters for '{key}' were taken with other kernel sources "
+              f"({entry.get('kernel_sha16')} at {entry.get('commit')}, now {kernel_fingerprint()}); "
+              f"the executed-work figures in the line are stale", file=sys.stderr)
+    return entry
+
+
+def executed_work(c: dict, launch_ms: float) -> dict:
+    """Roofline figures from executed instructions (per launch): fp32 flop actually issued =
+    512 per MFMA 'MOPS' unit (a 16x16x4 fp32 MFMA is 4 of them, 2048 flop) + 64 lanes x
+    (2 per FMA, 1 per add / mul / transcendental), against the launch time.  ``frac`` prices all
+    of it at the matrix-core peak (the published fp32 figure); ``engine_time_frac`` prices each
+    engine at its own peak (the vector ALUs run unpacked here) -- the two kinds of instruction
+    share a SIMD's issue slot, so their times add; ``issue_frac`` is the same in issue cycles
+    (4 per vector instruction, 32 per fp32 16x16x4 MFMA) for every vector instruction, flop or not."""
+    mfma_flop = c["mfma_mops_f32"] * 512.0 if "mfma_mops_f32" in c else c["mfma"] * 2048.0
+    if "fma" in c:
+        valu_flop = 64.0 * (2.0 * c["fma"] + c.get("add", 0) + c.get("mul", 0) + c.get("trans", 0))
+    else:                                   # upper bound: every non-MFMA vector instruction an FMA
+        valu_flop = 64.0 * 2.0 * (c["valu"] - c["mfma"])
+    t = launch_ms * 1e-3
+    cycles = (c["valu"] - c["mfma"]) * 4.0 + c["mfma"] * 32.0
+    issue_ms = cycles / (c.get("cus", 256) * 4 * c.get("clock_ghz", 2.4) * 1e9) * 1e3
+    engine_ms = (mfma_flop / (PEAK_FP32_TFLOPS * 1e12) + valu_flop / (PEAK_FP32_VALU_TFLOPS * 1e12)) * 1e3
+    return {"executed_tflops": round((mfma_flop + valu_flop) / t / 1e12, 3),
+            "frac": round((mfma_flop + valu_flop) / t / 1e12 / PEAK_FP32_TFLOPS, 4),
+            "mfma_flop": mfma_flop, "valu_flop": valu_flop,
+            "engine_time_frac": round(engine_ms / launch_ms, 4),
+            "issue_frac": round(issue_ms / launch_ms, 4), "issue_ms": round(issue_ms, 4),
+            "valu_insts": c["valu"], "mfma_insts": c["mfma"]}
+
+
+def host_description() -> dict:
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return {"cpu_model": model, "logical_cpus": os.cpu_count() or 1, "usable_cpus": usable}
+
+
+def cpu_threads() -> int:
+    """Threads for the CPU baseline: the cores this process may use, at most the 16 a one-GPU box grants."""
+    return max(1, min(host_description()["usable_cpus"], 16))
+
+
+def ingest_counters(directory: str, key: str, kernel: str) -> int:
+    """Average the per-dispatch counters of ``kernel`` (substring of the kernel name) and of the
+    calibration copy over every ``*counter_collection.csv`` below ``directory`` (one rocprofv3 --pmc
+    run per counter group) and store them under ``key`` in profiles/traffic.json with the commit,
+    date and kernel-source fingerprint."""
+    import collections
+    import csv
+    import datetime
+    import glob
+    import subprocess
+    agg = collections.defaultdict(lambda: collections.defaultdict(list))
+    files = glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True)
+    if not files:
+        raise SystemExit(f"bench.py: no *counter_collection.csv below {directory}")
+    for path in files:
+        per_dispatch = collections.defaultdict(lambda: collections.defaultdict(float))
+        with open(path) as f:
+            for r in csv.DictReader(f):
+                per_dispatch[(r["Kernel_Name"], r["Dispatch_Id"])][r["Counter_Name"]] += float(r["Counter_Value"])
+        for (name, _), counters in per_dispatch.items():
+            which = "copy" if "copyBuffer" in name else ("kernel" if kernel in name else None)
+            if which:
+                for cname, v in counters.items():
+                    agg[which][cname].append(v)
+    if not agg["kernel"]:
+        raise SystemExit(f"bench.py: no dispatch of a kernel named *{kernel}* in {directory}")
+    mean = lambda xs: sum(xs) / len(xs)
+    k = {c: mean(v) for c, v in agg["kernel"].items()}
+    names = {"SQ_INSTS_VALU": "valu", "SQ_INSTS_VALU_MFMA_F32": "mfma", "SQ_INSTS_VALU_FMA_F32": "fma",
+             "SQ_INSTS_VALU_ADD_F32": "add", "SQ_INSTS_VALU_MUL_F32": "mul", "SQ_INSTS_VALU_TRANS_F32": "trans",
+             "SQ_INSTS_VALU_MFMA_MOPS_F32": "mfma_mops_f32", "SQ_WAVES": "waves", "SQ_INSTS_SALU": "salu",
+             "SQ_INSTS_LDS": "lds"}
+    entry = {short: round(k[c], 1) for c, short in names.items() if c in k}
+    copy_kib = 256.0 * 1024.0
+    for cname, field in (("FETCH_SIZE", "fetch"), ("WRITE_SIZE", "write")):
+        if cname in k:
+            factor = copy_kib / mean(agg["copy"][cname]) if agg["copy"].get(cname) else None
+            entry[f"{field}_kib_counter"] = round(k[cname], 1)
+            entry[f"{field}_copy_factor"] = None if factor is None else round(factor, 4)
+            if factor is not None:
+                entry[f"{field}_bytes"] = int(k[cname] * factor * 1024)
+    if "fetch_bytes" in entry and "write_bytes" in entry:
+        entry["hbm_bytes"] = entry["fetch_bytes"] + entry["write_bytes"]
+    entry.update({"kernel": kernel, "dispatches_averaged": len(next(iter(agg["kernel"].values()))),
+                  "cus": 256, "clock_ghz": 2.4, "kernel_sha16": kernel_fingerprint(),
+                  "date": datetime.date.today().isoformat()})
+    try:
+        entry["commit"] = subprocess.check_output(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"],
+                                                  text=True).strip()
+    except Exception:
+        entry["commit"] = "unknown"
+    data = {}
+    if os.path.exists(PROFILE_FILE):
+        with open(PROFILE_FILE) as f:
+            data = json.load(f)
+    data[key] = {**data.get(key, {}), **entry} if isinstance(data.get(key), dict) and \
+        data[key].get("kernel_sha16") == entry["kernel_sha16"] else entry
+    with open(PROFILE_FILE, "w") as f:
+        json.dump(data, f, indent=1, sort_keys=True)
+    print(json.dumps({key: data[key]}, indent=1))
+    return 0
 
 
 def flop_per_eval(H: int, K: int) -> int:
@@ -121,24 +271,30 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
     # backward work per eval: the forward's accumulation twice (S and Q) + geometry and weights
     flop_bwd = evals * (23 + 4 * H + 2 + 2 * K + 4 * H * K) + float(E) * H * 3 * 2 * D * K
     bwd_ms = avg("real_enc_bwd")
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get(f"{args.config}:{args.rule}:bwd")
+    counters = stored_counters(f"{args.config}:{args.rule}:bwd", required=not args.no_counters)
+    work = executed_work(counters, bwd_ms) if (counters and bwd_ms > 0) else None
     roofline = {
         "kernel": "real_enc_bwd_pair_kernel + reductions (periodic encoding backward)",
-        "bound": "mfma", "achieved": round(flop_bwd / (bwd_ms * 1e-3) / 1e12, 3) if bwd_ms > 0 else 0.0,
-        "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(flop_bwd / (bwd_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4) if bwd_ms > 0 else 0.0,
-        "traffic": traffic, "avg_launch_ms": bwd_ms,
+        "bound": "mfma", "achieved": work["executed_tflops"] if work else None,
+        "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": work["frac"] if work else None,
+        "peaks": {"mfma_fp32": PEAK_FP32_TFLOPS, "valu_fp32_unpacked": PEAK_FP32_VALU_TFLOPS},
+        "executed": work,
+        "counters_from": None if not counters else {k: counters.get(k) for k in
+                                                    ("commit", "date", "kernel_sha16", "current")},
+        "traffic": counters.get("hbm_bytes") if counters else None,
+        "traffic_note": "HBM bytes per launch from the stored rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs "
+                        "(not measured in this run)" if counters else None,
+        "avg_launch_ms": bwd_ms,
+        "algorithmic_equivalent": {"tflops": round(flop_bwd / (bwd_ms * 1e-3) / 1e12, 3) if bwd_ms > 0 else 0.0},
         "note": "HIP event pairs around cf_real_enc_bwd (pair kernel + its two fixed-order reductions), the "
                 "step's four launches re-issued back to back",
         "real_enc_fwd_avg_ms": avg("real_enc_fwd"), "fused_dpa_fwd_avg_ms": avg("fused_dpa_fwd"),
         "fused_dpa_bwd_avg_ms": avg("fused_dpa_bwd"),
     }
     cpu_baseline = None
+    parity = None
     if not args.skip_cpu_baseline:
+        from crystalformer_amd.latticeformer import Latticeformer
         # bounded sample: the first 64 crystals of the batch, one training-mode forward + backward on the CPU oracle
         from oracle import torch_model as om
         from crystalformer_amd.synthetic import CrystalBatch
@@ -148,21 +304,48 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
                            batch.y[:nb])
         ocfg = type(cfg)(**{**vars(cfg), "adaptive_cutoff_sigma": 0.0})
         P = {k: v.clone().requires_grad_("scale" not in k and v.dtype.is_floating_point) for k, v in state_cpu.items()}
-        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        torch.set_num_threads(cpu_threads())
         reps, cpu_s = 0, 0.0
         while reps < 8 and cpu_s < 12.0:            # bounded sample: about 12 s of host work
-            for v in P.values():
+            for name, v in P.items():
                 v.grad = None
+                if "gauss_scale" in name:           # every repeat starts from the initial state
+                    with torch.no_grad():
+                        v.copy_(state_cpu[name])
             t0 = time.perf_counter()
-            y = om.latticeformer_forward(P, ocfg, sub, training=True)
-            torch.nn.functional.l1_loss(y[:, 0], sub.y).backward()
+            y_cpu = om.latticeformer_forward(P, ocfg, sub, training=True)
+            loss_cpu = torch.nn.functional.l1_loss(y_cpu[:, 0], sub.y)
+            loss_cpu.backward()
             cpu_s += time.perf_counter() - t0
             reps += 1
         cpu_baseline = {"value": round(nb * reps / cpu_s, 3), "unit": "crystals/s",
-                        "cores": torch.get_num_threads(), "kind": "port",
+                        "cores": torch.get_num_threads(), "kind": "port", **host_description(),
                         "sample": f"{reps} x forward + backward (autograd) of the first {nb} crystals "
                                   f"({int((sub.sizes ** 2).sum())} edges) on the CPU oracle, {cpu_s:.1f} s in all; "
                                   f"no optimiser step"}
+        # parity of the step's gradients: the same sub-batch and initial weights through the HIP path
+        if args.rule == "A":
+            twin = Latticeformer(cfg)
+            twin.load_state_dict(state_cpu)
+            twin.to(data.pos.device).train()
+            subd = sub.to(data.pos.device)
+            yg = twin(subd)
+            lg = torch.nn.functional.l1_loss(yg[:, 0], subd.y)
+            lg.backward()
+            worst, worst_name = 0.0, ""
+            for name, prm in twin.named_parameters():
+                ref = P[name].grad
+                if prm.grad is None or ref is None:
+                    continue
+                err = float((prm.grad.cpu().double() - ref.double()).abs().max() / max(float(ref.abs().max()), 1e-30))
+                if err > worst:
+                    worst, worst_name = err, name
+            parity = {"loss_rel_err": abs(float(lg) - float(loss_cpu)) / abs(float(loss_cpu)),
+                      "output_rel_err": float((yg.detach().cpu().double() - y_cpu.detach().double()).abs().max()
+                                              / y_cpu.detach().abs().max()),
+                      "worst_grad_rel_err": worst, "worst_grad": worst_name,
+                      "note": f"training-mode forward + L1 loss + backward on the first {nb} crystals, HIP path "
+                              f"against autograd through the float32 CPU oracle; per tensor max|x-ref|/max|ref|"}
     out = {
         "metric": "crystals/sec train step (fwd+bwd+AdamW, 4-block default, B=128)",
         "value": round(B * args.steps / elapsed, 2), "unit": "crystals/s", "n_gpus": 1, "steps": args.steps,
@@ -172,6 +355,7 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
                    "heads": H, "value_pe_bins": K, "translation_rule": args.rule, "optimizer": "AdamW lr 5e-4",
                    "loss": "L1", "submission": submission},
         "eager": eager, "final_loss": float(loss), "roofline": roofline, "cpu_baseline": cpu_baseline,
+        "parity_vs_cpu": parity,
     }
     print(json.dumps(out))
     return 0
@@ -197,6 +381,7 @@ def main() -> int:
     ap.add_argument("--launch-share", type=float, default=0.75,
                     help="with several steps in flight: share of the GPU one periodic-encoding launch "
                          "occupies (384 of its 512 work-groups by default)")
+    ap.add_argument("--no-fresh", action="store_true", help="skip the fresh-batch (layout rebuilt every step) figure")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--train", action="store_true",
                     help="time full training steps (forward + backward + AdamW) instead of forwards")
@@ -204,7 +389,20 @@ def main() -> int:
                     help="counter-collection helper: launch only a 256 MiB device copy (calibration) and the "
                          "periodic-encoding kernel on the workload (with --train: its backward), 5 times each, "
                          "and exit")
+    ap.add_argument("--no-counters", action="store_true",
+                    help="do not require stored hardware counters for this workload: roofline.frac is then null")
+    ap.add_argument("--ingest-counters", metavar="DIR",
+                    help="no benchmark: read the rocprofv3 --pmc CSVs below DIR (runs of --profile-kernel) and store "
+                         "the per-launch counters in profiles/traffic.json under --ingest-key")
+    ap.add_argument("--ingest-key", default=None, help="default: <config>:<rule>:fwd (or :bwd with --train)")
+    ap.add_argument("--ingest-kernel", default=None, help="kernel name substring (default: the pair kernel)")
     args = ap.parse_args()
+
+    if args.ingest_counters:
+        cfg_name = "cfg4_train_b128" if (args.train and args.config == "cfg2_default_b128") else args.config
+        key = args.ingest_key or f"{cfg_name}:{args.rule}:{'bwd' if args.train else 'fwd'}"
+        kernel = args.ingest_kernel or ("real_enc_bwd_pair_kernel" if args.train else "real_enc_fwd_pair_kernel")
+        return ingest_counters(args.ingest_counters, key, kernel)
 
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (every kernel works on one GPU's share of crystals; "
@@ -352,20 +550,34 @@ def main() -> int:
     D = cfg.model_dim // H
     H_enc = H // 2 if args.domain == "multihead" else H     # heads served by the real-space kernel
     flop_launch = evals_per_launch * flop_per_eval(H_enc, K) + (float(E) * H_enc * 2 * D * K if K > 0 else 0.0)
-    achieved_tflops = flop_launch / (enc_avg_ms * 1e-3) / 1e12 if enc_avg_ms > 0 else 0.0
+    algorithmic_tflops = flop_launch / (enc_avg_ms * 1e-3) / 1e12 if enc_avg_ms > 0 else 0.0
+    counters = None if args.domain != "real" else stored_counters(f"{args.config}:{args.rule}:fwd",
+                                                                  required=not args.no_counters)
+    work = executed_work(counters, enc_avg_ms) if (counters and enc_avg_ms > 0) else None
     roofline = {
         "kernel": "real_enc_fwd_pair_kernel (periodic encoding forward, projection fused)",
         "bound": "mfma",
-        "achieved": round(achieved_tflops, 3),
+        # executed fp32 work (instruction counters of a stored rocprofv3 --pmc run of this kernel
+        # on this workload) over the launch time measured in this run
+        "achieved": work["executed_tflops"] if work else None,
         "peak": PEAK_FP32_TFLOPS,
         "unit": "TFLOP/s",
-        "frac": round(achieved_tflops / PEAK_FP32_TFLOPS, 4),
-        "traffic": None,
+        "frac": work["frac"] if work else None,
+        "peaks": {"mfma_fp32": PEAK_FP32_TFLOPS, "valu_fp32_unpacked": PEAK_FP32_VALU_TFLOPS},
+        "executed": work,
+        "counters_from": None if not counters else {k: counters.get(k) for k in
+                                                    ("commit", "date", "kernel_sha16", "current")},
+        "traffic": counters.get("hbm_bytes") if counters else None,
+        "traffic_note": "HBM bytes per launch from the stored rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs "
+                        "(not measured in this run)" if counters else None,
         "launches_timed": len(enc_ms),
         "avg_launch_ms": round(enc_avg_ms, 4),
-        "evals_per_launch": evals_per_launch,
-        "g_evals_per_s": round(evals_per_launch / (enc_avg_ms * 1e-3) / 1e9, 3) if enc_avg_ms > 0 else 0.0,
-        "flop_per_eval": flop_per_eval(H, K),
+        # the reference's work per (edge, translation) evaluation, which the kernel does not execute
+        # term by term (Gaussians once per atom pair, only inside their window, negligible terms skipped)
+        "algorithmic_equivalent": {
+            "tflops": round(algorithmic_tflops, 3), "flop_per_eval": flop_per_eval(H_enc, K),
+            "evals_per_launch": evals_per_launch,
+            "g_evals_per_s": round(evals_per_launch / (enc_avg_ms * 1e-3) / 1e9, 3) if enc_avg_ms > 0 else 0.0},
         "fused_dpa_fwd_avg_ms": round(sum(dpa_ms) / max(len(dpa_ms), 1), 4),
     }
     # the attention kernel is the memory-bound one: algorithmic bytes per edge 4 H (Dv + 2)
@@ -377,25 +589,27 @@ def main() -> int:
                                      "peak": 8000.0, "unit": "GB/s",
                                      "frac": round(dpa_bytes / (dpa_avg_ms * 1e-3) / 1e9 / 8000.0, 4),
                                      "avg_launch_ms": round(dpa_avg_ms, 4)}
-    traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(traffic_file):
-        try:
-            with open(traffic_file) as f:
-                tr = json.load(f).get(f"{args.config}:{args.rule}")
-            if tr:
-                roofline["traffic"] = tr
-            with open(traffic_file) as f:
-                ins = json.load(f).get(f"{args.config}:{args.rule}:insts")
-            if ins and enc_avg_ms > 0:
-                # the kernel's own bound, from its rocprofv3 instruction counters: a wave64 vector
-                # instruction occupies its SIMD for 4 cycles, an fp32 16x16x4 MFMA for 32, and the
-                # two do not overlap in this kernel; 4 SIMDs per CU at the peak engine clock
-                cycles = (ins["valu"] - ins["mfma"]) * 4.0 + ins["mfma"] * 32.0
-                issue_ms = cycles / (ins["cus"] * 4 * ins["clock_ghz"] * 1e9) * 1e3
-                roofline["issue"] = {"valu_insts": ins["valu"], "mfma_insts": ins["mfma"],
-                                     "issue_ms": round(issue_ms, 4), "frac": round(issue_ms / enc_avg_ms, 4)}
-        except Exception:
-            pass
+
+    # ---- forwards over batches never seen before: every step a batch with other crystal sizes, so
+    # the layout (offsets, edge list, pair list) is rebuilt and no captured graph can be reused
+    fresh = None
+    if not args.no_fresh:
+        from crystalformer_amd.synthetic import make_batch
+        pool = [make_batch(seed=args.seed + 1000 + k, **CONFIGS[args.config]["batch"]).to(dev)
+                for k in range(min(args.steps + args.warmup, 48))]
+        turn = [0]
+
+        def fresh_step():
+            ops._index_cache.clear()                      # a batch whose layout is in no cache
+            b = pool[turn[0] % len(pool)]
+            turn[0] += 1
+            return model(b)
+        with torch.no_grad():
+            fresh_elapsed, _ = timed(fresh_step, args.steps, max(args.warmup, 2))
+        crystals = sum(int(pool[(max(args.warmup, 2) + k) % len(pool)].sizes.numel()) for k in range(args.steps))
+        fresh = {"value": round(crystals / fresh_elapsed, 2), "ms_per_step": round(fresh_elapsed / args.steps * 1e3, 4),
+                 "note": f"eager forwards over {len(pool)} different batches of the same distribution in turn, index "
+                         f"caches emptied before every step: one host read of the sizes + layout rebuild per step"}
 
     # ---- CPU baseline: the oracle's restated PyTorch path on the host cores
     cpu_baseline = None
@@ -403,7 +617,7 @@ def main() -> int:
     if not args.skip_cpu_baseline:
         from oracle import torch_model as om
         ocfg = default_params(adaptive_cutoff_sigma=0.0, **mcfg)
-        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        torch.set_num_threads(cpu_threads())
         with torch.no_grad():
             reps, cpu_s = 0, 0.0
             while reps < 8 and cpu_s < 12.0:        # bounded sample: about 12 s of host work
@@ -413,7 +627,7 @@ def main() -> int:
                 reps += 1
         cpu_baseline = {
             "value": round(B * reps / cpu_s, 3), "unit": "crystals/s", "cores": torch.get_num_threads(),
-            "kind": "port",
+            "kind": "port", **host_description(),
             "sample": f"{reps} forwards of the same {B}-crystal batch and weights (fixed cube of 125 "
                       f"translations), {cpu_s:.1f} s in all",
         }
@@ -445,6 +659,7 @@ def main() -> int:
         "single_stream": None if args.no_graph else single,
         "eager": {"value": round(B * args.steps / eager_elapsed, 2),
                   "ms_per_step": round(eager_elapsed / args.steps * 1e3, 4)},
+        "fresh_batch": fresh,
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
         "parity_rel_err_vs_cpu": parity,

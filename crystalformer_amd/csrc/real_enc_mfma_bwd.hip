@@ -4,6 +4,7 @@
 // Per directed edge and head, with p_t = exp(a d2_t - z):
 //     PX = sum_t p_t d2_t,  S_k = sum_t p_t g_k(t),  Q_k = sum_t p_t d2_t g_k(t)
 //     ga_edge = gz PX + gv.(W Q) - PX gv.(W S)          (gradient wrt the exponent a)
+//             = gz PX + gv.(W (Q - PX S))
 //     gW     += gv (x) S                                 (gradient wrt the projection)
 // Same decomposition as the forward kernel: a unit is an unordered atom pair, its
 // Gaussians are evaluated once per translation for 2 x 16 weight columns
@@ -75,11 +76,12 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     };
     // edge of product column c of round rd_: direction c/8 of the unit of wave c%8
     // (-1: no such unit, or the reverse of a self edge)
-    auto load_col_edge = [&](int rd_, const RoundPos &rp) -> int64_t {
+    // (32-bit: the launcher refuses edge counts of 2^31 and more)
+    auto load_col_edge = [&](int rd_, const RoundPos &rp) -> int {
         const int64_t u_ = (int64_t)rp.r * WPB + (c & 7);
         if (rd_ >= rounds || u_ >= p.U) return -1;
         const int64_t e0 = g_pairs[u_ * PAIR_FIELDS], e1 = g_pairs[u_ * PAIR_FIELDS + 1];
-        return (c < 8) ? e0 : (e1 != e0 ? e1 : -1);
+        return (int)((c < 8) ? e0 : (e1 != e0 ? e1 : -1));
     };
     auto flush_gW = [&](int hg_) {
         // lane (q, j) holds gW[d = 4q + r][bin = 16t + j] of head hg_*8 + wave
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     float a_cur, z_cur;
     UnitGeom geo;
     UnitIds ids_next;
-    int64_t col_edge = load_col_edge(blockIdx.x, pos);
+    int col_edge = load_col_edge(blockIdx.x, pos);
     {
         const float gv0 = load_unit_geom(ids, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
         a_cur = load_a(ids, pos);
@@ -120,8 +122,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         const float gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
         const float a_next = load_a(ids_next, pos_next);
         const float z_next = load_z(ids_next, pos_next);
-        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane);
-        const int64_t col_edge_next = load_col_edge(rd + stride, pos_next);
+        const int col_edge_next = load_col_edge(rd + stride, pos_next);
         if (hg != wa_hg) {
             if (wa_hg >= 0) flush_gW(wa_hg);
 #pragma unroll
@@ -274,9 +275,11 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             }
             wave_mem_sync();
         }
-        // the loads issued at the top of the round have landed
+        // the loads issued at the top of the round have landed; the descriptor of the round after
+        // next is requested here and looked at after the exchange (it would otherwise occupy two
+        // registers through the whole accumulation)
         const UnitGeom geo_next = unit_geom(gv_next, !UNIFORM);
-        const UnitIds ids_next2 = unit_ids(dv_next2);
+        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane);
         px += __shfl_xor(px, 16, WAVE);
         px += __shfl_xor(px, 32, WAVE);
 
@@ -285,16 +288,17 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         const int hw = hg * 8 + wave;
         const int jcol = c, unit_j = jcol & 7, dir_j = jcol >> 3;    // product column j = dir*8 + unit
         const float *src = Sbuf + xch_base(q, wave, unit_j, dir_j);
-        float dotS = 0.f, dotQ = 0.f;
         // projection operands of this wave's head (W stays in cache across rounds)
         float Wa[4 * NT];
         if (hw < H && K == 16 * NT && D == 16) {
             // full tiles: one base address per lane, 16-byte loads at fixed offsets
             // (proj_bin(s, q) = 16 (s / 4) + 4 q + s % 4)
-            const float *wrow = p.W + ((int64_t)hw * D + c) * K + 4 * q;
+            // (wave-uniform base + 32-bit lane offset: no 64-bit address per lane kept across rounds)
+            const float *wbase = p.W + (int64_t)hw * D * K;
+            const unsigned woff = (unsigned)(c * K + 4 * q);
 #pragma unroll
             for (int t4 = 0; t4 < NT; t4++) {
-                const float4_t w4 = *reinterpret_cast<const float4_t *>(wrow + 16 * t4);
+                const float4_t w4 = *reinterpret_cast<const float4_t *>(wbase + (woff + 16u * t4));
 #pragma unroll
                 for (int r = 0; r < 4; r++) Wa[4 * t4 + r] = w4[r];
             }
@@ -312,6 +316,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         float gz_out = 0.f;
         float gvk[4] = {0.f, 0.f, 0.f, 0.f};
         if (hw < H) {
+            if (e_out >= 0 && g_gz && q == 0) gz_out = g_gz[e_out * H + hw];
             if (e_out >= 0 && g_gv) {
                 const float *gp = g_gv + (e_out * H + hw) * D + 4 * q;
                 if (4 * q + 3 < D) {
@@ -322,18 +327,19 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                         if (4 * q + r < D) gv4[r] = gp[r];
                 }
             }
-            if (e_out >= 0 && g_gz && q == 0) gz_out = g_gz[e_out * H + hw];
-            if (p.gW_part && g_gv) {
-#pragma unroll
-                for (int s4 = 0; s4 < 4; s4++) {
-                    const int64_t e_k = __shfl(col_edge, 4 * s4 + q, WAVE);      // column 4*s4 + q
-                    if (e_k >= 0 && c < D) gvk[s4] = g_gv[(e_k * H + hw) * D + c];
-                }
-            }
         }
+        // With PX in hand the two projected sums collapse into one: gv.(W Q) - PX gv.(W S) =
+        // gv.(W Q'), Q' = Q - PX S, formed here on the unit's own columns (px is complete in
+        // every lane of a column).  One projection instead of two, and S crosses the exchange
+        // only for the weight gradient.
 #pragma unroll
-        for (int pass = 0; pass < 2; pass++) {
-            // pass 0 exchanges S (also feeds gW), pass 1 exchanges Q
+        for (int m = 0; m < NT; m++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) accQ[m][r] = fmaf(-px, accS[m][r], accQ[m][r]);
+        const int passes = p.gW_part ? 2 : 1;
+        for (int pass = 0; pass < passes; pass++) {
+            // pass 0 exchanges Q' (projection, dot with gv, ga), pass 1 exchanges S (gW update):
+            // Q' first, so that its accumulators are dead before the gW block comes in from LDS
             {
                 float *col = Sbuf + xch_base(q, c & 7, wave, c >> 3);
 #pragma unroll
@@ -341,34 +347,39 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
                         // (inactive columns hold zeros: their weights are masked in the loop)
-                        col[(4 * m + r) * XPLANE] = pass == 0 ? accS[m][r] : accQ[m][r];
+                        col[(4 * m + r) * XPLANE] = pass == 0 ? accQ[m][r] : accS[m][r];
                     }
             }
             __syncthreads();
-            float4_t out = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int t4 = 0; t4 < NT; t4++) {
-                float sb[4];
-#pragma unroll
-                for (int r = 0; r < 4; r++) sb[r] = src[(4 * t4 + r) * XPLANE];
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    out = __builtin_amdgcn_mfma_f32_16x16x4f32(Wa[4 * t4 + r], sb[r], out, 0, 0, 0);
-            }
-            // lane (q, j): components d = 4q + r of (W S) or (W Q) for column j; dot with gv
-            float dot = out[0] * gv4[0] + out[1] * gv4[1] + out[2] * gv4[2] + out[3] * gv4[3];
-            dot += __shfl_xor(dot, 16, WAVE);
-            dot += __shfl_xor(dot, 32, WAVE);
             if (pass == 0) {
-                dotS = dot;
-            } else {
-                dotQ = dot;
+                float4_t out = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t4 = 0; t4 < NT; t4++) {
+                    float sb[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) sb[r] = src[(4 * t4 + r) * XPLANE];
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        out = __builtin_amdgcn_mfma_f32_16x16x4f32(Wa[4 * t4 + r], sb[r], out, 0, 0, 0);
+                }
+                // lane (q, j): components d = 4q + r of W Q' for column j; dot with gv
+                float dot = out[0] * gv4[0] + out[1] * gv4[1] + out[2] * gv4[2] + out[3] * gv4[3];
+                dot += __shfl_xor(dot, 16, WAVE);
+                dot += __shfl_xor(dot, 32, WAVE);
                 if (q == 0 && e_out >= 0 && hw < H) {
                     const float PX = PXbuf[unit_j * 16 + dir_j * 8 + wave];
-                    p.ga_edge[e_out * H + hw] = PX * gz_out + (dotQ - PX * dotS);
+                    p.ga_edge[e_out * H + hw] = fmaf(PX, gz_out, dot);
                 }
-            }
-            if (pass == 0 && p.gW_part) {
+                // operands of the gW update of the next pass, requested now so that they arrive
+                // while S is being exchanged
+                if (hw < H && p.gW_part && g_gv) {
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; s4++) {
+                        const int64_t e_k = __shfl(col_edge, 4 * s4 + q, WAVE);      // column 4*s4 + q (sign-extended)
+                        if (e_k >= 0 && c < D) gvk[s4] = g_gv[(e_k * H + hw) * D + c];
+                    }
+                }
+            } else {
                 // gW_h[d][bin] += sum over the 16 columns of gv[col][d] * S[bin][col]
                 // A[i = d][k = col], B[k = col][j = bin]; column 4*s4 + kk
                 float4_t gWacc[NT];
@@ -393,7 +404,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         geo = geo_next;
         a_cur = a_next;
         z_cur = z_next;
-        ids_next = ids_next2;
+        ids_next = unit_ids(dv_next2);
         col_edge = col_edge_next;
         pos = pos_next;
         pos_next = pos_next2;
@@ -500,6 +511,7 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
     const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)4 * NT * XPLANE + WPB * 16 +
                                         (size_t)WPB * NT * WAVE * 4) + 16;
     if (((U + WPB - 1) / WPB) * ((H + 7) / 8) >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // 32-bit round positions
+    if (E >= (1ll << 31)) return CF_ERR_UNSUPPORTED;                                        // 32-bit column edge ids
     const int blocks = real_enc_bwd_pairs_blocks(U, H);
 #define CF_BPAIR(NTV)                                                                              \
     do {                                                                                           \

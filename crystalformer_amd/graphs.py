@@ -19,6 +19,22 @@ from . import ops
 from .synthetic import CrystalBatch
 
 
+def _same_layout(owner, batch: CrystalBatch) -> None:
+    """Raise unless ``batch`` has exactly the crystal sizes the graph of ``owner`` was captured
+    with: edges, pair list and row offsets are baked into it.  The comparison reads ``sizes``
+    back once per tensor (identity and version are remembered)."""
+    if batch.pos.shape != owner.static.pos.shape or batch.sizes.shape != owner.static.sizes.shape:
+        raise ValueError("batch layout differs from the captured one")
+    key = (id(batch.sizes), batch.sizes.data_ptr(), batch.sizes._version)
+    if key in owner._checked:
+        return
+    if batch.sizes.tolist() != owner._sizes_host:
+        raise ValueError("crystal sizes differ from the captured batch (same totals, other layout)")
+    if len(owner._checked) > 64:
+        owner._checked.clear()
+    owner._checked[key] = batch.sizes          # keeps the tensor alive: its identity stays unique
+
+
 class GraphedForward:
     """Capture ``model(batch)`` (inference, no autograd) and replay it.
 
@@ -40,6 +56,7 @@ class GraphedForward:
                                    batch.trans_vec.clone(), batch.sizes.clone(),
                                    None if batch.y is None else batch.y.clone())
         self._sizes_host = batch.sizes.tolist()
+        self._checked: dict = {}
         self.graph = torch.cuda.CUDAGraph()
         stream = torch.cuda.Stream()            # default priority
         stream.wait_stream(torch.cuda.current_stream())
@@ -56,8 +73,7 @@ class GraphedForward:
 
     def __call__(self, batch: Optional[CrystalBatch] = None) -> torch.Tensor:
         if batch is not None and batch is not self.static:
-            if batch.pos.shape != self.static.pos.shape or batch.sizes.shape != self.static.sizes.shape:
-                raise ValueError("batch layout differs from the captured one")
+            _same_layout(self, batch)
             self.static.x.copy_(batch.x)
             self.static.pos.copy_(batch.pos)
             self.static.trans_vec.copy_(batch.trans_vec)
@@ -91,6 +107,8 @@ class GraphedTrainStep:
         self.model = model
         self.static = CrystalBatch(batch.x.clone(), batch.pos.clone(), batch.batch.clone(),
                                    batch.trans_vec.clone(), batch.sizes.clone(), batch.y.clone())
+        self._sizes_host = batch.sizes.tolist()
+        self._checked: dict = {}
         self.clip_norm = clip_norm
         self.lr0, self.decay = lr, sch_decay
         # clip + AdamW + schedule as one device-side update; its step counter lives on the device
@@ -119,8 +137,7 @@ class GraphedTrainStep:
 
     def __call__(self, batch: Optional[CrystalBatch] = None) -> torch.Tensor:
         if batch is not None and batch is not self.static:
-            if batch.pos.shape != self.static.pos.shape or batch.sizes.shape != self.static.sizes.shape:
-                raise ValueError("batch layout differs from the captured one")
+            _same_layout(self, batch)
             self.static.x.copy_(batch.x)
             self.static.pos.copy_(batch.pos)
             self.static.trans_vec.copy_(batch.trans_vec)

@@ -60,8 +60,10 @@ class KernelManager:
     # The edge list is the dense per-crystal block layout of get_edge_index
     # (edge (i,j) of a crystal with n atoms at e0 + i*n + j).  The reference's
     # transposes assume it too (models/cuda_funcs/fused_dpa.py:141-159).  With it
-    # the encoding evaluates both directions of an atom pair together; set False
-    # for arbitrary edge lists (per-edge kernels; attention backward unavailable).
+    # the encoding evaluates both directions of an atom pair together.  An edge
+    # list is checked against that layout the first time it is seen: any other list
+    # takes the per-edge kernels, and the attention backward raises for it.  False
+    # forces the per-edge kernels.
     DENSE_EDGE_BLOCKS: bool = True
     # The reference's reciprocal-space backward kernel differentiates log(sum) only and drops
     # d/da of the normalisation term 1.5 log(-4 pi a) (models/kernels/reci_enc_bwd.cu:41-69),

@@ -332,6 +332,11 @@ def fused_dpa_bwd(que: Tensor, key: Tensor, val: Tensor, bij_ehd: Optional[Tenso
     N, H, Dk = que.shape
     Dv = val.shape[-1]
     E = edge_ij_e.shape[1]
+    # the key-side kernel walks the column (i,j) of a crystal's block at e0 + i*n + j
+    if cached_dense_sizes(batch_i, edge_ij_e) is None:
+        raise _lib.CrystalformerHipError(
+            "fused_dpa_bwd needs the dense per-crystal edge blocks of get_edge_index "
+            "(sorted batch_i, edge (i,j) at e0 + i*n + j); this edge list is not of that form")
     if atom_start_n is None or edge_start_n is None:
         atom_start_n, edge_start_n = cached_crystal_offsets(batch_i)
     atom_start_n, edge_start_n = _i64(atom_start_n, "atom_start_n"), _i64(edge_start_n, "edge_start_n")
@@ -452,13 +457,60 @@ def cached_edge_row_offsets(edge_ij_e: Tensor, num_atoms: int) -> Tensor:
     return _cache_store(sig, (edge_ij_e,), edge_row_offsets(edge_ij_e, num_atoms))
 
 
-def cached_edge_pairs(batch_i: Tensor, edge_ij_e: Tensor, num_crystals: int) -> Tensor:
-    """Pair list for a dense per-crystal edge layout (see :func:`edge_pairs`)."""
+def dense_block_layout(batch_i: Tensor, edge_ij_e: Tensor) -> Optional[Tensor]:
+    """Crystal sizes (B,) if ``edge_ij_e`` is exactly the dense per-crystal block list of
+    ``get_edge_index`` for the crystals of ``batch_i`` (atoms of a crystal contiguous, edge
+    (i,j) of a crystal with n atoms at e0 + i*n + j), else ``None``.  Plain torch ops on the
+    tensors' own device; reads three small results back to the host, so it is meant for the
+    first sight of a batch, not for every launch."""
+    N, E = batch_i.numel(), edge_ij_e.shape[1]
+    dev = batch_i.device
+    if edge_ij_e.dim() != 2 or edge_ij_e.shape[0] != 2:
+        return None
+    if N == 0:
+        return torch.zeros(0, dtype=torch.int64, device=dev) if E == 0 else None
+    head = torch.stack([(batch_i[1:] >= batch_i[:-1]).all().long(), batch_i[0], batch_i[-1]]).tolist()
+    if not head[0] or head[1] < 0 or head[2] >= (1 << 24):
+        return None
+    B = head[2] + 1                       # crystal ids index the lattices as they are
+    sizes = torch.zeros(B, dtype=torch.int64, device=dev)
+    sizes.scatter_add_(0, batch_i, torch.ones_like(batch_i))
+    if int((sizes * sizes).sum().item()) != E:
+        return None
+    atom_start = F.pad(sizes.cumsum(0), (1, 0))
+    edge_start = F.pad((sizes * sizes).cumsum(0), (1, 0))
+    crystal = torch.repeat_interleave(torch.arange(B, device=dev), sizes * sizes, output_size=E)
+    local = torch.arange(E, device=dev) - edge_start[crystal]
+    n_e = sizes[crystal]
+    dense = torch.stack([local // n_e, local % n_e]) + atom_start[crystal]
+    return sizes if torch.equal(dense, edge_ij_e) else None
+
+
+def cached_dense_sizes(batch_i: Tensor, edge_ij_e: Tensor) -> Optional[Tensor]:
+    """:func:`dense_block_layout`, verified once per (batch_i, edge_ij_e) pair."""
+    sig, hit = _cache_lookup("dense", batch_i, edge_ij_e)
+    if hit is not None:
+        return hit[0]
+    if batch_i.is_cuda and torch.cuda.is_current_stream_capturing():
+        raise _lib.CrystalformerHipError(
+            "an edge list first seen under stream capture cannot be checked for the dense block "
+            "layout (the check reads back to the host): run one eager call on it first")
+    return _cache_store(sig, (batch_i, edge_ij_e), (dense_block_layout(batch_i, edge_ij_e),))[0]
+
+
+def cached_edge_pairs(batch_i: Tensor, edge_ij_e: Tensor, num_crystals: int) -> Optional[Tensor]:
+    """Pair list (see :func:`edge_pairs`) if the edge list is the dense per-crystal block
+    layout, verified on first sight; ``None`` for any other edge list (the callers then take
+    the per-edge kernels, which read the list as it is)."""
     sig, hit = _cache_lookup("pairs", batch_i, edge_ij_e)
     if hit is not None:
         return hit
-    sizes = torch.zeros(num_crystals, dtype=torch.int64, device=batch_i.device)
-    sizes.scatter_add_(0, batch_i, torch.ones_like(batch_i))
+    sizes = cached_dense_sizes(batch_i, edge_ij_e)
+    if sizes is None:
+        return None
+    if sizes.numel() > num_crystals:
+        raise _lib.CrystalformerHipError(
+            f"batch_i names {sizes.numel()} crystals but only {num_crystals} lattices were given")
     pairs = edge_pairs(sizes, batch_i.numel(), edge_ij_e.shape[1])
     return _cache_store(sig, (batch_i, edge_ij_e), pairs)
 
@@ -522,6 +574,8 @@ def batch_layout(sizes: Tensor, batch_i: Tensor) -> BatchLayout:
     if lay.pairs is not None:
         s_, _ = _cache_lookup("pairs", lay.batch, lay.edges)
         _cache_store(s_, (lay.batch, lay.edges), lay.pairs)
+    s_, _ = _cache_lookup("dense", lay.batch, lay.edges)       # dense by construction
+    _cache_store(s_, (lay.batch, lay.edges), (sizes,))
     s_, _ = _cache_lookup("offsets", lay.batch)
     _cache_store(s_, (lay.batch,), (lay.atom_start, lay.edge_start))
     s_, _ = _cache_lookup("mean_start", sizes)

@@ -119,3 +119,14 @@ CONFIGS = {
 
 def make_config_batch(name: str, seed: int = 0) -> CrystalBatch:
     return make_batch(seed=seed, **CONFIGS[name]["batch"])
+
+
+def select_crystals(b: CrystalBatch, crystals) -> CrystalBatch:
+    """The batch made of the listed crystals of ``b`` (in the order given), renumbered from 0."""
+    idx = torch.as_tensor(list(crystals), dtype=torch.long)
+    start = torch.cat([torch.zeros(1, dtype=torch.long), b.sizes.cumsum(0)])
+    atoms = torch.cat([torch.arange(int(start[c]), int(start[c + 1])) for c in idx.tolist()])
+    sizes = b.sizes[idx]
+    batch = torch.repeat_interleave(torch.arange(idx.numel()), sizes)
+    return CrystalBatch(b.x[atoms], b.pos[atoms].contiguous(), batch, b.trans_vec[idx].contiguous(), sizes,
+                        None if b.y is None else b.y[idx])

@@ -89,9 +89,27 @@ def real_enc_fwd(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wsca
     return z, v
 
 
+def real_enc_fwd_cond(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, rvlen_n=None,
+                      cutoff_radius=0.0, lattice_range=2, minimum_range=0) -> Tensor:
+    """(E,H,K) first-order float32 conditioning of the Gaussian averages (see kernels_ref.c):
+    a tolerance, not a restatement of reference code."""
+    a_ik, rpos_ij_e, tvecs_n, rvlen_n = _f(a_ik), _f(rpos_ij_e), _f(tvecs_n), _f(rvlen_n)
+    batch_i, edge_ij_e = _l(batch_i), _l(edge_ij_e)
+    N, H = a_ik.shape
+    E = edge_ij_e.shape[1]
+    cond = torch.empty((E, H, K), dtype=torch.float32)
+    lib().ref_real_enc_fwd_cond(_p(a_ik), _p(rpos_ij_e), _p(tvecs_n), _p(batch_i), _p(edge_ij_e), _i64(N),
+                                _i64(H), _i64(E), _i64(K), _dbl(dist_max), _dbl(wscale), _p(rvlen_n),
+                                _dbl(cutoff_radius if cutoff_radius is not None else 0.0),
+                                _int(lattice_range), _int(minimum_range), _p(cond))
+    return cond
+
+
 def real_enc_bwd(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd,
                  K, dist_max, wscale, W_k=None, rvlen_n=None, cutoff_radius=0.0,
-                 lattice_range=2, minimum_range=0) -> Tuple[Tensor, Optional[Tensor]]:
+                 lattice_range=2, minimum_range=0, magnitude=False) -> Tuple[Tensor, Optional[Tensor]]:
+    """``magnitude``: the same sums over the magnitudes of their terms (a tolerance for the
+    tests, see kernels_ref.c), not the gradients."""
     a_ik, rpos_ij_e, tvecs_n = _f(a_ik), _f(rpos_ij_e), _f(tvecs_n)
     batch_i, edge_ij_e, e_start_i = _l(batch_i), _l(edge_ij_e), _l(e_start_i)
     W_k, rvlen_n, z_ek, gz_ek, gv_ekd = _f(W_k), _f(rvlen_n), _f(z_ek), _f(gz_ek), _f(gv_ekd)
@@ -104,12 +122,11 @@ def real_enc_bwd(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, 
         D = W_k.shape[-2]
         gW = torch.zeros_like(W_k)
     ga = torch.empty_like(a_ik)
-    lib().ref_real_enc_bwd(_p(a_ik), _p(rpos_ij_e), _p(tvecs_n), _p(batch_i), _p(edge_ij_e),
-                           _p(e_start_i), _p(z_ek), _p(gz_ek), _p(gv_ekd), _i64(N), _i64(H),
-                           _i64(E), _i64(K), _i64(D), _dbl(dist_max), _dbl(wscale), _p(W_k),
-                           _i64(W_num), _p(rvlen_n),
-                           _dbl(cutoff_radius if cutoff_radius is not None else 0.0),
-                           _int(lattice_range), _int(minimum_range), _p(ga), _p(gW))
+    fn = lib().ref_real_enc_bwd_magnitude if magnitude else lib().ref_real_enc_bwd
+    fn(_p(a_ik), _p(rpos_ij_e), _p(tvecs_n), _p(batch_i), _p(edge_ij_e), _p(e_start_i), _p(z_ek), _p(gz_ek),
+       _p(gv_ekd), _i64(N), _i64(H), _i64(E), _i64(K), _i64(D), _dbl(dist_max), _dbl(wscale), _p(W_k),
+       _i64(W_num), _p(rvlen_n), _dbl(cutoff_radius if cutoff_radius is not None else 0.0),
+       _int(lattice_range), _int(minimum_range), _p(ga), _p(gW))
     return ga, gW
 
 

@@ -159,16 +159,71 @@ void ref_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const float *tv
     free(sv);
 }
 
+/* First-order float32 conditioning of the Gaussian averages s[e,h,k] = sum_n p_n g_k(d_n):
+ *     cond[e,h,k] = sum_n p_n g_k(d_n) * ( 2 |b_k(d_n)| d_n / (sqrt2 ws mu0)  +  |a| d_n^2 )
+ * A relative rounding error u in a computed distance moves g_k by g_k 2|b| d/(sqrt2 ws mu0) u
+ * (b = Gaussian argument), and one in a d^2 moves the weight p_n by p_n |a| d^2 u: u * cond
+ * is the error any float32 evaluation of s carries, whatever its order of operations.  Used by
+ * the tests as the element-wise tolerance of narrow Gaussians far from their centre; not a
+ * restatement of reference code. */
+void ref_real_enc_fwd_cond(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                           const i64 *batch_i, const i64 *edge_ij_e, i64 N, i64 H, i64 E,
+                           i64 K, double dist_max, double wscale, const float *rvlen_n,
+                           double cutoff_radius, int lattice_range, int minimum_range, float *cond_ehk)
+{
+    static const float zero3[3] = {0, 0, 0};
+    (void)N;
+    double *sv = (double *)malloc(sizeof(double) * (size_t)(K > 0 ? K : 1));
+    const double inv_ws_sqrt2 = 1.0 / (wscale * sqrt(2.0));
+    const double mu0 = K > 0 ? dist_max / (double)K : 1.0;
+    for (i64 e = 0; e < E; e++) {
+        const i64 i = edge_ij_e[e];
+        const i64 n = batch_i[i];
+        const float *r = rpos_ij_e + e * 3;
+        const float *t = tvecs_n + n * 9;
+        const float *rvl = rvlen_n ? rvlen_n + n * 3 : zero3;
+        for (i64 h = 0; h < H; h++) {
+            const float a = a_ik[i * H + h];
+            int R[3];
+            range_rule(a, rvl, rvlen_n ? cutoff_radius : 0.0, lattice_range, minimum_range, R);
+            float d2min = 1e10f;
+            for (int n1 = -R[0]; n1 <= R[0]; n1++)
+                for (int n2 = -R[1]; n2 <= R[1]; n2++)
+                    for (int n3 = -R[2]; n3 <= R[2]; n3++) {
+                        float d2 = dist2_f(r, t, (float)n1, (float)n2, (float)n3);
+                        if (d2 < d2min) d2min = d2;
+                    }
+            double sum = 0;
+            for (i64 k = 0; k < K; k++) sv[k] = 0;
+            for (int n1 = -R[0]; n1 <= R[0]; n1++)
+                for (int n2 = -R[1]; n2 <= R[1]; n2++)
+                    for (int n3 = -R[2]; n3 <= R[2]; n3++) {
+                        float d2 = dist2_f(r, t, (float)n1, (float)n2, (float)n3);
+                        double w = exp((double)a * ((double)d2 - (double)d2min));
+                        sum += w;
+                        double d = sqrt((double)d2);
+                        for (i64 k = 0; k < K; k++) {
+                            double b = -d / mu0 * inv_ws_sqrt2 + inv_ws_sqrt2 * (double)(k + 1);
+                            sv[k] += exp(-b * b) * w *
+                                     (2.0 * fabs(b) * d / mu0 * inv_ws_sqrt2 + fabs((double)a) * (double)d2);
+                        }
+                    }
+            for (i64 k = 0; k < K; k++) cond_ehk[(e * H + h) * K + k] = (float)(sv[k] / sum);
+        }
+    }
+    free(sv);
+}
+
 /* Gradient wrt a_ik (N,H) and, when W_k != NULL, wrt W (W_num,H,D,K), already
  * reduced to W's own shape.  gv_ekd is (E,H,K) without W and (E,H,D) with it;
  * gv_ekd may be NULL (treated as zero).  gW_k may be NULL. */
-void ref_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
-                      const i64 *batch_i, const i64 *edge_ij_e, const i64 *e_start_i,
-                      const float *z_ek, const float *gz_ek, const float *gv_ekd,
-                      i64 N, i64 H, i64 E, i64 K, i64 D, double dist_max, double wscale,
-                      const float *W_k, i64 W_num, const float *rvlen_n,
-                      double cutoff_radius, int lattice_range, int minimum_range,
-                      float *ga_ik, float *gW_k)
+static void real_enc_bwd_impl(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                              const i64 *batch_i, const i64 *edge_ij_e, const i64 *e_start_i,
+                              const float *z_ek, const float *gz_ek, const float *gv_ekd,
+                              i64 N, i64 H, i64 E, i64 K, i64 D, double dist_max, double wscale,
+                              const float *W_k, i64 W_num, const float *rvlen_n,
+                              double cutoff_radius, int lattice_range, int minimum_range,
+                              float *ga_ik, float *gW_k, int magnitude)
 {
     static const float zero3[3] = {0, 0, 0};
     (void)edge_ij_e;   /* rows are walked through e_start_i */
@@ -196,7 +251,7 @@ void ref_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tv
                 const float *r = rpos_ij_e + e * 3;
                 const i64 eh = e * H + h;
                 const double z = z_ek[eh];
-                const double gz = gz_ek ? gz_ek[eh] : 0.0;
+                const double gz = gz_ek ? (magnitude ? fabs((double)gz_ek[eh]) : gz_ek[eh]) : 0.0;
                 i64 w_ind = 0;
                 if (W_num == E) w_ind = e;
                 else if (W_num == N) w_ind = i;
@@ -204,11 +259,13 @@ void ref_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tv
                 for (i64 k = 0; k < K; k++) {
                     sv[k] = 0;
                     if (!gv_ekd) sgv[k] = 0;
-                    else if (!W) sgv[k] = gv_ekd[eh * K + k];
+                    else if (!W) sgv[k] = magnitude ? fabs((double)gv_ekd[eh * K + k]) : gv_ekd[eh * K + k];
                     else {
                         double acc = 0;
-                        for (i64 d = 0; d < D; d++)
-                            acc += (double)W[d * K + k] * (double)gv_ekd[eh * D + d];
+                        for (i64 d = 0; d < D; d++) {
+                            const double term = (double)W[d * K + k] * (double)gv_ekd[eh * D + d];
+                            acc += magnitude ? fabs(term) : term;
+                        }
                         sgv[k] = acc;
                     }
                 }
@@ -231,12 +288,14 @@ void ref_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tv
                                 pbg_avr += p * bg;
                             }
                         }
-                total += px_avr * gz + pxbg - px_avr * pbg_avr;
+                total += px_avr * gz + pxbg + (magnitude ? px_avr * pbg_avr : -px_avr * pbg_avr);
                 if (gWacc && gv_ekd) {
                     double *gW = gWacc + (w_ind * H + h) * D * K;
                     for (i64 d = 0; d < D; d++)
-                        for (i64 k = 0; k < K; k++)
-                            gW[d * K + k] += sv[k] * (double)gv_ekd[eh * D + d];
+                        for (i64 k = 0; k < K; k++) {
+                            const double g = gv_ekd[eh * D + d];
+                            gW[d * K + k] += sv[k] * (magnitude ? fabs(g) : g);
+                        }
                 }
             }
             ga_ik[i * H + h] = (float)total;
@@ -248,6 +307,36 @@ void ref_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tv
     }
     free(sgv);
     free(sv);
+}
+
+void ref_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                      const i64 *batch_i, const i64 *edge_ij_e, const i64 *e_start_i,
+                      const float *z_ek, const float *gz_ek, const float *gv_ekd,
+                      i64 N, i64 H, i64 E, i64 K, i64 D, double dist_max, double wscale,
+                      const float *W_k, i64 W_num, const float *rvlen_n,
+                      double cutoff_radius, int lattice_range, int minimum_range,
+                      float *ga_ik, float *gW_k)
+{
+    real_enc_bwd_impl(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd, N, H, E, K, D,
+                      dist_max, wscale, W_k, W_num, rvlen_n, cutoff_radius, lattice_range, minimum_range, ga_ik,
+                      gW_k, 0);
+}
+
+/* The same sums with every term replaced by its magnitude (|gz| PX + sum_n p_n (d_n^2 + PX)
+ * sum_k g_k |W^T| |gv| for ga, sum_e S |gv| for gW): what a float32 evaluation's rounding error
+ * is proportional to, used by the tests as the element-wise tolerance of these gradients.  Not a
+ * restatement of reference code. */
+void ref_real_enc_bwd_magnitude(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                                const i64 *batch_i, const i64 *edge_ij_e, const i64 *e_start_i,
+                                const float *z_ek, const float *gz_ek, const float *gv_ekd,
+                                i64 N, i64 H, i64 E, i64 K, i64 D, double dist_max, double wscale,
+                                const float *W_k, i64 W_num, const float *rvlen_n,
+                                double cutoff_radius, int lattice_range, int minimum_range,
+                                float *ga_ik, float *gW_k)
+{
+    real_enc_bwd_impl(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd, N, H, E, K, D,
+                      dist_max, wscale, W_k, W_num, rvlen_n, cutoff_radius, lattice_range, minimum_range, ga_ik,
+                      gW_k, 1);
 }
 
 /* que is already divided by sqrt(Dk).  aij_eh / bij_ehd may be NULL. */

@@ -25,3 +25,18 @@ def pytest_collection_modifyitems(config, items):
 @pytest.fixture(scope="session")
 def dev():
     return torch.device("cuda:0")
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """After a GPU session: the worst element-wise error per quantity, in units of its bound."""
+    from tests import helpers
+    if not helpers.elementwise_record:
+        return
+    import json
+    out = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, "elementwise_errors.json"), "w") as f:
+            json.dump({k: round(v, 4) for k, v in sorted(helpers.elementwise_record.items())}, f, indent=1)
+    except OSError:
+        pass

@@ -225,3 +225,53 @@ def test_reference_checkpoint_loading(tmp_path):
     assert all(torch.equal(v, other.state_dict()[k]) for k, v in plain.state_dict().items())
     with pytest.raises(KeyError):
         load_reference_checkpoint(Latticeformer(cfg), {"state_dict": {"x": torch.zeros(1)}})
+
+
+def test_dense_block_layout_check_on_the_host():
+    """The check that guards the pair kernels and the attention backward: only the exact dense
+    per-crystal block list of get_edge_index (with a sorted batch index) passes."""
+    from crystalformer_amd import ops
+    from oracle import torch_path as tp
+    sizes = [3, 1, 4]
+    batch = torch.repeat_interleave(torch.arange(3), torch.tensor(sizes))
+    edges = tp.get_edge_index(sizes)
+    assert ops.dense_block_layout(batch, edges).tolist() == sizes
+    assert ops.dense_block_layout(batch, edges[:, :-1].contiguous()) is None          # an edge missing
+    swapped = edges.clone()
+    swapped[:, [1, 2]] = swapped[:, [2, 1]]
+    assert ops.dense_block_layout(batch, swapped) is None                             # same set, other order
+    assert ops.dense_block_layout(batch, edges.flip(0)) is None                       # key-major instead of query-major
+    assert ops.dense_block_layout(batch.flip(0), edges) is None                       # unsorted batch index
+    wrong = edges.clone()
+    wrong[1, 0] = 5
+    assert ops.dense_block_layout(batch, wrong) is None                               # right count, wrong target
+    gap = batch.clone()
+    gap[batch == 2] = 4                                                               # crystal ids 0, 1, 4
+    assert ops.dense_block_layout(gap, edges).tolist() == [3, 1, 0, 0, 4]
+    empty = torch.zeros(0, dtype=torch.long)
+    assert ops.dense_block_layout(empty, torch.zeros(2, 0, dtype=torch.long)).numel() == 0
+    assert ops.dense_block_layout(batch, torch.zeros(3, 5, dtype=torch.long)) is None
+    # cached per tensor pair; the cached answer for a sparse list stays None
+    sparse = edges[:, ::2].contiguous()
+    assert ops.cached_dense_sizes(batch, sparse) is None and ops.cached_dense_sizes(batch, sparse) is None
+    assert ops.cached_dense_sizes(batch, edges).tolist() == sizes
+
+
+def test_graph_replay_refuses_other_crystal_sizes():
+    """Same atom and crystal counts, other sizes: the captured edges would be wrong."""
+    from types import SimpleNamespace
+    from crystalformer_amd.graphs import _same_layout
+    from crystalformer_amd.synthetic import CrystalBatch
+    mk = lambda sizes: CrystalBatch(torch.zeros(6, 98), torch.zeros(6, 3), torch.zeros(6, dtype=torch.long),
+                                    torch.zeros(2, 3, 3), torch.tensor(sizes))
+    owner = SimpleNamespace(static=mk([2, 4]), _sizes_host=[2, 4], _checked={})
+    _same_layout(owner, mk([2, 4]))
+    same = mk([2, 4])
+    _same_layout(owner, same)
+    _same_layout(owner, same)                          # remembered: no second read-back
+    assert len(owner._checked) == 2
+    with pytest.raises(ValueError, match="sizes differ"):
+        _same_layout(owner, mk([3, 3]))
+    with pytest.raises(ValueError, match="layout differs"):
+        _same_layout(owner, CrystalBatch(torch.zeros(5, 98), torch.zeros(5, 3), torch.zeros(5, dtype=torch.long),
+                                         torch.zeros(2, 3, 3), torch.tensor([2, 3])))

@@ -16,7 +16,7 @@ from crystalformer_amd.synthetic import CONFIGS, make_config_batch
 from oracle import kernel_semantics as ks
 from oracle import torch_model as om
 from oracle import torch_path as tp
-from tests.helpers import Problem, assert_close, rel_err, to_dev
+from tests.helpers import Problem, assert_close, atol_rows, rel_err, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -198,6 +198,98 @@ def test_full_model_forward_against_oracle(dev, name):
     for li in range(cfg.num_layers):
         assert_close(outs[li], cap[f"layer{li}.out"], f"layer {li}")
     assert_close(y, y_ref, "model output")
+
+
+# Configurations whose dense CPU evaluation takes minutes are compared with the oracle's stored
+# results (tests/golden/make_oracle_fixtures.py); the fixture is refused when the inputs or the
+# initial parameters it was computed from differ from the ones rebuilt here.
+def oracle_fixture(tag, batch, model):
+    from make_oracle_fixtures import digest
+    fx = torch.load(os.path.join(GOLD, f"oracle_{tag}.pt"), weights_only=True)
+    assert fx["digest"] == digest(batch, {k: v.cpu() for k, v in model.state_dict().items()}), \
+        f"oracle_{tag}.pt was written for other inputs: re-run tests/golden/make_oracle_fixtures.py"
+    return fx
+
+
+def check_forward_against_fixture(dev, name, batch, tag):
+    cfg, model = build_model(name, adaptive_cutoff_sigma=0.0)
+    fx = oracle_fixture(tag, batch, model)
+    model.to(dev).eval()
+    outs, alphas = {}, {}
+    for li, layer in enumerate(model.encoder.layers):
+        layer.register_forward_hook(lambda m, i, o, li=li: outs.__setitem__(li, o))
+    with torch.no_grad():
+        y = model(batch.to(dev))
+    sel = fx["atoms"]
+    for li in range(cfg.num_layers):
+        ref = fx[f"layer{li}.out"]
+        assert_close(outs[li].cpu()[sel], ref, f"layer {li} out", atol=atol_rows(ref))
+    assert_close(y, fx["y"], "model output")
+    return cfg, model, y
+
+
+def test_seven_block_forward_at_256_crystals(dev):
+    """Config 3: 7 blocks with scale_real 1.4 / 1.4 / 2.0 / 2.0 / 3.0 / 3.0 / 3.0, 256 crystals of
+    1..96 atoms (N = 4762, E = 221,920), fixed cube, whole forward on the HIP path against the
+    CPU oracle: every block's output on every 37th atom and the model output of all crystals."""
+    b = make_config_batch("cfg3_7block_b256")
+    cfg, _, _ = check_forward_against_fixture(dev, "cfg3_7block_b256", b, "cfg3_forward")
+    assert cfg.num_layers == 7 and list(cfg.scale_real) == [1.4, 1.4, 2.0, 2.0, 3.0, 3.0, 3.0]
+
+
+def test_four_block_forward_on_large_cells(dev):
+    """Config 5 at model level: the 4-block default model (scale_real 3.0) on the two smallest of
+    the 200..444-atom elongated cells against the CPU oracle (chunked over edges)."""
+    from make_oracle_fixtures import cfg5_subset
+    b = cfg5_subset(make_config_batch("cfg5_stress_b16"))
+    assert int(b.sizes.min()) >= 200
+    check_forward_against_fixture(dev, "cfg5_stress_b16", b, "cfg5_subset_forward")
+
+
+def test_training_step_at_128_crystals(dev):
+    """Config 4: one training-mode forward + the reference's step loss + backward at 128 crystals
+    (models/regression.py:117-121) on the HIP path (periodic-encoding and attention backward
+    kernels at N = 1774, E = 56,440) against autograd through the CPU oracle in float64: loss,
+    outputs, the stored batch statistics and every parameter gradient, plain and through the
+    fused training step.  Parameters are the seeded initialisation with the first feed-forward
+    biases moved by a few 1e-5 so that no ReLU argument of this batch lies within 2e-6 of zero
+    (stored with the fixture): at a kink the mask, and with it one atom's share of a weight
+    gradient's row, is decided by rounding, and float32 and float64 then differ by 1e-2 there."""
+    from crystalformer_amd.training import FusedAdamW, fused_training_step
+    b = make_config_batch("cfg4_train_b128")
+    cfg, model = build_model("cfg4_train_b128", adaptive_cutoff_sigma=0.0)
+    fx = oracle_fixture("cfg4_train_step", b, model)
+    import copy
+    model.load_state_dict(fx["adjusted"], strict=False)
+    model.to(dev).train()
+    twin = copy.deepcopy(model)
+    bd = b.to(dev)
+    y = model(bd)
+    loss = tp.l1_training_loss(y, bd.y.reshape(-1, 1))
+    loss.backward()
+    assert_close(y, fx["y"], "y")
+    assert abs(float(loss.detach()) - float(fx["loss"])) <= 1e-5 * abs(float(fx["loss"]))
+    scales = torch.stack([l.self_attn.gauss_scale.detach() for l in model.encoder.layers])
+    assert_close(scales, fx["gauss_scale_after"], "gauss_scale")
+    params = dict(model.named_parameters())
+    assert set(fx["grads"]) == {k for k, p in params.items() if p.requires_grad}
+    worst = {}
+    for k, g in fx["grads"].items():
+        worst[k] = rel_err(params[k].grad, g)
+        # element-wise against the scale of the entry's own row (one output unit's sum over all
+        # atoms or edges); the sum of the magnitudes of its terms is not at hand at model level
+        # (a bias vector is one row: the key bias' gradient, for one, is zero but for rounding)
+        rows = g.reshape(1, -1) if g.dim() == 1 else g.reshape(g.shape[0], -1)
+        assert_close(params[k].grad, g, f"grad {k}", atol=atol_rows(rows).reshape(
+            (rows.shape[0],) + (1,) * (g.dim() - 1)))
+    # the same gradients out of the fused step (row-block linear Functions, deferred weight
+    # gradients, loss kernel), read before its optimiser update overwrites nothing of them
+    opt = FusedAdamW(twin, lr=0.0)
+    fused_training_step(twin, bd, opt)
+    for k, p in twin.named_parameters():
+        if k in fx["grads"]:
+            assert_close(p.grad, fx["grads"][k], f"fused grad {k}")
+    print("worst gradient error:", max(worst.items(), key=lambda kv: kv[1]))
 
 
 def test_full_size_properties_and_sampled_edges(dev):
