@@ -18,6 +18,8 @@
 // All exponentials go through v_exp_f32 with log2(e) folded into the operands.
 #include "cf_common.h"
 
+#include <mutex>
+
 namespace {
 
 using namespace cf;
@@ -983,6 +985,66 @@ extern "C" int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const 
         }
     }
     return CF_OK;
+}
+
+// ---- backward without a caller-provided workspace ----------------------------------
+// Scratch of cf_real_enc_bwd (per-edge ga, per-work-group gW blocks, or the per-edge kernels'
+// Gaussian averages) in a fixed array that every GPU running this library holds until the
+// process ends.  The array's name is a host-side stand-in for the symbol: the device address
+// is looked up once per device, with that device current, and only that address is ever
+// handed to a kernel.
+#define CF_STATIC_SCRATCH_BYTES (32ll << 20)
+static __device__ __align__(256) unsigned char scratch[CF_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[MAX_DEVICES] = {};
+
+int static_scratch(void **out)
+{
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return cf::hip_failed(err, "cf_real_enc_bwd_static: hipGetDevice");
+    CF_REQUIRE(dev >= 0 && dev < MAX_DEVICES, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_bwd_static: device %d outside 0..%d", dev, MAX_DEVICES - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return cf::hip_failed(err, "cf_real_enc_bwd_static: hipGetSymbolAddress");
+        CF_REQUIRE(ptr != nullptr, CF_ERR_HIP, "cf_real_enc_bwd_static: no device address for the scratch array");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return CF_OK;
+}
+}  // namespace
+
+extern "C" int64_t cf_static_scratch_bytes(void) { return CF_STATIC_SCRATCH_BYTES; }
+
+extern "C" int cf_real_enc_bwd_static(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                                      const int64_t *batch_i, const int64_t *edge_ij_e,
+                                      const int64_t *e_start_i, const float *z_ek, const float *gz_ek,
+                                      const float *gv_ekd, int64_t N, int64_t H, int64_t E, int64_t B, int64_t K,
+                                      int64_t D, double dist_max, double wscale, const float *W_k, int64_t W_num,
+                                      const float *rvlen_n, double cutoff_radius, int lattice_range,
+                                      int minimum_range, const int64_t *pairs_u, int64_t U, float *ga_ik,
+                                      float *gW_k, void *stream)
+{
+    CF_REQUIRE(N >= 0 && H >= 1 && E >= 0 && K >= 0 && D >= 0 && W_num >= 0, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_bwd_static: negative size");
+    const bool want_gW = gW_k != nullptr && W_k != nullptr && K > 0 && gv_ekd != nullptr;
+    const int64_t need = cf_real_enc_bwd_workspace(N, H, E, K, D, W_num, want_gW);
+    CF_REQUIRE(need <= CF_STATIC_SCRATCH_BYTES, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_bwd_static: these sizes need %lld bytes of scratch, the built-in buffer holds %lld; "
+               "use cf_real_enc_bwd with a workspace", (long long)need, (long long)CF_STATIC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    int rc = static_scratch(&ws);
+    if (rc) return rc;
+    return cf_real_enc_bwd(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd, N, H, E,
+                           B, K, D, dist_max, wscale, W_k, W_num, rvlen_n, cutoff_radius, lattice_range,
+                           minimum_range, pairs_u, U, ws, CF_STATIC_SCRATCH_BYTES, ga_ik, gW_k, stream);
 }
 
 extern "C" int cf_translation_ranges(const float *a_ik, const float *rvlen_n, const int64_t *batch_i,

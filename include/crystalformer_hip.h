@@ -138,6 +138,32 @@ int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tvec
                     float *ga_ik, float *gW_k, void *stream);
 
 /*
+ * cf_real_enc_bwd without a workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference, whose wrappers allocate their scratch with
+ * torch.empty on every call (models/cuda_funcs/real_space_enc_proj.py:137-151).
+ *
+ * Same arguments, kernels and results as cf_real_enc_bwd; the scratch lives in a fixed
+ * array of cf_static_scratch_bytes() = 32 MiB inside the library's device code, which every
+ * GPU the library runs on holds until the process ends.  Sizes for which
+ * cf_real_enc_bwd_workspace() exceeds that are rejected with CF_ERR_INVALID_ARGUMENT (the
+ * benchmark's training batch of 128 crystals needs 18.6 MB, 256 crystals of up to 96 atoms
+ * 24 MB).  Calls nothing that allocates or frees.  All calls on one GPU share the one array:
+ * calls that overlap in time on the same GPU (different streams or threads) race and give
+ * wrong gradients; calls on one stream are ordered and safe.
+ */
+int64_t cf_static_scratch_bytes(void);
+int cf_real_enc_bwd_static(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                           const int64_t *batch_i, const int64_t *edge_ij_e,
+                           const int64_t *e_start_i, const float *z_ek, const float *gz_ek,
+                           const float *gv_ekd, int64_t N, int64_t H, int64_t E, int64_t B,
+                           int64_t K, int64_t D, double dist_max, double wscale,
+                           const float *W_k, int64_t W_num, const float *rvlen_n,
+                           double cutoff_radius, int lattice_range, int minimum_range,
+                           const int64_t *pairs_u, int64_t U,
+                           float *ga_ik, float *gW_k, void *stream);
+
+/*
  * Per (atom, head) translation half-widths the encoding kernels use,
  * R_out (N,H,3) int32.  Exposes the rule of models/kernels/real_enc_fwd.cu:58-85
  * for bit-exact checks and work counting.
