@@ -32,15 +32,17 @@ PEAK_FP32_TFLOPS = 157.3          # fp32 on the matrix cores (and packed vector 
 PEAK_FP32_VALU_TFLOPS = 78.6      # one fp32 FMA per lane and cycle: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz x 2
 PEAK_HBM_GBS = 8000.0
 PROFILE_FILE = os.path.join(ROOT, "profiles", "traffic.json")
-KERNEL_SOURCES = ("real_enc_mfma.hip", "real_enc_mfma_bwd.hip", "real_enc_pair.h", "cf_common.h")
+KERNEL_SOURCES = {"fwd": ("real_enc_mfma.hip", "real_enc_pair.h", "cf_common.h"),
+                  "bwd": ("real_enc_mfma_bwd.hip", "real_enc_pair.h", "cf_common.h")}
 
 
-def kernel_fingerprint() -> str:
-    """SHA-256 (first 16 hex digits) of the sources of the periodic-encoding pair kernels: stored
-    beside hardware counters when they are taken, compared when they are used."""
+def kernel_fingerprint(direction: str) -> str:
+    """SHA-256 (first 16 hex digits) of the sources of the periodic-encoding pair kernel of one
+    direction ("fwd" / "bwd"): stored beside hardware counters when they are taken, compared
+    when they are used."""
     import hashlib
     h = hashlib.sha256()
-    for name in KERNEL_SOURCES:
+    for name in KERNEL_SOURCES[direction]:
         with open(os.path.join(ROOT, "crystalformer_amd", "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]
@@ -64,10 +66,11 @@ def stored_counters(key: str, required: bool):
                              f"or pass --no-counters to report the roofline without executed work")
         return None
     entry = dict(entry)
-    entry["current"] = entry.get("kernel_sha16") == kernel_fingerprint()
+    now = kernel_fingerprint(key.rsplit(":", 1)[1])
+    entry["current"] = entry.get("kernel_sha16") == now
     if not entry["current"]:
         print(f"bench.py: WARNING: counters for '{key}' were taken with other kernel sources "
-              f"({entry.get('kernel_sha16')} at {entry.get('commit')}, now {kernel_fingerprint()}); "
+              f"({entry.get('kernel_sha16')} at {entry.get('commit')}, now {now}); "
               f"the executed-work figures in the line are stale", file=sys.stderr)
     return entry
 
@@ -163,7 +166,7 @@ def ingest_counters(directory: str, key: str, kernel: str) -> int:
     if "fetch_bytes" in entry and "write_bytes" in entry:
         entry["hbm_bytes"] = entry["fetch_bytes"] + entry["write_bytes"]
     entry.update({"kernel": kernel, "dispatches_averaged": len(next(iter(agg["kernel"].values()))),
-                  "cus": 256, "clock_ghz": 2.4, "kernel_sha16": kernel_fingerprint(),
+                  "cus": 256, "clock_ghz": 2.4, "kernel_sha16": kernel_fingerprint(key.rsplit(":", 1)[1]),
                   "date": datetime.date.today().isoformat()})
     try:
         entry["commit"] = subprocess.check_output(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"],
@@ -381,6 +384,8 @@ def main() -> int:
     ap.add_argument("--launch-share", type=float, default=0.75,
                     help="with several steps in flight: share of the GPU one periodic-encoding launch "
                          "occupies (384 of its 512 work-groups by default)")
+    ap.add_argument("--two-launch-blocks", action="store_true",
+                    help="blocks without value bins: run bias and attention as two operators instead of one launch")
     ap.add_argument("--no-fresh", action="store_true", help="skip the fresh-batch (layout rebuilt every step) figure")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--train", action="store_true",
@@ -419,6 +424,9 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     lib.load()
+    if args.two_launch_blocks:
+        from crystalformer_amd import hip_funcs
+        hip_funcs.KernelManager.FUSE_ENCODING_ATTENTION = False
     dev = torch.device("cuda:0")
     if args.train and args.config == "cfg2_default_b128":
         args.config = "cfg4_train_b128"

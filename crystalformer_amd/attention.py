@@ -296,11 +296,19 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                 adaptive = (rvlen, cutoff)
             if proj is not None and not P.value_pe_headed:
                 proj = proj.expand(proj.shape[0], H, proj.shape[2], proj.shape[3])
-            enc = RealPeriodicEncodingWithProjFuncCUDA if P.use_low_memory else RealPeriodicEncodingFuncCUDA
-            out = hip_funcs.call(enc, a, points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real, dist_max,
-                                 P.value_pe_width_scale, proj, *adaptive)
-            bias = out[0]
-            values = out[1] if len(out) >= 2 else None
+            attn = None
+            if (P.value_pe_dist_real <= 0 and qs is not None and not need_weights and P.norm_func_mode == 0
+                    and config.REPRODUCIBLITY_STATE >= 2 and batch_q is batch_kv and not torch.is_grad_enabled()):
+                # no value bins and nobody asks for the bias: lattice sums and attention in one launch
+                attn = hip_funcs.fused_encoding_attention(a, points, tvecs, batch_q, edges, qs, k, v, *adaptive)
+            if attn is None:
+                enc = RealPeriodicEncodingWithProjFuncCUDA if P.use_low_memory else RealPeriodicEncodingFuncCUDA
+                out = hip_funcs.call(enc, a, points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real,
+                                     dist_max, P.value_pe_width_scale, proj, *adaptive)
+                bias = out[0]
+                values = out[1] if len(out) >= 2 else None
+            else:
+                return self._project_output(attn, n, vd, fused_linear, fused_train, residual, need_weights, None)
 
         if P.norm_func_mode != 0:
             raise NotImplementedError("norm_func_mode != 0 is not served by the HIP path")
@@ -308,10 +316,21 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             raise NotImplementedError("attention dropout is not served by the HIP path")
         if qs is None:
             qs = q / math.sqrt(q.shape[-1])
-        if config.REPRODUCIBLITY_STATE >= 2 and batch_q is batch_kv:
+        weights = None
+        if need_weights:
+            # softmax weights averaged over the heads, (E,), as the reference's loop path returns them
+            # (models/indexed_lattice_multi_head_attention_cuda.py:782-786)
+            attn, prob = hip_funcs.call(hip_funcs.FusedDotProductAttentionWithWeights, qs, k, v, bias, values,
+                                        batch_q, edges)
+            weights = prob.mean(dim=1)
+        elif config.REPRODUCIBLITY_STATE >= 2 and batch_q is batch_kv:
             attn = hip_funcs.call(FusedDotProductAttentionCUDA, qs, k, v, bias, values, batch_q, edges)
         else:
             attn = loop_attention(qs, k, v, batch_q, edges, bias, values)
+        return self._project_output(attn, n, vd, fused_linear, fused_train, residual, need_weights,
+                                    weights if need_weights else values)
+
+    def _project_output(self, attn, n, vd, fused_linear, fused_train, residual, need_weights, values):
         attn = attn.contiguous().view(n, vd)
         if fused_linear:
             attn, = ops.linear_rows(attn, (self.out_proj.weight,), self.out_proj.bias, residual=residual)
@@ -322,8 +341,6 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             attn = linear_hip(attn, self.out_proj.weight, self.out_proj.bias)
             if residual is not None:
                 attn = residual + attn
-        if need_weights:
-            raise NotImplementedError("need_weights=True: attention weights are not returned by the fused path")
         return attn, values
 
 

@@ -210,6 +210,171 @@ __global__ __launch_bounds__(256) void real_enc_fwd_bias_kernel(EncArgs p)
 }
 
 // ---------------------------------------------------------------------------
+// forward, K == 0, fused with the attention that consumes the bias: one work-group per query
+// atom.  Phase 1 (a wavefront per edge of the row, lane = translation) forms the lattice-sum
+// bias z of the row exactly as the kernel above does and leaves it in LDS; phase 2 adds the
+// scaled dot products q_i . k_j (thread = (key, head)); phase 3 is the softmax over the row's
+// keys (a wavefront per head); phase 4 aggregates the values (thread = (head, component)).
+// Neither z nor the probabilities ever reach HBM.  The unordered-pair trick of the matrix-core
+// kernel buys nothing here: without Gaussian bins the exponentials are per (edge, head) anyway
+// and only the distance of a translation would be shared.
+// LDS: logits / probabilities [row length][H], key atoms [row length].
+// ---------------------------------------------------------------------------
+struct RowArgs {
+    const float *que, *key, *val;
+    float *out;
+    int Dk, Dv;
+    int max_row;
+};
+
+template <int H>
+__global__ __launch_bounds__(1024) void enc_dpa_row_kernel(EncArgs p, RowArgs r)
+{
+    extern __shared__ float lds[];
+    float *zl = lds;                                            // [row][H]
+    int *jl = reinterpret_cast<int *>(lds + (size_t)r.max_row * H);   // [row]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wpb = blockDim.x >> 6;
+    const int64_t i = blockIdx.x;
+    const int64_t e0 = p.e_start[i];
+    const int n = (int)(p.e_start[i + 1] - e0);
+    const int Dk = r.Dk, Dv = r.Dv;
+    if (n == 0) {                                               // an atom without edges: zero row
+        for (int x = threadIdx.x; x < H * Dv; x += blockDim.x) r.out[i * H * Dv + x] = 0.f;
+        return;
+    }
+    // ---- phase 1: lattice sums of the row
+    {
+        const int64_t nb = p.batch[i];
+        float a[H];
+#pragma unroll
+        for (int h = 0; h < H; h++) a[h] = p.a_ik[i * H + h];
+        float rvl[3] = {0.f, 0.f, 0.f};
+        if (p.rvlen) {
+            rvl[0] = p.rvlen[nb * 3 + 0];
+            rvl[1] = p.rvlen[nb * 3 + 1];
+            rvl[2] = p.rvlen[nb * 3 + 2];
+        }
+        Box<H> box;
+        make_box(box, a, p.cutoff, rvl, p.lattice_range, p.min_range);
+        // The box belongs to the row's atom: boxes of up to 128 translations (the default cube has
+        // 125) are decoded once, two translations per lane, with the heads whose own box holds
+        // them as a bit set; every edge of the row then costs two distance evaluations per lane.
+        const bool small = box.T <= 2 * WAVE;
+        float nf[2][3] = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
+        int hbits[2] = {0, 0};
+        if (small) {
+#pragma unroll
+            for (int ch = 0; ch < 2; ch++) {
+                const int idx = ch * WAVE + lane;
+                if (idx < box.T) {
+                    int n1, n2, n3;
+                    decode(box, idx, n1, n2, n3);
+                    nf[ch][0] = (float)n1;
+                    nf[ch][1] = (float)n2;
+                    nf[ch][2] = (float)n3;
+#pragma unroll
+                    for (int h = 0; h < H; h++)
+                        if (box.uniform || inside(box, h, n1, n2, n3)) hbits[ch] |= 1 << h;
+                }
+            }
+        }
+        for (int jj = wave; jj < n; jj += wpb) {
+            const int64_t e = e0 + jj;
+            Cell c;
+            load_cell(c, p, e, nb);
+            float d2min[H];
+            float sum[H];
+#pragma unroll
+            for (int h = 0; h < H; h++) sum[h] = 0.f;
+            if (small) {
+                float d2[2];
+#pragma unroll
+                for (int ch = 0; ch < 2; ch++) d2[ch] = dist2(c, nf[ch][0], nf[ch][1], nf[ch][2]);
+                if (box.uniform) {
+                    const float m = wave_min(fminf(hbits[0] ? d2[0] : 1e10f, hbits[1] ? d2[1] : 1e10f));
+#pragma unroll
+                    for (int h = 0; h < H; h++) d2min[h] = m;
+                } else {
+#pragma unroll
+                    for (int h = 0; h < H; h++)
+                        d2min[h] = wave_min(fminf((hbits[0] >> h) & 1 ? d2[0] : 1e10f,
+                                                  (hbits[1] >> h) & 1 ? d2[1] : 1e10f));
+                }
+#pragma unroll
+                for (int ch = 0; ch < 2; ch++)
+#pragma unroll
+                    for (int h = 0; h < H; h++) {
+                        const float w = exp2_hw(a[h] * LOG2E * (d2[ch] - d2min[h]));
+                        sum[h] += ((hbits[ch] >> h) & 1) ? w : 0.f;
+                    }
+            } else {
+                box_minimum(box, c, lane, d2min);
+                for (int c0 = 0; c0 < box.T; c0 += WAVE) {
+                    int idx = c0 + lane;
+                    if (idx < box.T) {
+                        int n1, n2, n3;
+                        decode(box, idx, n1, n2, n3);
+                        float d2 = dist2(c, (float)n1, (float)n2, (float)n3);
+#pragma unroll
+                        for (int h = 0; h < H; h++) {
+                            float w = exp2_hw(a[h] * LOG2E * (d2 - d2min[h]));
+                            if (!box.uniform && !inside(box, h, n1, n2, n3)) w = 0.f;
+                            sum[h] += w;
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < H; h++) {
+                float s = wave_sum(sum[h]);
+                if (lane == h) zl[jj * H + h] = log2_hw(s) * LN2 + d2min[h] * a[h];
+            }
+            if (lane == 0) jl[jj] = (int)p.edges[p.E + e];
+        }
+    }
+    __syncthreads();
+    // ---- phase 2: logits q_i . k_j + z (the query comes pre-divided by sqrt(Dk))
+    for (int x = threadIdx.x; x < n * H; x += blockDim.x) {
+        const int jj = x / H, h = x - jj * H;
+        const float *qp = r.que + (i * H + h) * Dk;
+        const float *kp = r.key + ((int64_t)jl[jj] * H + h) * Dk;
+        float s = 0.f;
+        for (int d = 0; d < Dk; d++) s = fmaf(qp[d], kp[d], s);
+        zl[x] += s;
+    }
+    __syncthreads();
+    // ---- phase 3: softmax over the keys of the row, a wavefront per head
+    for (int h = wave; h < H; h += wpb) {
+        float m = -3.0e38f;
+        for (int jj = lane; jj < n; jj += WAVE) m = fmaxf(m, zl[jj * H + h]);
+        m = wave_max(m);
+        float sum = 0.f;
+        for (int jj = lane; jj < n; jj += WAVE) {
+            const float w = exp2_hw((zl[jj * H + h] - m) * LOG2E);
+            zl[jj * H + h] = w;
+            sum += w;
+        }
+        const float inv = 1.0f / wave_sum(sum);
+        for (int jj = lane; jj < n; jj += WAVE) zl[jj * H + h] *= inv;
+    }
+    __syncthreads();
+    // ---- phase 4: out[i,h,:] = sum_j p_ij v_j
+    for (int x = threadIdx.x; x < H * Dv; x += blockDim.x) {
+        const int h = x / Dv;
+        float acc0 = 0.f, acc1 = 0.f;
+        int jj = 0;
+        for (; jj + 1 < n; jj += 2) {
+            acc0 = fmaf(zl[jj * H + h], r.val[(int64_t)jl[jj] * H * Dv + x], acc0);
+            acc1 = fmaf(zl[(jj + 1) * H + h], r.val[(int64_t)jl[jj + 1] * H * Dv + x], acc1);
+        }
+        if (jj < n) acc0 = fmaf(zl[jj * H + h], r.val[(int64_t)jl[jj] * H * Dv + x], acc0);
+        r.out[i * H * Dv + x] = acc0 + acc1;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // forward, K > 0.  NB = bins per lane (K <= 64*NB).
 // LDS: [W: H*D*KP floats if PROJ && W_num==1][per wave: H*KP floats]
 // ---------------------------------------------------------------------------
@@ -1045,6 +1210,45 @@ extern "C" int cf_real_enc_bwd_static(const float *a_ik, const float *rpos_ij_e,
     return cf_real_enc_bwd(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd, N, H, E,
                            B, K, D, dist_max, wscale, W_k, W_num, rvlen_n, cutoff_radius, lattice_range,
                            minimum_range, pairs_u, U, ws, CF_STATIC_SCRATCH_BYTES, ga_ik, gW_k, stream);
+}
+
+namespace {
+template <int H>
+int launch_enc_dpa_rows(const EncArgs &p, const RowArgs &r, int64_t N, hipStream_t st)
+{
+    const size_t lds = sizeof(float) * (size_t)r.max_row * (H + 1);
+    // a wavefront per edge of the longest row, 4 to 16 of them
+    const int waves = r.max_row <= 4 ? 4 : r.max_row <= 8 ? 8 : 16;
+    enc_dpa_row_kernel<H><<<(int)N, waves * WAVE, lds, st>>>(p, r);
+    return CF_OK;
+}
+}  // namespace
+
+extern "C" int cf_fused_enc_dpa_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                                    const int64_t *batch_i, const int64_t *edge_ij_e, const int64_t *e_start_i,
+                                    const float *que, const float *key, const float *val, int64_t N, int64_t H,
+                                    int64_t E, int64_t B, int64_t Dk, int64_t Dv, const float *rvlen_n,
+                                    double cutoff_radius, int lattice_range, int minimum_range, int64_t max_row,
+                                    float *out, void *stream)
+{
+    EncArgs p;
+    int rc = fill_args(p, "cf_fused_enc_dpa_fwd", a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, N, H, E, B, 0, 0,
+                       1.0, 1.0, nullptr, 0, rvlen_n, cutoff_radius, lattice_range, minimum_range);
+    if (rc) return rc;
+    CF_REQUIRE(Dk >= 1 && Dv >= 1 && Dk <= 256 && Dv <= 256, CF_ERR_INVALID_ARGUMENT,
+               "cf_fused_enc_dpa_fwd: head widths %lld / %lld outside 1..256", (long long)Dk, (long long)Dv);
+    CF_REQUIRE(N < (1ll << 31), CF_ERR_UNSUPPORTED, "cf_fused_enc_dpa_fwd: more than 2^31 atoms");
+    if (N == 0) return CF_OK;
+    CF_REQUIRE(que && key && val && out && e_start_i, CF_ERR_INVALID_ARGUMENT, "cf_fused_enc_dpa_fwd: null pointer");
+    CF_REQUIRE(max_row >= 0 && max_row * (H + 1) * 4 <= 64 * 1024, CF_ERR_UNSUPPORTED,
+               "cf_fused_enc_dpa_fwd: rows of up to %lld edges; this kernel keeps a row's %lld logits in 64 KB of "
+               "LDS (use cf_real_enc_fwd + cf_fused_dpa_fwd)", (long long)max_row, (long long)(max_row * H));
+    p.e_start = e_start_i;
+    RowArgs r{que, key, val, out, (int)Dk, (int)Dv, (int)(max_row < 1 ? 1 : max_row)};
+    rc = CF_DISPATCH_H(H, launch_enc_dpa_rows, p, r, N, (hipStream_t)stream);
+    if (rc) return rc;
+    CF_CHECK_LAUNCH("cf_fused_enc_dpa_fwd");
+    return CF_OK;
 }
 
 extern "C" int cf_translation_ranges(const float *a_ik, const float *rvlen_n, const int64_t *batch_i,

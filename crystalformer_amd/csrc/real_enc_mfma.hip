@@ -121,9 +121,12 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
     }
     // Fixed cube: the translation a lane evaluates in chunk ch is the same in every round; the
     // first two chunks (128 translations, the default cube has 125) are decoded once.
+    // The adaptive rule yields that very cube for every unit whose 16 columns all stay at the
+    // floor of lattice_range (most units when the floor is on and the Gaussians are narrow), so
+    // the adaptive kernel keeps the decoded cube as well and takes the cube's shortcuts for them.
     constexpr int NPRE = 2;
-    float npre[UNIFORM ? NPRE : 1][3];
-    if (UNIFORM) {
+    float npre[NPRE][3];
+    {
         BoxDims b0;
         b0.U1 = b0.U2 = b0.U3 = p.lattice_range;
         b0.S3 = b0.S2 = 2 * p.lattice_range + 1;
@@ -214,9 +217,16 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         bx.inv_plane = __builtin_amdgcn_rcpf((float)bx.plane);
         bx.inv_S3 = __builtin_amdgcn_rcpf((float)bx.S3);
         const int T = bx.T;
+        // all active columns of this unit have the box [-lattice_range, lattice_range]^3 (wave-uniform)
+        bool cube = UNIFORM;
+        if (!UNIFORM) {
+            const int lr = p.lattice_range;
+            const bool other = col_on && (R1 != lr || R2 != lr || R3 != lr);
+            cube = bx.U1 == lr && bx.U2 == lr && bx.U3 == lr && NPRE * WAVE >= T && __ballot(other) == 0ull;
+        }
 
         ColumnBoxes cbox{0, 0, 0};
-        if (!UNIFORM) cbox = column_boxes(R1, R2, R3, bx, lane);
+        if (!UNIFORM && !cube) cbox = column_boxes(R1, R2, R3, bx, lane);
         // geometry of one translation: d^2 and the in-box bits of the 16 columns
         auto geometry = [&](int idx, bool valid, float &d2, int &colbits) {
             int n1, n2, n3;
@@ -252,9 +262,9 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 d2c[ch] = 0.f;
                 if (ch < nchunk) {
                     int cb;
-                    if (UNIFORM && ch < NPRE) {
-                        d2c[ch] = dist2(cell, npre[UNIFORM ? ch : 0][0], npre[UNIFORM ? ch : 0][1],
-                                        npre[UNIFORM ? ch : 0][2]);
+                    if (cube && ch < NPRE) {
+                        d2c[ch] = dist2(cell, npre[ch < NPRE ? ch : 0][0], npre[ch < NPRE ? ch : 0][1],
+                                        npre[ch < NPRE ? ch : 0][2]);
                         cb = ch * WAVE + lane < T ? 0xFFFF : 0;
                     } else {
                         geometry(ch * WAVE + lane, ch * WAVE + lane < T, d2c[ch], cb);
@@ -275,7 +285,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         // nearest image lies inside the column's box (nearly always); otherwise a pass that
         // tracks the 16 columns separately.
         float d2min = wave_min(best);
-        if (!UNIFORM) {
+        if (!UNIFORM && !cube) {
             const unsigned long long holders = __ballot(best == d2min);
             const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)holders) - 1);
             const int idx_star = __builtin_amdgcn_readlane(best_idx, src);

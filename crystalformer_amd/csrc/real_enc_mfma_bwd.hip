@@ -160,8 +160,17 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         bx.inv_plane = __builtin_amdgcn_rcpf((float)bx.plane);
         bx.inv_S3 = __builtin_amdgcn_rcpf((float)bx.S3);
         const int T = bx.T;
+        // all active columns have the cube [-lattice_range, lattice_range]^3 (wave-uniform): under
+        // the adaptive rule with its floor switched on that is most units, and they skip the
+        // per-column box tables and lookups
+        bool cube = UNIFORM;
+        if (!UNIFORM) {
+            const int lr = p.lattice_range;
+            const bool other = col_on && (R1 != lr || R2 != lr || R3 != lr);
+            cube = bx.U1 == lr && bx.U2 == lr && bx.U3 == lr && __ballot(other) == 0ull;
+        }
         ColumnBoxes cbox{0, 0, 0};
-        if (!UNIFORM) cbox = column_boxes(R1, R2, R3, bx, lane);
+        if (!cube) cbox = column_boxes(R1, R2, R3, bx, lane);
 
         // p_t <= 2^-40 in every column when a2_weak d2 - z2_floor <= -40
         // (every row of 16 lanes holds the 16 columns, so a reduction over a row is complete)
@@ -181,7 +190,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 decode(bx, valid ? s0 + c0 + lane : 0, n1, n2, n3);
                 const float d2 = dist2(cell, (float)n1, (float)n2, (float)n3);
                 int bits = 0;
-                if (UNIFORM) {
+                if (cube) {
                     bits = valid ? 0xFFFF : 0;
                 } else {
                     bits = column_bits(cbox, n1, n2, n3);     // all lanes take part in the lookup

@@ -32,7 +32,7 @@ __all__ = [
     "KernelManager", "compile_kernels", "CUPY_AVAILABLE", "HIP_AVAILABLE",
     "RealPeriodicEncodingFuncCUDA", "RealPeriodicEncodingWithProjFuncCUDA",
     "FusedDotProductAttentionCUDA", "IrregularMeanCUDA", "compute_minimum_distance",
-    "ReciPeriodicEncodingFuncCUDA",
+    "ReciPeriodicEncodingFuncCUDA", "fused_encoding_attention",
 ]
 
 
@@ -69,6 +69,14 @@ class KernelManager:
     # d/da of the normalisation term 1.5 log(-4 pi a) (models/kernels/reci_enc_bwd.cu:41-69),
     # unlike autograd on its PyTorch path.  False reproduces the kernel, True the full derivative.
     RECI_NORMALISATION_GRAD: bool = False
+    # Blocks without Gaussian value bins (value_pe_dim 0), inference: lattice-sum bias and
+    # attention in one launch, the bias never written to memory (fused_encoding_attention).
+    FUSE_ENCODING_ATTENTION: bool = True
+    # Inside a captured graph the two operators are the faster choice (measured on the 32-crystal
+    # simplified model: 0.173 ms per replayed forward against 0.183 ms with the one-launch blocks,
+    # whose work-group per atom is bound by its chain of dependent loads), eager launches gain
+    # from the launch saved (0.55 against 0.78 ms), so capture keeps the two operators.
+    FUSE_ENCODING_ATTENTION_IN_GRAPHS: bool = False
     compiled: bool = False
 
 
@@ -221,25 +229,28 @@ class RealPeriodicEncodingFuncCUDA(torch.autograd.Function):
         return _enc_backward_tail(ga_ik, gW_k, ctx.adaptive_args)
 
 
+def _dpa_forward(ctx, que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e):
+    que_ihk = que_ihk.contiguous().detach()
+    key_ihk = key_ihk.contiguous().detach()
+    val_ihk = val_ihk.contiguous().detach()
+    aij_eh = aij_eh.contiguous().detach() if aij_eh is not None else None
+    bij_ehk = bij_ehk.contiguous().detach() if bij_ehk is not None else None
+    batch_i = batch_i.contiguous()
+    edge_ij_e = edge_ij_e.contiguous()
+    e_start_i = ops.cached_edge_row_offsets(edge_ij_e, que_ihk.shape[0])
+    output, prob_eh = ops.fused_dpa_fwd(que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, edge_ij_e, e_start_i)
+    ctx.save_for_backward(que_ihk, key_ihk, val_ihk, bij_ehk, batch_i, edge_ij_e, e_start_i, prob_eh, output)
+    ctx.has_aij = aij_eh is not None
+    return output, prob_eh
+
+
 class FusedDotProductAttentionCUDA(torch.autograd.Function):
     """out[i,h,:] = sum_j softmax_j(q_i.k_j + a_ij) (v_j + b_ij) over each atom's
     edge row.  ``que_ihk`` is expected pre-divided by sqrt(head dim)."""
 
     @staticmethod
     def forward(ctx, que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e):
-        que_ihk = que_ihk.contiguous().detach()
-        key_ihk = key_ihk.contiguous().detach()
-        val_ihk = val_ihk.contiguous().detach()
-        aij_eh = aij_eh.contiguous().detach() if aij_eh is not None else None
-        bij_ehk = bij_ehk.contiguous().detach() if bij_ehk is not None else None
-        batch_i = batch_i.contiguous()
-        edge_ij_e = edge_ij_e.contiguous()
-        e_start_i = ops.cached_edge_row_offsets(edge_ij_e, que_ihk.shape[0])
-        output, prob_eh = ops.fused_dpa_fwd(que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, edge_ij_e, e_start_i)
-        ctx.save_for_backward(que_ihk, key_ihk, val_ihk, bij_ehk, batch_i, edge_ij_e, e_start_i, prob_eh,
-                              output)
-        ctx.has_aij = aij_eh is not None
-        return output
+        return _dpa_forward(ctx, que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e)[0]
 
     @staticmethod
     def backward(ctx, go_ihk):
@@ -248,6 +259,47 @@ class FusedDotProductAttentionCUDA(torch.autograd.Function):
             que_ihk, key_ihk, val_ihk, bij_ehk, batch_i, edge_ij_e, e_start_i, prob_eh, output,
             go_ihk.contiguous().detach())
         return gque, gkey, gval, (gaij if ctx.has_aij else None), gbij, None, None
+
+
+def fused_encoding_attention(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, que_ihk, key_ihk, val_ihk,
+                             rvlen_n=None, cutoff_radius=None) -> Optional[Tensor]:
+    """``FusedDotProductAttentionCUDA(que, key, val, RealPeriodicEncoding...(a, ..., K=0)[0], None, ...)``
+    as one launch, for inference (no autograd graph is recorded and nothing is saved for a
+    backward pass).  Returns ``None`` when the fused kernel does not serve the call (switched off,
+    rows too long for it, row lengths unknown under stream capture): the caller then runs the two
+    operators."""
+    if not KernelManager.FUSE_ENCODING_ATTENTION or not a_ik.is_cuda:
+        return None
+    if torch.cuda.is_current_stream_capturing() and not KernelManager.FUSE_ENCODING_ATTENTION_IN_GRAPHS:
+        return None
+    edge_ij_e = edge_ij_e.contiguous()
+    N, H = a_ik.shape
+    e_start_i = ops.cached_edge_row_offsets(edge_ij_e, N)
+    max_row = ops.cached_max_row(edge_ij_e, e_start_i)
+    if max_row is None or max_row * (H + 1) * 4 > 64 * 1024 or H not in (1, 2, 4, 8, 16):
+        return None
+    return ops.fused_enc_dpa_fwd(a_ik.detach(), rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i,
+                                 que_ihk.detach(), key_ihk.detach(), val_ihk.detach(), max_row, rvlen_n,
+                                 cutoff_radius, KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
+
+
+class FusedDotProductAttentionWithWeights(torch.autograd.Function):
+    """:class:`FusedDotProductAttentionCUDA` that also hands out the softmax weights (E,H), which
+    the kernel writes anyway; they carry no gradient.  For ``need_weights=True`` of the module
+    (the reference's fused operator returns no weights, so its module can only serve that option
+    through the per-crystal loop, models/indexed_lattice_multi_head_attention_cuda.py:181-186, 782-786)."""
+
+    @staticmethod
+    def forward(ctx, que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e):
+        out, prob = _dpa_forward(ctx, que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e)
+        weights = prob.clone()          # (the saved tensor itself must not be an output)
+        if hasattr(ctx, "mark_non_differentiable"):
+            ctx.mark_non_differentiable(weights)
+        return out, weights
+
+    @staticmethod
+    def backward(ctx, go_ihk, _gprob):
+        return FusedDotProductAttentionCUDA.backward(ctx, go_ihk)
 
 
 class ReciPeriodicEncodingFuncCUDA(torch.autograd.Function):

@@ -39,6 +39,7 @@ SIGNATURES = {
     "cf_static_scratch_bytes": (_i64, []),
     "cf_real_enc_bwd_static": (_int, [_ptr] * 9 + [_i64] * 6 + [_dbl, _dbl, _ptr, _i64, _ptr, _dbl, _int, _int,
                                                                 _ptr, _i64, _ptr, _ptr, _ptr]),
+    "cf_fused_enc_dpa_fwd": (_int, [_ptr] * 9 + [_i64] * 6 + [_ptr, _dbl, _int, _int, _i64, _ptr, _ptr]),
     "cf_translation_ranges": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _dbl, _int, _int, _ptr, _ptr]),
     "cf_fused_dpa_fwd": (_int, [_ptr] * 7 + [_i64] * 5 + [_ptr, _ptr, _ptr]),
     "cf_fused_dpa_bwd": (_int, [_ptr] * 9 + [_i64] * 6 + [_ptr] * 9),

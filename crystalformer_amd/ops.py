@@ -90,7 +90,7 @@ class _timed:
 # and the CSR offsets are built once.  Entries keep their key tensors alive, so a
 # recycled address can never alias a stale entry.
 _index_cache: list = []
-_INDEX_CACHE_SIZE = 24
+_INDEX_CACHE_SIZE = 64
 
 
 def _cache_lookup(kind: str, *keys: Tensor):
@@ -275,6 +275,48 @@ def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
             ptr(ga), ptr(gW), stream_handle(dev))
     check(rc, "cf_real_enc_bwd")
     return ga, gW
+
+
+def cached_max_row(edge_ij_e: Tensor, e_start_i: Tensor) -> Optional[int]:
+    """Largest number of edges of one source atom, read back once per edge list (batch layouts
+    know it from their sizes).  ``None`` when it is not known and cannot be read (stream capture)."""
+    sig, hit = _cache_lookup("max_row", edge_ij_e)
+    if hit is not None:
+        return hit
+    if edge_ij_e.is_cuda and torch.cuda.is_current_stream_capturing():
+        return None
+    rows = e_start_i[1:] - e_start_i[:-1]
+    return _cache_store(sig, (edge_ij_e,), int(rows.max().item()) if rows.numel() else 0)
+
+
+def fused_enc_dpa_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor,
+                      e_start_i: Tensor, que: Tensor, key: Tensor, val: Tensor, max_row: int,
+                      rvlen_n: Optional[Tensor] = None, cutoff_radius: Optional[float] = None,
+                      lattice_range: int = 2, minimum_range: int = 0) -> Tensor:
+    """Lattice-sum bias (no Gaussian value bins) and attention in one launch, inference only:
+    what ``real_enc_fwd(K=0)`` followed by ``fused_dpa_fwd`` yield, without ``z`` in memory."""
+    dev = require_device(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, que, key, val, rvlen_n)
+    a_ik, rpos_ij_e, tvecs_n = _f32(a_ik, "a_ik"), _f32(rpos_ij_e, "rpos_ij_e"), _f32(tvecs_n, "tvecs_n")
+    que, key, val, rvlen_n = _f32(que, "que"), _f32(key, "key"), _f32(val, "val"), _f32(rvlen_n, "rvlen_n")
+    batch_i, edge_ij_e, e_start_i = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e"), \
+        _i64(e_start_i, "e_start_i")
+    N, H = a_ik.shape
+    E = edge_ij_e.shape[1]
+    B = tvecs_n.shape[0]
+    Dk, Dv = que.shape[-1], val.shape[-1]
+    if que.shape != (N, H, Dk) or key.shape != (N, H, Dk) or val.shape != (N, H, Dv):
+        raise _lib.CrystalformerHipError("fused_enc_dpa_fwd: q/k/v must be (N,H,Dk), (N,H,Dk), (N,H,Dv)")
+    if rpos_ij_e.shape != (E, 3) or batch_i.shape != (N,) or e_start_i.shape != (N + 1,):
+        raise _lib.CrystalformerHipError("fused_enc_dpa_fwd: inconsistent input shapes")
+    cutoff = 0.0 if (cutoff_radius is None or rvlen_n is None) else float(cutoff_radius)
+    out = torch.empty((N, H, Dv), dtype=torch.float32, device=dev)
+    with device_guard(dev), _timed("fused_enc_dpa_fwd", E=E, H=H, Dk=Dk, Dv=Dv):
+        rc = _lib.load().cf_fused_enc_dpa_fwd(
+            ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i), ptr(que),
+            ptr(key), ptr(val), N, H, E, B, Dk, Dv, ptr(rvlen_n), cutoff, int(lattice_range), int(minimum_range),
+            int(max_row), ptr(out), stream_handle(dev))
+    check(rc, "cf_fused_enc_dpa_fwd")
+    return out
 
 
 def translation_ranges(a_ik: Tensor, rvlen_n: Optional[Tensor], batch_i: Tensor,
@@ -574,6 +616,8 @@ def batch_layout(sizes: Tensor, batch_i: Tensor) -> BatchLayout:
     if lay.pairs is not None:
         s_, _ = _cache_lookup("pairs", lay.batch, lay.edges)
         _cache_store(s_, (lay.batch, lay.edges), lay.pairs)
+    s_, _ = _cache_lookup("max_row", lay.edges)                # a row has as many edges as its crystal atoms
+    _cache_store(s_, (lay.edges,), max(sizes_host) if sizes_host else 0)
     s_, _ = _cache_lookup("dense", lay.batch, lay.edges)       # dense by construction
     _cache_store(s_, (lay.batch, lay.edges), (sizes,))
     s_, _ = _cache_lookup("offsets", lay.batch)

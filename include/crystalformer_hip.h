@@ -164,6 +164,28 @@ int cf_real_enc_bwd_static(const float *a_ik, const float *rpos_ij_e, const floa
                            float *ga_ik, float *gW_k, void *stream);
 
 /*
+ * Lattice-sum bias and the attention that consumes it in one launch, for blocks without
+ * Gaussian value bins (K = 0, the "simplified" model): out[i,h,:] = sum_j softmax_j(q_i.k_j +
+ * z_ij)[j] v_j with z_ij = log sum_n exp(a_ih |r_ij + n.L|^2), z and the probabilities kept
+ * on chip.  Replaces the pair of launches real_enc_proj_fwd -> fused_dpa_fwd
+ * (models/cuda_funcs/real_space_enc_proj.py:70-97 followed by
+ *  models/cuda_funcs/fused_dpa.py:36-61) when nothing downstream needs z (inference).
+ *
+ * Arguments as for cf_real_enc_fwd (K = 0) and cf_fused_dpa_fwd (no b_ij); que is pre-divided
+ * by sqrt(Dk).  edge_ij_e must be sorted by source atom (e_start_i its CSR offsets); any
+ * such list is accepted.  max_row is an upper bound on the edges of one source atom: a
+ * work-group keeps its row's max_row * H logits in LDS, 64 KB at most (rows of up to 1820
+ * edges at H = 8), beyond that CF_ERR_UNSUPPORTED.
+ * Output: out (N,H,Dv); rows of atoms without edges are zero.
+ */
+int cf_fused_enc_dpa_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                         const int64_t *batch_i, const int64_t *edge_ij_e, const int64_t *e_start_i,
+                         const float *que, const float *key, const float *val,
+                         int64_t N, int64_t H, int64_t E, int64_t B, int64_t Dk, int64_t Dv,
+                         const float *rvlen_n, double cutoff_radius, int lattice_range,
+                         int minimum_range, int64_t max_row, float *out, void *stream);
+
+/*
  * Per (atom, head) translation half-widths the encoding kernels use,
  * R_out (N,H,3) int32.  Exposes the rule of models/kernels/real_enc_fwd.cu:58-85
  * for bit-exact checks and work counting.

@@ -1106,3 +1106,71 @@ def test_sparse_edge_list_takes_the_per_edge_kernels(dev):
         out.sum().backward()
     # an unsorted batch index is refused as well
     assert ops.dense_block_layout(torch.tensor([1, 0, 0], device=dev), tp.get_edge_index([1, 2]).to(dev)) is None
+
+
+# ------------------------------------ lattice sums and attention in one launch
+def test_fused_encoding_attention_on_the_simplified_model_batch(dev):
+    """Blocks without Gaussian value bins: bias and attention from one launch against the CPU
+    path's two steps (dense (E,R) lattice sum, per-crystal softmax) on the 32-crystal batch of the
+    simplified configuration, and against the two separate kernels."""
+    from crystalformer_amd.synthetic import make_config_batch
+    b = make_config_batch("cfg1_simplified_b32")
+    p = Problem(b, H=8, K=0, seed=91)
+    p.a = -(1.0 + 0.1 * p.randn(p.N, 8)).clamp_min(0.5) / (2 * 1.4 * 1.4)
+    q, k, v = p.randn(p.N, 8, 16), p.randn(p.N, 8, 16), p.randn(p.N, 8, 16)
+    z_ref, _ = tp.periodic_encoding(p.a, p.b.pos, p.b.batch, p.b.trans_vec, p.edges, 2)
+    out_ref, prob_ref = tp.indexed_attention(q.double(), k.double(), v.double(), p.b.sizes, p.edges, z_ref.double(),
+                                             None)
+    a, rpos, tv, bt, ed, es, qd, kd, vd = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start,
+                                                 q / 4.0, k, v)
+    out = ops.fused_enc_dpa_fwd(a, rpos, tv, bt, ed, es, qd, kd, vd, int(p.b.sizes.max()), None, 0.0, 2, 0)
+    out_atol, _ = dpa_atols(p, q, k, v, None, prob_ref.float(), out_ref.float())
+    assert_close(out, out_ref.float(), "out", atol=out_atol)
+    z, _ = ops.real_enc_fwd(a, rpos, tv, bt, ed, 0, 1.0, 1.0, None, None, 0.0, 2, 0)
+    two, _ = ops.fused_dpa_fwd(qd, kd, vd, z, None, ed, es)
+    assert_close(out, two, "one launch vs two", rtol=2e-6)
+
+
+@pytest.mark.parametrize("H,Dk,Dv,sizes", [(8, 16, 16, [1, 5, 70, 2]), (4, 8, 32, [3, 130]), (1, 5, 4, [7, 2]),
+                                           (16, 16, 16, [9, 1]), (2, 64, 20, [4, 33])])
+@pytest.mark.parametrize("cutoff,lr,mr", [(0.0, 2, 0), (-3.5, 2, 2), (-3.5, 1, 0), (4.0, 1, 1)])
+def test_fused_encoding_attention_against_the_kernel_oracles(dev, H, Dk, Dv, sizes, cutoff, lr, mr):
+    """Head counts and widths, rows longer than a wavefront, adaptive boxes per head, and an
+    arbitrary sorted edge list with an atom that keeps no edge (its output row is zero)."""
+    p = Problem(sizes, H=H, K=0, seed=92)
+    g = p.g
+    q = p.randn(p.N, H, Dk) / math.sqrt(Dk)
+    k, v = p.randn(p.N, H, Dk), p.randn(p.N, H, Dv)
+    keep = torch.rand(p.E, generator=g) > 0.25
+    keep &= p.edges[0] != 3
+    for edges, rpos in ((p.edges, p.rpos), (p.edges[:, keep].contiguous(), p.rpos[keep].contiguous())):
+        e_start = tp.edge_row_offsets(edges, p.N)
+        z_ref, _ = ks.real_enc_fwd(p.a, rpos, p.b.trans_vec, p.b.batch, edges, 0, 1.0, 1.0, None, p.rvlen, cutoff, lr,
+                                   mr)
+        out_ref, _ = ks.fused_dpa_fwd(q, k, v, z_ref, None, edges, e_start)
+        max_row = int((e_start[1:] - e_start[:-1]).max())
+        out = ops.fused_enc_dpa_fwd(*to_dev(dev, p.a, rpos, p.b.trans_vec, p.b.batch, edges, e_start, q, k, v),
+                                    max_row, p.rvlen.to(dev), cutoff, lr, mr)
+        assert_close(out, out_ref, "out")
+        if edges.shape[1] < p.E and p.N > 3:
+            assert float(out[3].abs().max()) == 0.0
+
+
+def test_fused_encoding_attention_limits(dev):
+    p = Problem([2, 3], H=8, K=0, seed=93)
+    q = p.randn(p.N, 8, 16)
+    args = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, q, q, q)
+    with pytest.raises(lib.CrystalformerHipError, match="64 KB"):
+        ops.fused_enc_dpa_fwd(*args, 4000)
+    empty = ops.fused_enc_dpa_fwd(torch.zeros(0, 8, device=dev), torch.zeros(0, 3, device=dev),
+                                  torch.zeros(0, 3, 3, device=dev), torch.zeros(0, dtype=torch.long, device=dev),
+                                  torch.zeros(2, 0, dtype=torch.long, device=dev),
+                                  torch.zeros(1, dtype=torch.long, device=dev), torch.zeros(0, 8, 16, device=dev),
+                                  torch.zeros(0, 8, 16, device=dev), torch.zeros(0, 8, 16, device=dev), 0)
+    assert empty.shape == (0, 8, 16)
+    # the module takes the one-launch path only when nothing needs the bias afterwards
+    assert hip_funcs.KernelManager.FUSE_ENCODING_ATTENTION
+    a = p.a.to(dev).requires_grad_(True)
+    hip_funcs.compile_kernels(2, 8, 16, 0, 16, False)
+    got = hip_funcs.fused_encoding_attention(a, *args[1:5], *args[6:9])
+    assert got is not None and not got.requires_grad

@@ -292,6 +292,29 @@ def test_training_step_at_128_crystals(dev):
     print("worst gradient error:", max(worst.items(), key=lambda kv: kv[1]))
 
 
+def test_simplified_model_takes_the_one_launch_blocks(dev):
+    """The simplified configuration (no value bins) in inference runs bias + attention as one
+    launch per block: same outputs as with the switch off (two operators), and the encoding
+    operator is not called at all."""
+    cfg, model = build_model("cfg1_simplified_b32", adaptive_cutoff_sigma=0.0)
+    model.to(dev).eval()
+    b = make_config_batch("cfg1_simplified_b32").to(dev)
+    calls = []
+    orig = ops.real_enc_fwd
+    ops.real_enc_fwd = lambda *a, **kw: (calls.append(1), orig(*a, **kw))[1]
+    try:
+        with torch.no_grad():
+            y_one = model(b)
+            assert not calls
+            hip_funcs.KernelManager.FUSE_ENCODING_ATTENTION = False
+            y_two = model(b)
+            assert len(calls) == cfg.num_layers
+    finally:
+        hip_funcs.KernelManager.FUSE_ENCODING_ATTENTION = True
+        ops.real_enc_fwd = orig
+    assert_close(y_one, y_two, "one launch vs two operators", rtol=2e-6)
+
+
 def test_full_size_properties_and_sampled_edges(dev):
     """Config 2 and the 444-atom stress cells at full size: sampled edges
     against the C oracle under the adaptive box, plus properties that hold at any
@@ -579,3 +602,38 @@ def test_fused_training_step_follows_plain_step_on_changing_batches(dev):
         lf = float(fused_training_step(m_fused, b, fopt))
         assert abs(lp - lf) <= 2e-4 * max(1.0, abs(lp)), (step, lp, lf)
     assert float(fopt.state[0]) == 5
+
+
+def test_attention_module_returns_weights_on_request(dev):
+    """need_weights=True (the reference forward's default): the module returns the softmax weights
+    averaged over the heads, one per edge, as the reference's per-crystal loop does
+    (models/indexed_lattice_multi_head_attention_cuda.py:782-786); output and gradients are those
+    of the call without weights."""
+    cfg, model = build_model("cfg2_default_b128", num_layers=1, value_pe_dist_real=16, adaptive_cutoff_sigma=0.0)
+    model.to(dev).train()
+    attn = model.encoder.layers[0].self_attn
+    p = Problem([3, 1, 6], H=8, K=0, seed=95)
+    x = p.randn(p.N, 128).to(dev).requires_grad_(True)
+    bt, ed = p.b.batch.to(dev), p.edges.to(dev)
+    rpos, tv = p.rpos.to(dev), p.b.trans_vec.to(dev)
+    out_w, weights = attn(x, x, x, bt, bt, ed, rpos, None, tv, need_weights=True)
+    go = p.randn(p.N, 128).to(dev)
+    (out_w * go).sum().backward()
+    gx_w, x.grad = x.grad.clone(), None
+    out, values = attn(x, x, x, bt, bt, ed, rpos, None, tv, need_weights=False)
+    (out * go).sum().backward()
+    assert torch.equal(out_w, out) and torch.equal(gx_w, x.grad)
+    assert weights.shape == (p.E,) and not weights.requires_grad and values.shape == (p.E, 8, 16)
+    rows = torch.zeros(p.N, device=dev).index_add_(0, ed[0], weights)
+    assert float((rows - 1).abs().max()) < 1e-5                  # each atom's weights sum to one
+    # against the oracle's probabilities for the same projections
+    P = {k: v.detach().cpu() for k, v in attn.state_dict().items()}
+    xq = x.detach().cpu()
+    q = (xq @ P["q_proj_weight"].T + P["in_proj_bias"][:128]).view(p.N, 8, 16)
+    k = (xq @ P["k_proj_weight"].T + P["in_proj_bias"][128:256]).view(p.N, 8, 16)
+    v = (xq @ P["v_proj_weight"].T + P["in_proj_bias"][256:]).view(p.N, 8, 16)
+    a = tp.gaussian_exponents(q, P["lattice_pos_weights"], P["gauss_scale"].clone(), False, True, cfg.gauss_lb_real,
+                              0.1, 1.4)
+    z, vpe = tp.periodic_encoding(a, p.b.pos, p.b.batch, p.b.trans_vec, p.edges, 2, 16, 14.0, 1.0, P["pe_dist_proj"])
+    _, prob = tp.indexed_attention(q, k, v, p.b.sizes, p.edges, z, vpe)
+    assert_close(weights, prob.mean(dim=1), "weights")
