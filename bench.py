@@ -158,7 +158,9 @@ def ingest_counters(directory: str, key: str, kernel: str) -> int:
     copy_kib = 256.0 * 1024.0
     for cname, field in (("FETCH_SIZE", "fetch"), ("WRITE_SIZE", "write")):
         if cname in k:
-            factor = copy_kib / mean(agg["copy"][cname]) if agg["copy"].get(cname) else None
+            # the calibration copies are the large ones (small host-side copies share the kernel name)
+            big = [x for x in agg["copy"].get(cname, []) if x >= 0.5 * max(agg["copy"][cname])]
+            factor = copy_kib / mean(big) if big else None
             entry[f"{field}_kib_counter"] = round(k[cname], 1)
             entry[f"{field}_copy_factor"] = None if factor is None else round(factor, 4)
             if factor is not None:
