@@ -310,6 +310,9 @@ def fused_enc_dpa_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i:
         raise _lib.CrystalformerHipError("fused_enc_dpa_fwd: inconsistent input shapes")
     cutoff = 0.0 if (cutoff_radius is None or rvlen_n is None) else float(cutoff_radius)
     out = torch.empty((N, H, Dv), dtype=torch.float32, device=dev)
+    if _eval_counter is not None:
+        _eval_counter.append(count_translation_evals(a_ik, rvlen_n, batch_i, edge_ij_e, cutoff,
+                                                     int(lattice_range), int(minimum_range)))
     with device_guard(dev), _timed("fused_enc_dpa_fwd", E=E, H=H, Dk=Dk, Dv=Dv):
         rc = _lib.load().cf_fused_enc_dpa_fwd(
             ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i), ptr(que),
