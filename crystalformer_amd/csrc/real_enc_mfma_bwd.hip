@@ -97,6 +97,27 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 }
         }
     };
+    // The cube [-lattice_range, lattice_range]^3 (every unit of the fixed rule, most units of the adaptive
+    // one) is decoded once: for the lane's translation of each of the first two chunks of 64, n + 8 per
+    // axis in 4 bits, all in one register (unpacking costs a fifth of decoding again).
+    int npre = 0;
+    const int cube_T = (2 * p.lattice_range + 1) * (2 * p.lattice_range + 1) * (2 * p.lattice_range + 1);
+    const bool cube_packed = p.lattice_range <= 7 && cube_T <= 2 * WAVE;
+    if (cube_packed) {
+        BoxDims b0;
+        b0.U1 = b0.U2 = b0.U3 = p.lattice_range;
+        b0.S3 = b0.S2 = 2 * p.lattice_range + 1;
+        b0.plane = b0.S2 * b0.S3;
+        b0.T = cube_T;
+        b0.inv_plane = 1.0f / (float)b0.plane;
+        b0.inv_S3 = 1.0f / (float)b0.S3;
+#pragma unroll
+        for (int ch = 0; ch < 2; ch++) {
+            int n1, n2, n3;
+            decode(b0, min(ch * WAVE + lane, b0.T - 1), n1, n2, n3);
+            npre |= ((n1 + 8) | ((n2 + 8) << 4) | ((n3 + 8) << 8)) << (12 * ch);
+        }
+    }
     const int stride = gridDim.x;
     RoundPos pos = round_pos(blockIdx.x, rounds_per_hg, p.head_groups);
     RoundPos pos_next = round_pos(blockIdx.x + stride, rounds_per_hg, p.head_groups);
@@ -187,7 +208,14 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             for (int c0 = 0; c0 < cnt; c0 += WAVE) {
                 const bool valid = c0 + lane < cnt;
                 int n1, n2, n3;
-                decode(bx, valid ? s0 + c0 + lane : 0, n1, n2, n3);
+                if (cube && cube_packed) {                   // (wave-uniform; the cube is a single pass: s0 == 0)
+                    const unsigned f = (unsigned)npre >> (c0 == 0 ? 0 : 12);
+                    n1 = (int)(f & 15u) - 8;
+                    n2 = (int)((f >> 4) & 15u) - 8;
+                    n3 = (int)((f >> 8) & 15u) - 8;
+                } else {
+                    decode(bx, valid ? s0 + c0 + lane : 0, n1, n2, n3);
+                }
                 const float d2 = dist2(cell, (float)n1, (float)n2, (float)n3);
                 int bits = 0;
                 if (cube) {
