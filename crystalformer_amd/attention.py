@@ -122,24 +122,47 @@ def conditional_projection(proj: Tensor, onehot: Tensor, edges: Tensor, mode: st
     return W.reshape(-1, proj.shape[1], proj.shape[2], proj.shape[3])
 
 
+NORM_FUNC_MODES = {"default": 0, "softmax": 1, "exp": 2, "linear": 3, "sigmoid": 4, "softplus": 5, "elu": 6,
+                   "elu+1": 7, "abs": 8}
+
+
 def loop_attention(q: Tensor, k: Tensor, v: Tensor, batch: Tensor, edges: Tensor,
-                   bias: Optional[Tensor], values: Optional[Tensor]) -> Tensor:
-    """Per-crystal softmax/aggregate with stock torch ops: what the reference
-    runs when its numerics switch is below 2
-    (models/indexed_lattice_multi_head_attention_cuda.py:231-306, mode 0)."""
+                   bias: Optional[Tensor], values: Optional[Tensor], norm_func_mode=0,
+                   dropout_p: float = 0.0) -> Tuple[Tensor, Tensor]:
+    """Per-crystal normalise/aggregate with stock torch ops: what the reference itself runs, on its
+    kernel path too, whenever its fused operator does not apply -- numerics switch below 2, a
+    normalisation other than the softmax over all keys, or dropout on the weights
+    (models/indexed_lattice_multi_head_attention_cuda.py:231-306).  Returns (output, weights (E,H))."""
     logits = (q[edges[0]] * k[edges[1]]).sum(dim=-1)
-    if bias is not None:
-        logits = logits + bias
     sizes = torch.zeros(int(batch.max().item()) + 1, dtype=torch.long, device=q.device)
     sizes.scatter_add_(0, batch, torch.ones_like(batch))
     sizes = sizes.tolist()
     esz = [s * s for s in sizes]
-    prob = torch.cat([F.softmax(a.view(s, s, -1), dim=1).view(s * s, -1)
-                      for a, s in zip(torch.split_with_sizes(logits, esz), sizes)])
+
+    def row_softmax(x):
+        return torch.cat([F.softmax(a.view(s, s, -1), dim=1).view(s * s, -1)
+                          for a, s in zip(torch.split_with_sizes(x, esz), sizes)])
+    mode = NORM_FUNC_MODES.get(norm_func_mode, norm_func_mode)
+    mode = abs(mode) if isinstance(mode, int) else mode
+    w = 0 if bias is None else bias
+    if mode == 0:
+        prob = row_softmax(logits + w)                       # softmax over all keys of the crystal
+    elif mode == 1:
+        prob = row_softmax(logits) * torch.exp(w) if bias is not None else row_softmax(logits)
+    elif mode == 2:
+        prob = torch.exp(logits + w)
+    elif mode in (3, 4, 5, 6, 7, 8):
+        f = {3: lambda x: x, 4: torch.sigmoid, 5: F.softplus, 6: F.elu, 7: lambda x: F.elu(x) + 1, 8: torch.abs}[mode]
+        prob = f(logits) * (torch.exp(w) if bias is not None else 1.0)
+    else:
+        raise ValueError(f"norm_func_mode must be 0 to 8 but {norm_func_mode} is given.")
+    if dropout_p > 0.0:
+        prob = F.dropout(prob, p=dropout_p)
     msg = v[edges[1]] if values is None else v[edges[1]] + values
     msg = prob[..., None] * msg
-    return torch.cat([m.view((s, s) + m.shape[1:]).sum(dim=1)
-                      for m, s in zip(torch.split_with_sizes(msg, esz), sizes)])
+    out = torch.cat([m.view((s, s) + m.shape[1:]).sum(dim=1)
+                     for m, s in zip(torch.split_with_sizes(msg, esz), sizes)])
+    return out, prob
 
 
 class CrystalformerMultiheadAttentionCUDA(Module):
@@ -310,25 +333,45 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             else:
                 return self._project_output(attn, n, vd, fused_linear, fused_train, residual, need_weights, None)
 
-        if P.norm_func_mode != 0:
-            raise NotImplementedError("norm_func_mode != 0 is not served by the HIP path")
-        if self.training and self.dropout > 0.0:
-            raise NotImplementedError("attention dropout is not served by the HIP path")
         if qs is None:
             qs = q / math.sqrt(q.shape[-1])
         weights = None
-        if need_weights:
+        dropout_p = self.dropout if self.training else 0.0
+        plain = P.norm_func_mode in (0, "default") and dropout_p == 0.0
+        if not plain or config.REPRODUCIBLITY_STATE < 2 or batch_q is not batch_kv:
+            # other normalisations, dropout on the weights, or the numerics switch: the per-crystal
+            # torch loop, as in the reference
+            attn, prob = loop_attention(qs, k, v, batch_q, edges, bias, values, P.norm_func_mode, dropout_p)
+            if isinstance(P.norm_func_mode, int) and P.norm_func_mode < 0:
+                attn = attn * self._attention_scale(prob, batch_q)
+            if need_weights:
+                weights = prob.detach().mean(dim=1)
+        elif need_weights:
             # softmax weights averaged over the heads, (E,), as the reference's loop path returns them
             # (models/indexed_lattice_multi_head_attention_cuda.py:782-786)
             attn, prob = hip_funcs.call(hip_funcs.FusedDotProductAttentionWithWeights, qs, k, v, bias, values,
                                         batch_q, edges)
             weights = prob.mean(dim=1)
-        elif config.REPRODUCIBLITY_STATE >= 2 and batch_q is batch_kv:
-            attn = hip_funcs.call(FusedDotProductAttentionCUDA, qs, k, v, bias, values, batch_q, edges)
         else:
-            attn = loop_attention(qs, k, v, batch_q, edges, bias, values)
+            attn = hip_funcs.call(FusedDotProductAttentionCUDA, qs, k, v, bias, values, batch_q, edges)
         return self._project_output(attn, n, vd, fused_linear, fused_train, residual, need_weights,
                                     weights if need_weights else values)
+
+    def _attention_scale(self, prob: Tensor, batch_q: Tensor) -> Tensor:
+        """Negative norm_func_mode: outputs times the stored scale, or the reciprocal of the mean (over
+        crystals, of the mean over queries and heads) total |weight| per query, stored once in training
+        (models/indexed_lattice_multi_head_attention_cuda.py:760-777)."""
+        if bool(self.atten_scale[0] > 0):
+            return self.atten_scale[0]
+        sizes = torch.zeros(int(batch_q.max().item()) + 1, dtype=torch.long, device=prob.device)
+        sizes.scatter_add_(0, batch_q, torch.ones_like(batch_q))
+        sizes = sizes.tolist()
+        parts = torch.split_with_sizes(prob.detach().abs(), [s * s for s in sizes])
+        scale = torch.stack([x.view(s, s, -1).sum(dim=1).mean() for x, s in zip(parts, sizes)]).mean().reciprocal()
+        if self.training:
+            with torch.no_grad():
+                self.atten_scale[0] = scale
+        return scale
 
     def _project_output(self, attn, n, vd, fused_linear, fused_train, residual, need_weights, values):
         attn = attn.contiguous().view(n, vd)

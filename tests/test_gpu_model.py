@@ -637,3 +637,61 @@ def test_attention_module_returns_weights_on_request(dev):
     z, vpe = tp.periodic_encoding(a, p.b.pos, p.b.batch, p.b.trans_vec, p.edges, 2, 16, 14.0, 1.0, P["pe_dist_proj"])
     _, prob = tp.indexed_attention(q, k, v, p.b.sizes, p.edges, z, vpe)
     assert_close(weights, prob.mean(dim=1), "weights")
+
+
+def test_other_normalisations_and_dropout_take_the_torch_loop(dev):
+    """norm_func_mode != 0 and dropout on the weights are served by the per-crystal torch loop, as
+    in the reference (models/indexed_lattice_multi_head_attention_cuda.py:231-306).  Mode 0 through
+    the loop equals the fused operator; the other modes are checked against their defining
+    expression on one crystal; dropout leaves the expectation of the output unchanged.  (The
+    reference ships no vectors for these modes: parity with it is not pinned beyond the formulas.)"""
+    from crystalformer_amd.attention import loop_attention
+    p = Problem([5, 1, 3], H=4, K=0, seed=96)
+    q, k, v = (p.randn(p.N, 4, 8).to(dev) for _ in range(3))
+    bias, vals = p.randn(p.E, 4).to(dev), p.randn(p.E, 4, 8).to(dev)
+    bt, ed = p.b.batch.to(dev), p.edges.to(dev)
+    fused = hip_funcs.FusedDotProductAttentionCUDA.apply(q, k, v, bias, vals, bt, ed)
+    out0, prob0 = loop_attention(q, k, v, bt, ed, bias, vals)
+    assert_close(out0, fused, "mode 0 loop vs fused")
+    i, j = ed
+    logits = (q[i] * k[j]).sum(-1)
+    msg = v[j] + vals
+    expect = {2: torch.exp(logits + bias), 3: logits * torch.exp(bias), 4: torch.sigmoid(logits) * torch.exp(bias),
+              7: (torch.nn.functional.elu(logits) + 1) * torch.exp(bias), 8: logits.abs() * torch.exp(bias)}
+    for mode, w in expect.items():
+        out, prob = loop_attention(q, k, v, bt, ed, bias, vals, mode)
+        ref = torch.zeros_like(out).index_add_(0, i, w[..., None] * msg)
+        assert_close(out, ref, f"mode {mode}", rtol=1e-5)
+        assert_close(loop_attention(q, k, v, bt, ed, bias, vals, -mode)[0], ref, f"mode -{mode}")
+    out1, prob1 = loop_attention(q, k, v, bt, ed, bias, vals, "softmax")
+    ref1 = torch.zeros_like(out1).index_add_(0, i, (loop_attention(q, k, v, bt, ed, None, None)[1] * torch.exp(bias))[..., None] * msg)
+    assert_close(out1, ref1, "mode 1")
+    # dropout: mean over many draws approaches the output without dropout
+    torch.manual_seed(0)
+    draws = torch.stack([loop_attention(q, k, v, bt, ed, bias, vals, 0, 0.3)[0] for _ in range(400)])
+    assert float((draws.mean(0) - out0).abs().max()) < 0.15 * float(out0.abs().max())
+    assert float((draws[0] - out0).abs().max()) > 1e-3
+    # the module: training with dropout runs, evaluation ignores it; a negative mode stores its scale once
+    cfg, model = build_model("cfg2_default_b128", num_layers=1, value_pe_dist_real=16, adaptive_cutoff_sigma=0.0,
+                             dropout=0.0)
+    attn = model.encoder.layers[0].self_attn.to(dev)
+    x = p.randn(p.N, 128).to(dev)
+    args = (x, x, x, bt, bt, ed, p.rpos.to(dev), None, p.b.trans_vec.to(dev))
+    attn.eval()
+    with torch.no_grad():
+        y_eval = attn(*args, need_weights=False)[0]
+    attn.dropout = 0.4
+    with torch.no_grad():
+        assert torch.equal(attn(*args, need_weights=False)[0], y_eval)
+    attn.train()
+    y_train = attn(*args, need_weights=False)[0]
+    assert y_train.requires_grad and float((y_train.detach() - y_eval).abs().max()) > 1e-4
+    attn.dropout = 0.0
+    attn.params.norm_func_mode = -3
+    y_scaled, w = attn(*args, need_weights=True)
+    assert float(attn.atten_scale[0]) > 0 and w.shape == (p.E,)
+    attn.params.norm_func_mode = 3
+    y_plain = attn(*args, need_weights=False)[0]
+    assert_close(y_scaled - attn.out_proj.bias, (y_plain - attn.out_proj.bias) * attn.atten_scale[0], "scaled output",
+                 rtol=1e-4)
+    attn.params.norm_func_mode = 0
