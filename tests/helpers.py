@@ -38,7 +38,7 @@ DROP = 2.0 ** -40
 U_DIST = 2.0 ** -22
 
 # worst element-wise error seen per quantity, in units of its bound (1.0 = at the bound); written
-# to gpurun_out/ by tests/conftest.py at the end of a GPU session
+# out by tests/conftest.py at the end of a session when CF_REPORT_DIR is set
 elementwise_record = {}
 
 
