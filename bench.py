@@ -214,7 +214,8 @@ def train_bench(args, torch, ops, model, data, batch, state_cpu, cfg, mcfg, B, N
     eager = {"value": round(B * args.steps / elapsed, 2), "ms_per_step": round(elapsed / args.steps * 1e3, 4)}
     # Kernel durations: the encoding / attention launches of one step are re-issued back to back
     # (queue kept full), each bracketed by a pair of HIP events on the launch stream.
-    calls = {"real_enc_fwd": [], "real_enc_bwd": [], "fused_dpa_fwd": [], "fused_dpa_bwd": []}
+    calls = {"real_enc_fwd": [], "real_enc_fwd_rings": [], "real_enc_bwd": [], "fused_dpa_fwd": [],
+             "fused_dpa_bwd": []}
     originals = {name: getattr(ops, name) for name in calls}
     def detached(v):       # no autograd graph may outlive the step through the recorded arguments
         return v.detach() if torch.is_tensor(v) else v
@@ -388,6 +389,9 @@ def main() -> int:
                          "occupies (384 of its 512 work-groups by default)")
     ap.add_argument("--two-launch-blocks", action="store_true",
                     help="blocks without value bins: run bias and attention as two operators instead of one launch")
+    ap.add_argument("--no-staged-rings", action="store_true",
+                    help="every block stages its translations itself (pair kernel) instead of starting from the "
+                         "rings staged once per forward")
     ap.add_argument("--no-fresh", action="store_true", help="skip the fresh-batch (layout rebuilt every step) figure")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--train", action="store_true",
@@ -426,9 +430,11 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     lib.load()
+    from crystalformer_amd import hip_funcs
     if args.two_launch_blocks:
-        from crystalformer_amd import hip_funcs
         hip_funcs.KernelManager.FUSE_ENCODING_ATTENTION = False
+    if args.no_staged_rings:
+        hip_funcs.KernelManager.STAGED_RINGS = False
     dev = torch.device("cuda:0")
     if args.train and args.config == "cfg2_default_b128":
         args.config = "cfg4_train_b128"
@@ -504,7 +510,8 @@ def main() -> int:
         eager_elapsed, y_eager = timed(lambda: model(data), args.steps, args.warmup)
         # Kernel durations: the encoding / attention launches of one forward are re-issued back to
         # back (queue kept full), each bracketed by a pair of HIP events on the launch stream.
-        calls = {"real_enc_fwd": [], "fused_dpa_fwd": [], "fused_enc_dpa_fwd": []}
+        calls = {"real_enc_fwd": [], "real_enc_fwd_rings": [], "fused_dpa_fwd": [], "fused_enc_dpa_fwd": [],
+                 "staged_rings": []}
         originals = {name: getattr(ops, name) for name in calls}
 
         def spy_on(name):
@@ -521,7 +528,9 @@ def main() -> int:
         ops.set_event_log(log)
         for name in calls:
             for _ in range(max(args.steps, 5)):
-                for a, kw in calls[name]:
+                for a, kw in calls[name][:1] if name == "staged_rings" else calls[name]:
+                    if name == "staged_rings":
+                        ops._ring_cache.clear()           # staged again, as for a new geometry
                     originals[name](*a, **kw)
         torch.cuda.synchronize()
         ops.set_event_log(None)
@@ -557,6 +566,7 @@ def main() -> int:
     enc_ms = [s.elapsed_time(e) for (name, s, e, info) in log if name == "real_enc_fwd"]
     one_launch_ms = [s.elapsed_time(e) for (name, s, e, info) in log if name == "fused_enc_dpa_fwd"]
     dpa_ms = [s.elapsed_time(e) for (name, s, e, info) in log if name == "fused_dpa_fwd"]
+    stage_ms = [s.elapsed_time(e) for (name, s, e, info) in log if name == "real_enc_ring_stage"]
     if not enc_ms and one_launch_ms:
         enc_ms = one_launch_ms
     enc_avg_ms = sum(enc_ms) / max(len(enc_ms), 1)
@@ -600,6 +610,8 @@ def main() -> int:
             "g_evals_per_s": round(evals_per_launch / (enc_avg_ms * 1e-3) / 1e9, 3) if enc_avg_ms > 0 else 0.0},
         "fused_dpa_fwd_avg_ms": round(sum(dpa_ms) / max(len(dpa_ms), 1), 4),
     }
+    if stage_ms:           # once per forward: the translations all blocks start from
+        roofline["ring_stage_avg_ms"] = round(sum(stage_ms) / len(stage_ms), 4)
     if one_launch_ms:      # blocks without value bins, eager: bias + attention in one launch
         roofline["kernel"] = "enc_dpa_row_kernel (lattice-sum bias + attention in one launch; eager launches only)"
         roofline["fused_enc_dpa_fwd_avg_ms"] = round(sum(one_launch_ms) / len(one_launch_ms), 4)

@@ -326,8 +326,15 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                 attn = hip_funcs.fused_encoding_attention(a, points, tvecs, batch_q, edges, qs, k, v, *adaptive)
             if attn is None:
                 enc = RealPeriodicEncodingWithProjFuncCUDA if P.use_low_memory else RealPeriodicEncodingFuncCUDA
-                out = hip_funcs.call(enc, a, points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real,
-                                     dist_max, P.value_pe_width_scale, proj, *adaptive)
+                # every positive map keeps rho >= gauss_lb, so no exponent of this block lies above this bound
+                # (it lets the encoding share its staged translations between the blocks of a model)
+                # (a few ulps of slack for the positive map's own rounding)
+                hip_funcs.KernelManager.WEAKEST_EXPONENT = -0.5 * P.gauss_lb_real * P.scale_real ** -2 * (1 - 1e-5)
+                try:
+                    out = hip_funcs.call(enc, a, points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real,
+                                         dist_max, P.value_pe_width_scale, proj, *adaptive)
+                finally:
+                    hip_funcs.KernelManager.WEAKEST_EXPONENT = None
                 bias = out[0]
                 values = out[1] if len(out) >= 2 else None
             else:

@@ -40,7 +40,15 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
                               const float *gz, const float *gv, int64_t N, int64_t H, int64_t E, int64_t K,
                               int64_t D, float bin_step, float s_scale, const float *W, const float *rvlen,
                               float cutoff, int lattice_range, int min_range, float *ga_edge,
-                              float *gW_part, float *gW, const int64_t *e_start, float *ga_ik, hipStream_t st);
+                              float *gW_part, float *gW, const int64_t *e_start, float *ga_ik,
+                              const float *rings, hipStream_t st);
+
+// real_enc_ring.hip
+int launch_ring_stage(const float *rpos, const float *tvecs, const int64_t *pairs, int64_t U, int64_t K,
+                      float bin_step, float s_scale, int lattice_range, float weak_a, float *cache, hipStream_t st);
+int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U, int64_t N, int64_t H, int64_t E,
+                              int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
+                              const float *cache, float *z, float *v, hipStream_t st);
 
 #define CF_REQUIRE(cond, code, ...)            \
     do {                                       \

@@ -1063,14 +1063,18 @@ extern "C" int64_t cf_real_enc_bwd_workspace(int64_t N, int64_t H, int64_t E, in
     return bytes;
 }
 
-extern "C" int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
-                               const int64_t *batch_i, const int64_t *edge_ij_e,
-                               const int64_t *e_start_i, const float *z_ek, const float *gz_ek,
-                               const float *gv_ekd, int64_t N, int64_t H, int64_t E, int64_t B, int64_t K,
-                               int64_t D, double dist_max, double wscale, const float *W_k, int64_t W_num,
-                               const float *rvlen_n, double cutoff_radius, int lattice_range,
-                               int minimum_range, const int64_t *pairs_u, int64_t U, void *workspace,
-                               int64_t workspace_bytes, float *ga_ik, float *gW_k, void *stream)
+// cf_real_enc_bwd and cf_real_enc_bwd_rings (rings != nullptr: the pair kernel starts from the
+// staged translations; shapes and gradient sets the pair kernel does not take go to the other
+// kernels, which have no use for the rings).
+static int real_enc_bwd_entry(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                              const int64_t *batch_i, const int64_t *edge_ij_e,
+                              const int64_t *e_start_i, const float *z_ek, const float *gz_ek,
+                              const float *gv_ekd, int64_t N, int64_t H, int64_t E, int64_t B, int64_t K,
+                              int64_t D, double dist_max, double wscale, const float *W_k, int64_t W_num,
+                              const float *rvlen_n, double cutoff_radius, int lattice_range,
+                              int minimum_range, const int64_t *pairs_u, int64_t U, void *workspace,
+                              int64_t workspace_bytes, float *ga_ik, float *gW_k, const float *rings,
+                              void *stream)
 {
     EncArgs p;
     int rc = fill_args(p, "cf_real_enc_bwd", a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, N, H, E, B, K,
@@ -1105,7 +1109,8 @@ extern "C" int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const 
         }
         rc = launch_real_enc_bwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, z_ek, gz_ek,
                                        gv_ekd, N, H, E, K, D, p.bin_step, p.s_scale, W_k, rvlen_n, p.cutoff,
-                                       lattice_range, minimum_range, ga_edge, gW_part, gW_k, e_start_i, ga_ik, st);
+                                       lattice_range, minimum_range, ga_edge, gW_part, gW_k, e_start_i, ga_ik,
+                                       rings, st);
         if (rc == CF_OK) {
             CF_CHECK_LAUNCH("cf_real_enc_bwd (pairs)");     // the pair kernel and its two reductions
             return CF_OK;
@@ -1150,6 +1155,35 @@ extern "C" int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const 
         }
     }
     return CF_OK;
+}
+
+extern "C" int cf_real_enc_bwd(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                               const int64_t *batch_i, const int64_t *edge_ij_e,
+                               const int64_t *e_start_i, const float *z_ek, const float *gz_ek,
+                               const float *gv_ekd, int64_t N, int64_t H, int64_t E, int64_t B, int64_t K,
+                               int64_t D, double dist_max, double wscale, const float *W_k, int64_t W_num,
+                               const float *rvlen_n, double cutoff_radius, int lattice_range,
+                               int minimum_range, const int64_t *pairs_u, int64_t U, void *workspace,
+                               int64_t workspace_bytes, float *ga_ik, float *gW_k, void *stream)
+{
+    return real_enc_bwd_entry(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd, N, H, E,
+                              B, K, D, dist_max, wscale, W_k, W_num, rvlen_n, cutoff_radius, lattice_range,
+                              minimum_range, pairs_u, U, workspace, workspace_bytes, ga_ik, gW_k, nullptr, stream);
+}
+
+extern "C" int cf_real_enc_bwd_rings(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                                     const int64_t *batch_i, const int64_t *edge_ij_e,
+                                     const int64_t *e_start_i, const float *z_ek, const float *gz_ek,
+                                     const float *gv_ekd, int64_t N, int64_t H, int64_t E, int64_t B, int64_t K,
+                                     int64_t D, double dist_max, double wscale, const float *W_k,
+                                     int lattice_range, const int64_t *pairs_u, int64_t U, const float *rings,
+                                     void *workspace, int64_t workspace_bytes, float *ga_ik, float *gW_k,
+                                     void *stream)
+{
+    CF_REQUIRE(rings && pairs_u, CF_ERR_INVALID_ARGUMENT, "cf_real_enc_bwd_rings: rings / pairs_u is null");
+    return real_enc_bwd_entry(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd, N, H, E,
+                              B, K, D, dist_max, wscale, W_k, 1, nullptr, 0.0, lattice_range, 0, pairs_u, U,
+                              workspace, workspace_bytes, ga_ik, gW_k, rings, stream);
 }
 
 // ---- backward without a caller-provided workspace ----------------------------------

@@ -23,12 +23,16 @@ namespace {
 using namespace cf;
 using namespace cfpair;
 
-constexpr int BRING_CAP = 128;              // translations staged per pass
-constexpr int BRING_SLOTS = BRING_CAP + 16;
+constexpr int BRING_CAP = RIMG_CAP;         // translations staged per pass
+constexpr int BRING_SLOTS = RIMG_SLOTS;
 
-template <int NT, bool UNIFORM>
+// RINGS: the staged translations of every unit come from memory (p.rings, written once per
+// geometry by the staging kernel of real_enc_ring.hip; fixed cube only) instead of being worked
+// out here: no lattice or offset loads, no decoding, distances, classification or ranking.
+template <int NT, bool UNIFORM, bool RINGS>
 __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 {
+    static_assert(UNIFORM || !RINGS, "staged rings hold the fixed cube");
     extern __shared__ __align__(16) float lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -102,7 +106,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     // axis in 4 bits, all in one register (unpacking costs a fifth of decoding again).
     int npre = 0;
     const int cube_T = (2 * p.lattice_range + 1) * (2 * p.lattice_range + 1) * (2 * p.lattice_range + 1);
-    const bool cube_packed = p.lattice_range <= 7 && cube_T <= 2 * WAVE;
+    const bool cube_packed = !RINGS && p.lattice_range <= 7 && cube_T <= 2 * WAVE;
     if (cube_packed) {
         BoxDims b0;
         b0.U1 = b0.U2 = b0.U3 = p.lattice_range;
@@ -123,15 +127,18 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
     RoundPos pos_next = round_pos(blockIdx.x + stride, rounds_per_hg, p.head_groups);
     UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x, pos), lane));
     float a_cur, z_cur;
-    UnitGeom geo;
+    UnitGeom geo{};
+    RingImage img{};
     UnitIds ids_next;
     int col_edge = load_col_edge(blockIdx.x, pos);
     {
-        const float gv0 = load_unit_geom(ids, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
+        float gv0 = 0.f;
+        if (RINGS) img = load_ring_image(p.rings, unit_of(blockIdx.x, pos), lane);
+        else gv0 = load_unit_geom(ids, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
         a_cur = load_a(ids, pos);
         z_cur = load_z(ids, pos);
         const int64_t dv1 = load_unit_ids(g_pairs, unit_of(blockIdx.x + stride, pos_next), lane);
-        geo = unit_geom(gv0, !UNIFORM);
+        if (!RINGS) geo = unit_geom(gv0, !UNIFORM);
         ids_next = unit_ids(dv1);
     }
     for (int rd = blockIdx.x; rd < rounds; rd += stride) {
@@ -139,8 +146,25 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         const int64_t u = (int64_t)pos.r * WPB + wave;
         const bool unit_on = u < p.U;
         const RoundPos pos_next2 = round_pos(rd + 2 * stride, rounds_per_hg, p.head_groups);
+        int near_cnt = 0, far_cnt = 0;
+        if (RINGS) {
+            // this round's image into the ring (its previous readers are done: same wavefront,
+            // and the exchange's barriers lie in between), then the next round's image requested
+            near_cnt = unit_on ? __builtin_amdgcn_readlane(img.hdr, 0) : 0;
+            far_cnt = unit_on ? __builtin_amdgcn_readlane(img.hdr, 1) : 0;
+            store_ring_image(img, ring_d2, ring_s, ring_bits, lane);
+            if (near_cnt + 8 > 2 * WAVE || far_cnt > 0)          // slots 128 .. 143 (wave-uniform, rare)
+                copy_ring_tail(p.rings, u, ring_d2, ring_s, ring_bits, lane);
+            if (!unit_on && lane < 8) {                          // no unit: an empty near block
+                ring_d2[lane] = __builtin_inff();
+                ring_s[lane] = 0.f;
+                ring_bits[lane] = 0;
+            }
+            img = load_ring_image(p.rings, unit_of(rd + stride, pos_next), lane);
+        }
         // loads for the coming rounds, consumed just before this round's exchange
-        const float gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
+        float gv_next = 0.f;
+        if (!RINGS) gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
         const float a_next = load_a(ids_next, pos_next);
         const float z_next = load_z(ids_next, pos_next);
         const int col_edge_next = load_col_edge(rd + stride, pos_next);
@@ -202,9 +226,9 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 #pragma unroll
         for (int m = 0; m < NT; m++) accS[m] = accQ[m] = float4_t{0.f, 0.f, 0.f, 0.f};
         float px = 0.f;
-        for (int s0 = 0; s0 < T; s0 += BRING_CAP) {
-            const int cnt = min(BRING_CAP, T - s0);
-            int near_cnt = 0, far_cnt = 0;
+        for (int s0 = 0; s0 < (RINGS ? 1 : T); s0 += BRING_CAP) {
+            const int cnt = RINGS ? 0 : min(BRING_CAP, T - s0);
+            if (!RINGS) near_cnt = far_cnt = 0;
             for (int c0 = 0; c0 < cnt; c0 += WAVE) {
                 const bool valid = c0 + lane < cnt;
                 int n1, n2, n3;
@@ -264,7 +288,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 near_cnt += near_now;
                 far_cnt += __popcll(far_mask);
             }
-            if (lane < 12) {
+            if (!RINGS && lane < 12) {
                 const int pos = lane < 8 ? near_cnt + lane : BRING_SLOTS - far_cnt - 1 - (lane - 8);
                 ring_d2[pos] = __builtin_inff();
                 ring_s[pos] = 0.f;
@@ -315,7 +339,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         // the loads issued at the top of the round have landed; the descriptor of the round after
         // next is requested here and looked at after the exchange (it would otherwise occupy two
         // registers through the whole accumulation)
-        const UnitGeom geo_next = unit_geom(gv_next, !UNIFORM);
+        UnitGeom geo_next{};
+        if (!RINGS) geo_next = unit_geom(gv_next, !UNIFORM);
         const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane);
         px += __shfl_xor(px, 16, WAVE);
         px += __shfl_xor(px, 32, WAVE);
@@ -530,7 +555,8 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
                               const float *gz, const float *gv, int64_t N, int64_t H, int64_t E, int64_t K,
                               int64_t D, float bin_step, float s_scale, const float *W, const float *rvlen,
                               float cutoff, int lattice_range, int min_range, float *ga_edge,
-                              float *gW_part, float *gW, const int64_t *e_start, float *ga_ik, hipStream_t st)
+                              float *gW_part, float *gW, const int64_t *e_start, float *ga_ik,
+                              const float *rings, hipStream_t st)
 {
     if (K < 1 || K > 64 || !W || D < 1 || D > 16) return CF_ERR_UNSUPPORTED;
     PairArgs p{};
@@ -545,6 +571,9 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
     p.window = sqrtf(40.0f) / bin_step;
     const int NT = K <= 16 ? 1 : K <= 32 ? 2 : 4;
     const bool uniform = cutoff == 0.0f;
+    const int side = 2 * lattice_range + 1;
+    if (rings && (!uniform || side * side * side > RIMG_CAP)) rings = nullptr;     // not what rings are staged for
+    p.rings = rings;
     const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)4 * NT * XPLANE + WPB * 16 +
                                         (size_t)WPB * NT * WAVE * 4) + 16;
     if (((U + WPB - 1) / WPB) * ((H + 7) / 8) >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // 32-bit round positions
@@ -552,8 +581,9 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
     const int blocks = real_enc_bwd_pairs_blocks(U, H);
 #define CF_BPAIR(NTV)                                                                              \
     do {                                                                                           \
-        if (uniform) real_enc_bwd_pair_kernel<NTV, true><<<blocks, WPB * WAVE, lds, st>>>(p);      \
-        else real_enc_bwd_pair_kernel<NTV, false><<<blocks, WPB * WAVE, lds, st>>>(p);             \
+        if (rings) real_enc_bwd_pair_kernel<NTV, true, true><<<blocks, WPB * WAVE, lds, st>>>(p);          \
+        else if (uniform) real_enc_bwd_pair_kernel<NTV, true, false><<<blocks, WPB * WAVE, lds, st>>>(p);  \
+        else real_enc_bwd_pair_kernel<NTV, false, false><<<blocks, WPB * WAVE, lds, st>>>(p);              \
     } while (0)
     switch (NT) {
         case 1: CF_BPAIR(1); break;

@@ -37,6 +37,7 @@ struct PairArgs {
     float bin_step, s_scale;
     float inv_bin_step;     // distance argument -> fractional bin coordinate
     float window;           // bins beyond which a Gaussian is below 2^-40 and is not evaluated
+    const float *rings;     // staged translations of every unit (RIMG_WORDS each), nullable
 };
 
 struct Cell {
@@ -224,5 +225,55 @@ __device__ __forceinline__ UnitGeom unit_geom(float gv, bool with_rvlen)
 // Bin handled by reduction step s (0..4*NT-1) and sub-lane kk (0..3) of the projection:
 // chosen so that a lane's 4 consecutive steps read 4 consecutive bins.
 __device__ __forceinline__ int proj_bin(int s, int kk) { return 16 * (s >> 2) + 4 * kk + (s & 3); }
+
+// ---- staged rings in memory ---------------------------------------------------
+// Image of a unit's staged translations (fixed cube of at most RIMG_CAP translations), RIMG_WORDS
+// 32-bit words: d2[RIMG_SLOTS], s[RIMG_SLOTS], bits[RIMG_SLOTS], header {near count, far count,
+// smallest d2, -}.  Near records occupy slots 0 .. near-1 followed by 8 neutral records
+// (d2 = +inf, no bits); far records occupy slots RIMG_SLOTS-1 downwards followed (below) by 4
+// neutral records.
+constexpr int RIMG_CAP = 128;
+constexpr int RIMG_SLOTS = RIMG_CAP + 16;
+constexpr int RIMG_WORDS = 3 * RIMG_SLOTS + 4;
+
+// slots lane and 64 + lane of the three arrays, and the header word min(lane, 3)
+struct RingImage { float d2[2], s[2]; int bits[2]; int hdr; };
+
+__device__ __forceinline__ RingImage load_ring_image(const float *__restrict__ rings, int64_t u, int lane)
+{
+    const float *base = rings + u * RIMG_WORDS;
+    RingImage im;
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        im.d2[k] = base[k * WAVE + lane];
+        im.s[k] = base[RIMG_SLOTS + k * WAVE + lane];
+        im.bits[k] = __float_as_int(base[2 * RIMG_SLOTS + k * WAVE + lane]);
+    }
+    im.hdr = __float_as_int(base[3 * RIMG_SLOTS + min(lane, 3)]);
+    return im;
+}
+
+__device__ __forceinline__ void store_ring_image(const RingImage &im, float *ring_d2, float *ring_s, int *ring_bits,
+                                                 int lane)
+{
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        ring_d2[k * WAVE + lane] = im.d2[k];
+        ring_s[k * WAVE + lane] = im.s[k];
+        ring_bits[k * WAVE + lane] = im.bits[k];
+    }
+}
+
+// slots 2*WAVE .. RIMG_SLOTS-1: the end of a full near block and the far block
+__device__ __forceinline__ void copy_ring_tail(const float *__restrict__ rings, int64_t u, float *ring_d2,
+                                               float *ring_s, int *ring_bits, int lane)
+{
+    if (lane < RIMG_SLOTS - 2 * WAVE) {
+        const float *base = rings + u * RIMG_WORDS;
+        ring_d2[2 * WAVE + lane] = base[2 * WAVE + lane];
+        ring_s[2 * WAVE + lane] = base[RIMG_SLOTS + 2 * WAVE + lane];
+        ring_bits[2 * WAVE + lane] = __float_as_int(base[2 * RIMG_SLOTS + 2 * WAVE + lane]);
+    }
+}
 
 }  // namespace cfpair

@@ -1,0 +1,498 @@
+// Real-space periodic encoding, forward, with the staged translations of every atom pair kept in
+// memory across the blocks of a model (fixed cube of at most 128 translations, shared projection).
+//
+// What the pair kernel of real_enc_mfma.hip stages per unit -- the translations that reach a bin,
+// ordered by the lowest 16-bin tile they reach, with their squared distance, Gaussian argument and
+// tile bits, the far ones that can still carry weight, and the smallest squared distance -- depends
+// on the geometry and on the bin grid only, not on the Gaussian exponents of a block.  All blocks of
+// a forward (and the backward passes) see the same crystals, so the staging is done once
+// (ring_stage_kernel, a wavefront per unit, image written to memory) and each block's launch
+// (real_enc_fwd_ring_kernel) starts from the stored image: no geometry, no classification, no
+// ranking, no lattice or position loads.  Accumulation, far block and projection are those of the
+// pair kernel.
+//
+// Ring image of a unit (RIMG_WORDS 32-bit words): d2[RS], s[RS], bits[RS], header {near count, far
+// count, smallest d2, -}.  Near records occupy slots 0 .. near-1 followed by 8 neutral records; far
+// records occupy slots RS-1 downwards followed (below) by 4 neutral records.  (Keeping d2 alone and
+// recomputing s and the bits in every launch makes the image three times smaller and the staging
+// faster, but costs each launch 5% more instructions: 46.4 against 43.8 us on 128 crystals.)
+#include "real_enc_pair.h"
+
+namespace {
+
+using namespace cf;
+using namespace cfpair;
+
+constexpr int RC = RIMG_CAP;                // translations of the cube, at most
+constexpr int RS = RIMG_SLOTS;              // ring slots
+
+// Gaussian argument s and record bits of a ring slot from its squared distance: 0xFFFF (a real
+// translation) plus one bit per 16-bin tile whose window the translation reaches; s = 0 and no
+// bits for a neutral slot (d2 = +inf).
+template <int NT>
+__device__ __forceinline__ int slot_record(const PairArgs &p, float d2, float &s)
+{
+    if (!(d2 < __builtin_inff())) {
+        s = 0.f;
+        return 0;
+    }
+    s = sqrt_hw(d2) * p.s_scale;
+    const float xb = s * p.inv_bin_step - 1.0f;          // fractional bin coordinate
+    int bits = 0xFFFF;
+#pragma unroll
+    for (int m = 0; m < NT; m++)
+        if (xb >= (float)(16 * m) - p.window && xb <= (float)(16 * m + 15) + p.window) bits |= (0x10000 << m);
+    return bits;
+}
+
+// ---------------------------------------------------------------- producer
+// A wavefront per unit and trip, lane = translation (two chunks of 64); the wavefronts of the grid
+// stride over the units, each with the next unit's lattice and offset already requested and the
+// pair record of the one after (the two dependent loads are off the critical path).  weak_a2 is
+// log2(e) times the weakest (closest to zero) exponent any block can have: a far translation is
+// kept when weak_a2 (d2 - d2min) > -40, a superset of what any block's own exponents keep.
+struct StageIds { int64_t e_ij, n; };
+
+template <int NT>
+__global__ __launch_bounds__(256) void ring_stage_kernel(PairArgs p, float weak_a2, float *__restrict__ cache)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t waves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    const int64_t first = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
+    if (first >= p.U) return;
+    auto ids_of = [&](int64_t u_) -> StageIds {
+        u_ = u_ < p.U ? u_ : p.U - 1;
+        return StageIds{p.pairs[u_ * PAIR_FIELDS], p.pairs[u_ * PAIR_FIELDS + 4]};
+    };
+    auto cell_of = [&](const StageIds &d) -> Cell {
+        Cell c_;
+        c_.rx = p.rpos[d.e_ij * 3 + 0];
+        c_.ry = p.rpos[d.e_ij * 3 + 1];
+        c_.rz = p.rpos[d.e_ij * 3 + 2];
+#pragma unroll
+        for (int x = 0; x < 9; x++) c_.t[x] = p.tvecs[d.n * 9 + x];
+        return c_;
+    };
+    Cell cell = cell_of(ids_of(first));
+    StageIds ids_next = ids_of(first + waves);
+    for (int64_t u = first; u < p.U; u += waves) {
+    const Cell cell_next = cell_of(ids_next);
+    ids_next = ids_of(u + 2 * waves);
+    BoxDims bx;
+    bx.U1 = bx.U2 = bx.U3 = p.lattice_range;
+    bx.S3 = bx.S2 = 2 * p.lattice_range + 1;
+    bx.plane = bx.S2 * bx.S3;
+    bx.T = bx.S2 * bx.plane;
+    bx.inv_plane = 1.0f / (float)bx.plane;
+    bx.inv_S3 = 1.0f / (float)bx.S3;
+    const int T = bx.T;                    // <= RC (checked by the host)
+    float d2c[2];
+    float best = 1e10f;
+#pragma unroll
+    for (int ch = 0; ch < 2; ch++) {
+        int n1, n2, n3;
+        decode(bx, min(ch * WAVE + lane, T - 1), n1, n2, n3);
+        d2c[ch] = dist2(cell, (float)n1, (float)n2, (float)n3);
+        if (ch * WAVE + lane < T) best = fminf(best, d2c[ch]);
+    }
+    const float d2min = wave_min(best);
+    float *ring_d2 = cache + u * RIMG_WORDS;
+    float *ring_s = ring_d2 + RS;
+    int *ring_bits = reinterpret_cast<int *>(ring_s + RS);
+    int near_cnt = 0, far_cnt = 0;
+#pragma unroll
+    for (int ch = 0; ch < 2; ch++) {
+        const bool valid = ch * WAVE + lane < T;
+        const float d2 = d2c[ch];
+        float s;
+        const int bits = valid ? slot_record<NT>(p, d2, s) : 0;
+        const int tiles = bits >> 16;
+        const bool is_near = valid && tiles != 0;
+        const bool is_far = valid && !is_near && weak_a2 * (d2 - d2min) > -40.0f;
+        const unsigned long long far_mask = __ballot(is_far);
+        const unsigned long long below = (1ull << lane) - 1ull;
+        int pos = -1;
+        int near_now;
+        if (NT > 1) {
+            // near translations ordered by the lowest tile they reach (8-bit counters per class)
+            const int key8 = tiles ? 8 * (__builtin_ctz(tiles) >> (NT > 4 ? 1 : 0)) : 0;
+            const int onehot = is_near ? (1 << key8) : 0;
+            const int incl = wave_inclusive_scan_i(onehot);
+            const int totals = __builtin_amdgcn_readlane(incl, 63);
+            const int before = (totals << 8) + (totals << 16) + (totals << 24);
+            if (is_near) pos = near_cnt + (((before + incl - onehot) >> key8) & 0xFF);
+            near_now = (int)(((unsigned)totals * 0x01010101u) >> 24);
+        } else {
+            const unsigned long long near_mask = __ballot(is_near);
+            if (is_near) pos = near_cnt + __popcll(near_mask & below);
+            near_now = __popcll(near_mask);
+        }
+        if (is_far) pos = RS - 1 - (far_cnt + __popcll(far_mask & below));
+        if (pos >= 0) {
+            ring_d2[pos] = d2;
+            ring_s[pos] = s;
+            ring_bits[pos] = bits;
+        }
+        near_cnt += near_now;
+        far_cnt += __popcll(far_mask);
+    }
+    // neutral records: 8 after the near block (last group + look-ahead), 4 below the far block
+    if (lane < 12) {
+        const int pos = lane < 8 ? near_cnt + lane : RS - far_cnt - 1 - (lane - 8);
+        ring_d2[pos] = __builtin_inff();
+        ring_s[pos] = 0.f;
+        ring_bits[pos] = 0;
+    }
+    if (lane == 0) {
+        int *hdr = reinterpret_cast<int *>(ring_d2 + 3 * RS);
+        hdr[0] = near_cnt;
+        hdr[1] = far_cnt;
+        reinterpret_cast<float *>(hdr)[2] = d2min;
+        hdr[3] = 0;
+    }
+    cell = cell_next;
+    }
+}
+
+// ---------------------------------------------------------------- consumer
+// Work-group of 8 wavefronts, one unit per wavefront and round, as in the pair kernel.  The image
+// of the next round's unit (its address follows from the round number alone) is requested a round
+// ahead into registers and copied to the wavefront's LDS ring at the top of its round.
+// LDS: per wave 3 x RS words, exchange buffer 4 NT x XPLANE, 8 x 2 edge ids, 8 x 16 reciprocals.
+template <int NT, int DT>
+__global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, const float *__restrict__ cache)
+{
+    extern __shared__ __align__(16) float lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane >> 4;
+    const int c = lane & 15;
+    const int H = p.H, K = p.K, D = p.D;
+    const int64_t *__restrict__ g_pairs = p.pairs;
+    const float *__restrict__ g_a = p.a_ik;
+    float *ring_d2 = lds + wave * (3 * RS);
+    float *ring_s = ring_d2 + RS;
+    int *ring_bits = reinterpret_cast<int *>(ring_s + RS);
+    float *Sbuf = lds + WPB * 3 * RS;                                       // [4 NT][XPLANE]
+    int64_t *meta = reinterpret_cast<int64_t *>(Sbuf + 4 * NT * XPLANE);    // [WPB][2]
+    float *invbuf = reinterpret_cast<float *>(meta + WPB * 2);              // [WPB][16]
+
+    float ck[NT];
+#pragma unroll
+    for (int m = 0; m < NT; m++) ck[m] = p.bin_step * (float)(16 * m + c + 1);
+    float Wa[DT][4 * NT];
+    int wa_hg = -1;
+
+    const int rounds_per_hg = (int)((p.U + WPB - 1) / WPB);
+    const int rounds = rounds_per_hg * p.head_groups;
+    const int stride = gridDim.x;
+    auto unit_of = [&](int rd_, const RoundPos &rp) -> int64_t {
+        const int64_t u_ = (int64_t)rp.r * WPB + wave;
+        return (rd_ < rounds && u_ < p.U) ? u_ : 0;
+    };
+    auto load_a = [&](const UnitIds &d, const RoundPos &rp) -> float {
+        const int h_ = min(rp.hg * 8 + (c & 7), H - 1);
+        return g_a[((c < 8) ? d.i : d.j) * H + h_];
+    };
+    using Image = RingImage;
+    auto load_image = [&](int64_t u_) -> Image { return load_ring_image(cache, u_, lane); };
+
+    RoundPos pos = round_pos(blockIdx.x, rounds_per_hg, p.head_groups);
+    RoundPos pos_next = round_pos(blockIdx.x + stride, rounds_per_hg, p.head_groups);
+    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x, pos), lane));
+    float a_cur = load_a(ids, pos);
+    Image img = load_image(unit_of(blockIdx.x, pos));
+    UnitIds ids_next = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x + stride, pos_next), lane));
+
+    for (int rd = blockIdx.x; rd < rounds; rd += stride) {
+        const int hg = pos.hg;
+        const int64_t u = (int64_t)pos.r * WPB + wave;
+        const bool unit_on = u < p.U;
+        const RoundPos pos_next2 = round_pos(rd + 2 * stride, rounds_per_hg, p.head_groups);
+        // this round's image into the ring (the previous round's readers of the ring are done:
+        // same wavefront, and the epilogue's barriers lie in between)
+        const int near_cnt = unit_on ? __builtin_amdgcn_readlane(img.hdr, 0) : 0;
+        const int far_cnt = unit_on ? __builtin_amdgcn_readlane(img.hdr, 1) : 0;
+        const float d2min = __int_as_float(__builtin_amdgcn_readlane(img.hdr, 2));
+        store_ring_image(img, ring_d2, ring_s, ring_bits, lane);
+        if (near_cnt + 8 > 2 * WAVE || far_cnt > 0)              // slots 128 .. 143 (wave-uniform, rare)
+            copy_ring_tail(cache, u, ring_d2, ring_s, ring_bits, lane);
+        if (!unit_on && lane < 8) {          // no unit: an empty near block (neutral records)
+            ring_d2[lane] = __builtin_inff();
+            ring_s[lane] = 0.f;
+            ring_bits[lane] = 0;
+        }
+        // loads for the coming rounds
+        const Image img_next = load_image(unit_of(rd + stride, pos_next));
+        const float a_next = load_a(ids_next, pos_next);
+        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane);
+        if (hg != wa_hg) {
+            const int hw = hg * 8 + wave;
+            if (hw < H && K == 16 * NT && D == 16 * DT) {
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++) {
+                    const float *wrow = p.W + ((int64_t)hw * D + 16 * dt + c) * K + 4 * q;
+#pragma unroll
+                    for (int t4 = 0; t4 < NT; t4++) {
+                        const float4_t w4 = *reinterpret_cast<const float4_t *>(wrow + 16 * t4);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) Wa[dt][4 * t4 + r] = w4[r];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int s = 0; s < 4 * NT; s++) {
+                        const int d = 16 * dt + c, k = proj_bin(s, q);
+                        Wa[dt][s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
+                    }
+            }
+            wa_hg = hg;
+        }
+        const int64_t e_ij = ids.e_ij, e_ji = ids.e_ji;
+        const int h = hg * 8 + (c & 7);
+        const bool col_on = unit_on && h < H && (c < 8 || e_ji != e_ij);
+        const float a = col_on ? a_cur : -1.0f;
+        const float a2 = a * LOG2E;
+
+        float4_t acc[NT];
+#pragma unroll
+        for (int m = 0; m < NT; m++) acc[m] = float4_t{0.f, 0.f, 0.f, 0.f};
+        float sum = 0.f;
+        wave_mem_sync();
+        // ---- accumulation over the near block: 4 translations per MFMA
+        {
+            const int groups = (near_cnt + 3) >> 2;
+            float d2n = ring_d2[q], sn = ring_s[q];
+            int bitsn = ring_bits[q];
+            for (int g = 0; g < groups; g++) {
+                const float d2t = d2n, st = sn;
+                const int bits = bitsn;
+                const int slot = 4 * (g + 1) + q;
+                d2n = ring_d2[slot];
+                sn = ring_s[slot];
+                bitsn = ring_bits[slot];
+                float w = exp2_hw(a2 * (d2t - d2min));
+                w = col_on ? w : 0.f;                   // (padding records carry d2 = +inf: weight 0)
+                sum += w;
+                const int reach = __builtin_amdgcn_readlane(bits, 0) | __builtin_amdgcn_readlane(bits, 16) |
+                                  __builtin_amdgcn_readlane(bits, 32) | __builtin_amdgcn_readlane(bits, 48);
+#pragma unroll
+                for (int m = 0; m < NT; m++) {
+                    if (reach & (0x10000 << m)) {                             // wave-uniform
+                        float b = ck[m] - st;
+                        float gm = exp2_hw(-(b * b));
+                        acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, w, acc[m], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        // ---- the far block only feeds the column sums
+        {
+            const int groups = (far_cnt + 3) >> 2;
+            for (int g = 0; g < groups; g++) {
+                const int slot = RS - 4 * (g + 1) + q;
+                const float d2t = ring_d2[slot];
+                const int bits = ring_bits[slot];
+                float w = exp2_hw(a2 * (d2t - d2min));
+                sum += (col_on && ((bits >> c) & 1)) ? w : 0.f;
+            }
+        }
+        wave_mem_sync();
+        const UnitIds ids_next2 = unit_ids(dv_next2);
+        sum += __shfl_xor(sum, 16, WAVE);
+        sum += __shfl_xor(sum, 32, WAVE);
+        const float inv = __builtin_amdgcn_rcpf(sum);
+        const int64_t e_col = (c < 8) ? e_ij : e_ji;
+        if (col_on && q == 0) p.z[e_col * H + h] = log2_hw(sum) * LN2 + d2min * a;
+
+        // epilogue: park the column sums, project per head (see the pair kernel)
+        float *col = Sbuf + xch_base(q, c & 7, wave, c >> 3);
+#pragma unroll
+        for (int m = 0; m < NT; m++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) col[(4 * m + r) * XPLANE] = acc[m][r];
+        if (q == 0) invbuf[wave * 16 + c] = inv;
+        if (lane == 0) {
+            meta[2 * wave + 0] = unit_on ? e_ij : -1;
+            meta[2 * wave + 1] = (unit_on && e_ji != e_ij) ? e_ji : -1;
+        }
+        __syncthreads();
+        {
+            const int hw = hg * 8 + wave;
+            const int j = c, unit_j = j & 7, dir_j = j >> 3;
+            const float *src = Sbuf + xch_base(q, wave, unit_j, dir_j);
+            float4_t out[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) out[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t4 = 0; t4 < NT; t4++) {
+                float sb[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) sb[r] = src[(4 * t4 + r) * XPLANE];
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int dt = 0; dt < DT; dt++)
+                        out[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(Wa[dt][4 * t4 + r], sb[r], out[dt], 0, 0, 0);
+            }
+            const int64_t e_out = meta[2 * unit_j + dir_j];
+            const float inv_j = invbuf[unit_j * 16 + dir_j * 8 + wave];
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) out[dt] *= inv_j;
+            if (e_out >= 0 && hw < H) {
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++) {
+                    const int dbase = 16 * dt + 4 * q;
+                    float *dst = p.v + (e_out * H + hw) * D + dbase;
+                    if (dbase + 3 < D) {
+                        *reinterpret_cast<float4_t *>(dst) = out[dt];
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 3; r++)
+                            if (dbase + r < D) dst[r] = out[dt][r];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        ids = ids_next;
+        a_cur = a_next;
+        img = img_next;
+        ids_next = ids_next2;
+        pos = pos_next;
+        pos_next = pos_next2;
+    }
+}
+
+}  // namespace
+
+namespace cf {
+
+int64_t real_enc_ring_words() { return RIMG_WORDS; }
+
+// Stages every unit's translations into `cache` (U x RIMG_WORDS floats).  Fixed cube of at most 128
+// translations, K in 1..128.  CF_ERR_UNSUPPORTED (no error text) otherwise.
+int launch_ring_stage(const float *rpos, const float *tvecs, const int64_t *pairs, int64_t U, int64_t K,
+                      float bin_step, float s_scale, int lattice_range, float weak_a, float *cache, hipStream_t st)
+{
+    const int64_t cube = (int64_t)(2 * lattice_range + 1) * (2 * lattice_range + 1) * (2 * lattice_range + 1);
+    if (K < 1 || K > 128 || cube > RC) return CF_ERR_UNSUPPORTED;
+    if (U == 0) return CF_OK;
+    PairArgs p{};
+    p.rpos = rpos; p.tvecs = tvecs; p.pairs = pairs; p.U = U; p.K = (int)K;
+    p.lattice_range = lattice_range;
+    p.bin_step = bin_step; p.s_scale = s_scale; p.inv_bin_step = 1.0f / bin_step;
+    p.window = sqrtf(40.0f) / bin_step;
+    const float weak_a2 = weak_a * LOG2E;
+    const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
+    int64_t blocks64 = (U + 3) / 4;
+    const int64_t cap = persistent_grid_cap(8);
+    if (blocks64 > cap) blocks64 = cap;
+    const int blocks = (int)blocks64;
+    switch (NT) {
+        case 1: ring_stage_kernel<1><<<blocks, 256, 0, st>>>(p, weak_a2, cache); break;
+        case 2: ring_stage_kernel<2><<<blocks, 256, 0, st>>>(p, weak_a2, cache); break;
+        case 4: ring_stage_kernel<4><<<blocks, 256, 0, st>>>(p, weak_a2, cache); break;
+        default: ring_stage_kernel<8><<<blocks, 256, 0, st>>>(p, weak_a2, cache); break;
+    }
+    return CF_OK;
+}
+
+// Forward from staged rings (shared projection, D <= 32).  CF_ERR_UNSUPPORTED otherwise.
+int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U, int64_t N, int64_t H, int64_t E,
+                              int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
+                              const float *cache, float *z, float *v, hipStream_t st)
+{
+    if (K < 1 || K > 128 || !W || D < 1 || D > 32) return CF_ERR_UNSUPPORTED;
+    PairArgs p{};
+    p.a_ik = a_ik; p.pairs = pairs; p.W = W; p.z = z; p.v = v;
+    p.N = N; p.E = E; p.U = U; p.W_num = 1;
+    p.H = (int)H; p.K = (int)K; p.D = (int)D;
+    p.head_groups = (int)((H + 7) / 8);
+    p.bin_step = bin_step; p.s_scale = s_scale; p.inv_bin_step = 1.0f / bin_step;
+    p.window = sqrtf(40.0f) / bin_step;
+    const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
+    const int DT = D > 16 ? 2 : 1;
+    size_t lds = sizeof(float) * ((size_t)WPB * 3 * RS + (size_t)4 * NT * XPLANE + WPB * 16) +
+                 sizeof(int64_t) * WPB * 2 + 8;
+    const int64_t rounds = ((U + WPB - 1) / WPB) * p.head_groups;
+    if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;
+    int64_t blocks = rounds;
+    const int64_t cap = persistent_grid_cap(2);
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) return CF_OK;
+#define CF_RING(NTV, DTV) real_enc_fwd_ring_kernel<NTV, DTV><<<(int)blocks, WPB * WAVE, lds, st>>>(p, cache)
+#define CF_RING_NT(NTV) do { if (DT == 1) CF_RING(NTV, 1); else CF_RING(NTV, 2); } while (0)
+    switch (NT) {
+        case 1: CF_RING_NT(1); break;
+        case 2: CF_RING_NT(2); break;
+        case 4: CF_RING_NT(4); break;
+        default: CF_RING_NT(8); break;
+    }
+#undef CF_RING_NT
+#undef CF_RING
+    return CF_OK;
+}
+
+}  // namespace cf
+
+namespace {
+// Gaussian argument per bin index and per unit of distance, as the other encoding entry points derive them
+void bin_scales(int64_t K, double dist_max, double wscale, float &bin_step, float &s_scale)
+{
+    const float reci_ws_sqrt2 = 1.0f / ((float)wscale * sqrtf(2.0f));
+    const float mu0 = (float)dist_max / (float)K;
+    bin_step = reci_ws_sqrt2 * sqrtf(cf::LOG2E);
+    s_scale = bin_step / mu0;
+}
+}  // namespace
+
+extern "C" int64_t cf_real_enc_ring_bytes(int64_t U) { return (U < 0 ? 0 : U) * RIMG_WORDS * (int64_t)sizeof(float); }
+
+extern "C" int cf_real_enc_ring_stage(const float *rpos_ij_e, const float *tvecs_n, const int64_t *pairs_u, int64_t U,
+                                      int64_t K, double dist_max, double wscale, int lattice_range,
+                                      double weakest_exponent, void *rings, void *stream)
+{
+    CF_REQUIRE(U >= 0, CF_ERR_INVALID_ARGUMENT, "cf_real_enc_ring_stage: negative U");
+    if (U == 0) return CF_OK;
+    CF_REQUIRE(rpos_ij_e && tvecs_n && pairs_u && rings, CF_ERR_INVALID_ARGUMENT, "cf_real_enc_ring_stage: null pointer");
+    CF_REQUIRE(K >= 1 && K <= 128 && dist_max > 0 && wscale > 0, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_ring_stage: needs 1 <= K <= 128 and positive dist_max, wscale");
+    CF_REQUIRE(weakest_exponent <= 0, CF_ERR_INVALID_ARGUMENT, "cf_real_enc_ring_stage: weakest_exponent must be <= 0");
+    CF_REQUIRE(lattice_range >= 0 && (2 * lattice_range + 1) * (2 * lattice_range + 1) * (2 * lattice_range + 1) <= RC,
+               CF_ERR_UNSUPPORTED, "cf_real_enc_ring_stage: the fixed cube of lattice_range %d has more than %d translations",
+               lattice_range, RC);
+    float bin_step, s_scale;
+    bin_scales(K, dist_max, wscale, bin_step, s_scale);
+    int rc = cf::launch_ring_stage(rpos_ij_e, tvecs_n, pairs_u, U, K, bin_step, s_scale, lattice_range,
+                                   (float)weakest_exponent, (float *)rings, (hipStream_t)stream);
+    CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_ring_stage: unsupported shape");
+    CF_CHECK_LAUNCH("cf_real_enc_ring_stage");
+    return CF_OK;
+}
+
+extern "C" int cf_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs_u, int64_t U, int64_t N, int64_t H,
+                                     int64_t E, int64_t K, int64_t D, double dist_max, double wscale,
+                                     const float *W_k, const void *rings, float *z_ek, float *v_ekd, void *stream)
+{
+    CF_REQUIRE(N >= 0 && E >= 0 && U >= 0, CF_ERR_INVALID_ARGUMENT, "cf_real_enc_fwd_rings: negative size");
+    CF_REQUIRE(H == 1 || H == 2 || H == 4 || H == 8 || H == 16, CF_ERR_UNSUPPORTED,
+               "cf_real_enc_fwd_rings: head count %lld not supported (1,2,4,8,16)", (long long)H);
+    CF_REQUIRE(2 * U == E + N, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_fwd_rings: a pair list over dense crystal blocks has (E+N)/2 = %lld entries, got %lld",
+               (long long)((E + N) / 2), (long long)U);
+    if (E == 0) return CF_OK;
+    CF_REQUIRE(a_ik && pairs_u && W_k && rings && z_ek && v_ekd, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_fwd_rings: null pointer");
+    CF_REQUIRE(K >= 1 && K <= 128 && D >= 1 && D <= 32 && dist_max > 0 && wscale > 0, CF_ERR_UNSUPPORTED,
+               "cf_real_enc_fwd_rings: needs 1 <= K <= 128, 1 <= D <= 32");
+    float bin_step, s_scale;
+    bin_scales(K, dist_max, wscale, bin_step, s_scale);
+    int rc = cf::launch_real_enc_fwd_rings(a_ik, pairs_u, U, N, H, E, K, D, bin_step, s_scale, W_k,
+                                           (const float *)rings, z_ek, v_ekd, (hipStream_t)stream);
+    CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported shape");
+    CF_CHECK_LAUNCH("cf_real_enc_fwd_rings");
+    return CF_OK;
+}

@@ -77,6 +77,12 @@ class KernelManager:
     # whose work-group per atom is bound by its chain of dependent loads), eager launches gain
     # from the launch saved (0.55 against 0.78 ms), so capture keeps the two operators.
     FUSE_ENCODING_ATTENTION_IN_GRAPHS: bool = False
+    # Fixed cube: the geometry-only part of the encoding (which translations reach a bin, in which
+    # order, their distances) is staged once per forward pass and shared by all blocks
+    # (ops.staged_rings).  Needs an upper bound of the exponents the rings will meet, which the
+    # attention module sets around its call (-gauss_lb / (2 r0^2)); None: every launch stages for itself.
+    STAGED_RINGS: bool = True
+    WEAKEST_EXPONENT: Optional[float] = None
     compiled: bool = False
 
 
@@ -152,14 +158,25 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         batch_i = batch_i.contiguous()
         edge_ij_e = edge_ij_e.contiguous()
         W_k = W_k.detach().contiguous() if W_k is not None else None
-        z_ek, v_ekd = ops.real_enc_fwd(
-            a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, W_k, rvlen_n,
-            cutoff_radius, KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE,
-            pairs_u=_pairs(batch_i, edge_ij_e, tvecs_n, K))
+        pairs_u = _pairs(batch_i, edge_ij_e, tvecs_n, K)
+        rings = None
+        fixed_cube = rvlen_n is None or cutoff_radius is None or float(cutoff_radius) == 0.0
+        if (KernelManager.STAGED_RINGS and KernelManager.WEAKEST_EXPONENT is not None and pairs_u is not None
+                and fixed_cube and K > 0 and W_k is not None and _w_leading(W_k) == 1 and W_k.shape[-2] <= 32):
+            rings = ops.staged_rings(rpos_ij_e, tvecs_n, pairs_u, K, dist_max, wscale, KernelManager.LATTICE_RANGE,
+                                     KernelManager.WEAKEST_EXPONENT)
+        if rings is not None:
+            z_ek, v_ekd = ops.real_enc_fwd_rings(a_ik, edge_ij_e, pairs_u, rings, K, dist_max, wscale, W_k)
+        else:
+            z_ek, v_ekd = ops.real_enc_fwd(
+                a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, W_k, rvlen_n,
+                cutoff_radius, KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE, pairs_u=pairs_u)
         ctx.save_for_backward(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, W_k, z_ek)
         ctx.K, ctx.dist_max, ctx.wscale, ctx.cutoff_radius = K, dist_max, wscale, cutoff_radius
         ctx.ranges = (KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
         ctx.adaptive_args = rvlen_n is not None
+        # the backward's pair kernel (K <= 64, D <= 16) starts from the same staged translations
+        ctx.rings = rings if (rings is not None and K <= 64 and W_k.shape[-2] <= 16) else None
         if K <= 0:
             return (z_ek,)
         return z_ek, v_ekd
@@ -174,7 +191,7 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
             a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz, gv, ctx.K, ctx.dist_max,
             ctx.wscale, W_k, rvlen_n, ctx.cutoff_radius, ctx.ranges[0], ctx.ranges[1],
             want_gW=W_k is not None and ctx.needs_input_grad[9],
-            pairs_u=_pairs(batch_i, edge_ij_e, tvecs_n, ctx.K))
+            pairs_u=_pairs(batch_i, edge_ij_e, tvecs_n, ctx.K), rings=ctx.rings)
         return _enc_backward_tail(ga_ik, gW_k, ctx.adaptive_args)
 
 

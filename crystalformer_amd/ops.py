@@ -232,14 +232,87 @@ def real_enc_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
     return z, v
 
 
+# Staged translation rings of the latest geometries (see staged_rings): large buffers, so only a
+# couple are kept, and only while the tensors they were built from are alive and unmodified.
+_ring_cache: list = []
+_RING_CACHE_SIZE = 2
+STAGED_RINGS_MAX_BYTES = 1 << 30     # 1744 bytes per atom pair: beyond this the blocks stage for themselves
+
+
+def staged_rings(rpos_ij_e: Tensor, tvecs_n: Tensor, pairs_u: Tensor, K: int, dist_max: float, wscale: float,
+                 lattice_range: int, weakest_exponent: float) -> Optional[Tensor]:
+    """Per-unit staged translations for :func:`real_enc_fwd_rings` (fixed cube of at most 128
+    translations), built once per geometry and bin grid: the blocks of a forward pass hand in the
+    same ``rpos_ij_e`` / ``tvecs_n`` / ``pairs_u`` tensors and share one buffer.  ``None`` when the
+    cube is too large for the staged kernels."""
+    if (2 * int(lattice_range) + 1) ** 3 > 128 or K < 1 or K > 128:
+        return None
+    # (a launch recorded into a graph and an eager one never share a buffer: a replay stages again)
+    dev = require_device(rpos_ij_e, tvecs_n, pairs_u)
+    sig = tuple((t.data_ptr(), tuple(t.shape), t._version) for t in (rpos_ij_e, tvecs_n, pairs_u)) + \
+        (bool(torch.cuda.is_current_stream_capturing()), int(K), float(dist_max), float(wscale),
+         int(lattice_range), float(weakest_exponent))
+    for entry in _ring_cache:
+        if entry[0] == sig:
+            return entry[2]
+    L = _lib.load()
+    U = pairs_u.shape[0]
+    if int(L.cf_real_enc_ring_bytes(U)) > STAGED_RINGS_MAX_BYTES:
+        return None
+    rings = torch.empty(max(int(L.cf_real_enc_ring_bytes(U)) // 4, 1), dtype=torch.float32, device=dev)
+    with device_guard(dev), _timed("real_enc_ring_stage", U=U, K=K):
+        rc = L.cf_real_enc_ring_stage(ptr(rpos_ij_e), ptr(tvecs_n), ptr(pairs_u), U, int(K), float(dist_max),
+                                      float(wscale), int(lattice_range), float(weakest_exponent), ptr(rings),
+                                      stream_handle(dev))
+    check(rc, "cf_real_enc_ring_stage")
+    _ring_cache.insert(0, (sig, (rpos_ij_e, tvecs_n, pairs_u), rings))
+    del _ring_cache[_RING_CACHE_SIZE:]
+    return rings
+
+
+def real_enc_fwd_rings(a_ik: Tensor, edge_ij_e: Tensor, pairs_u: Tensor, rings: Tensor, K: int, dist_max: float,
+                       wscale: float, W_k: Tensor) -> Tuple[Tensor, Tensor]:
+    """:func:`real_enc_fwd` for a shared projection and the fixed cube, from the staged rings."""
+    dev = require_device(a_ik, edge_ij_e, pairs_u, rings, W_k)
+    a_ik, W_k = _f32(a_ik, "a_ik"), _f32(W_k, "W_k")
+    pairs_u = _i64(pairs_u, "pairs_u")
+    N, H = a_ik.shape
+    E = edge_ij_e.shape[1]
+    W_num, D = _w_shape(W_k, H, int(K))
+    if W_num != 1:
+        raise _lib.CrystalformerHipError("real_enc_fwd_rings: one projection per head only")
+    if rings.dtype != torch.float32 or rings.numel() * 4 < int(_lib.load().cf_real_enc_ring_bytes(pairs_u.shape[0])):
+        raise _lib.CrystalformerHipError("real_enc_fwd_rings: rings buffer too small for this pair list")
+    z = torch.empty((E, H), dtype=torch.float32, device=dev)
+    v = torch.empty((E, H, D), dtype=torch.float32, device=dev)
+    if _eval_counter is not None:
+        _eval_counter.append(float(E) * (2 * _ring_lattice_range(rings, pairs_u) + 1) ** 3)
+    with device_guard(dev), _timed("real_enc_fwd", E=E, H=H, K=K, D=D, proj=True):
+        rc = _lib.load().cf_real_enc_fwd_rings(ptr(a_ik), ptr(pairs_u), pairs_u.shape[0], N, H, E, int(K), D,
+                                               float(dist_max), float(wscale), ptr(W_k), ptr(rings), ptr(z), ptr(v),
+                                               stream_handle(dev))
+    check(rc, "cf_real_enc_fwd_rings")
+    return z, v
+
+
+def _ring_lattice_range(rings: Tensor, pairs_u: Tensor) -> int:
+    for entry in _ring_cache:
+        if entry[2] is rings:
+            return entry[0][-2]
+    return 2
+
+
 def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor,
                  e_start_i: Tensor, z_ek: Tensor, gz_ek: Optional[Tensor], gv_ekd: Optional[Tensor],
                  K: int, dist_max: float, wscale: float, W_k: Optional[Tensor] = None,
                  rvlen_n: Optional[Tensor] = None, cutoff_radius: Optional[float] = None,
                  lattice_range: int = 2, minimum_range: int = 0,
-                 want_gW: bool = True, pairs_u: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
+                 want_gW: bool = True, pairs_u: Optional[Tensor] = None,
+                 rings: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
+    """``rings`` from :func:`staged_rings` (same geometry, pair list, bin grid and cube): the pair
+    kernel starts from the staged translations instead of working them out again."""
     dev = require_device(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd,
-                         W_k, rvlen_n, pairs_u)
+                         W_k, rvlen_n, pairs_u, rings)
     pairs_u = _i64(pairs_u, "pairs_u")
     a_ik, rpos_ij_e, tvecs_n = _f32(a_ik, "a_ik"), _f32(rpos_ij_e, "rpos_ij_e"), _f32(tvecs_n, "tvecs_n")
     batch_i, edge_ij_e, e_start_i = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e"), \
@@ -266,6 +339,20 @@ def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
     L = _lib.load()
     ws_bytes = int(L.cf_real_enc_bwd_workspace(N, H, E, K, D, W_num, 1 if want_gW else 0))
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    if rings is not None:
+        if pairs_u is None or W_k is None or W_num != 1 or cutoff != 0.0:
+            raise _lib.CrystalformerHipError("real_enc_bwd: staged rings need the pair list, one projection per "
+                                             "head and the fixed cube")
+        if rings.dtype != torch.float32 or rings.numel() * 4 < int(L.cf_real_enc_ring_bytes(pairs_u.shape[0])):
+            raise _lib.CrystalformerHipError("real_enc_bwd: rings buffer too small for this pair list")
+        with device_guard(dev), _timed("real_enc_bwd", E=E, H=H, K=K, D=D, proj=True):
+            rc = L.cf_real_enc_bwd_rings(
+                ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i),
+                ptr(z_ek), ptr(gz_ek), ptr(gv_ekd), N, H, E, B, K, D, float(dist_max), float(wscale), ptr(W_k),
+                int(lattice_range), ptr(pairs_u), pairs_u.shape[0], ptr(rings), ptr(ws), ws_bytes,
+                ptr(ga), ptr(gW), stream_handle(dev))
+        check(rc, "cf_real_enc_bwd_rings")
+        return ga, gW
     with device_guard(dev), _timed("real_enc_bwd", E=E, H=H, K=K, D=D, proj=W_k is not None):
         rc = L.cf_real_enc_bwd(
             ptr(a_ik), ptr(rpos_ij_e), ptr(tvecs_n), ptr(batch_i), ptr(edge_ij_e), ptr(e_start_i),

@@ -100,6 +100,45 @@ int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvec
                     float *z_ek, float *v_ekd, void *stream);
 
 /*
+ * Staged translations kept across the blocks of a model (fixed cube, cutoff_radius = 0, of at
+ * most 128 translations; K >= 1).  No counterpart in the reference, whose kernels redo the
+ * geometry of every (edge, head, translation) in every block
+ * (models/kernels/real_enc_proj_fwd.cu:94-131).
+ *
+ * What cf_real_enc_fwd stages per unit of pairs_u -- which translations reach a Gaussian bin, in
+ * which order they are accumulated, their squared distance and Gaussian argument, the smallest
+ * squared distance -- depends on rpos_ij_e, tvecs_n and the bin grid (K, dist_max, wscale) only,
+ * not on a_ik.  cf_real_enc_ring_stage writes it once for all units into `rings`
+ * (cf_real_enc_ring_bytes(U) bytes of device memory, 256-byte aligned); cf_real_enc_fwd_rings is
+ * cf_real_enc_fwd (shared W_k of shape (H,D,K), D <= 32, pair list) starting from it.  The rings
+ * stay valid while the positions, the lattices, the pair list and the bin grid do.
+ *   weakest_exponent  upper bound (<= 0) of every a_ik the rings will be used with, e.g.
+ *                     -gauss_lb / (2 r0^2): translations that reach no bin are kept only if
+ *                     exp(weakest_exponent (d^2 - d^2_min)) > 2^-40.  Exponents above the bound
+ *                     make the lattice sums drop terms they should hold; 0 keeps every translation.
+ */
+int64_t cf_real_enc_ring_bytes(int64_t U);
+int cf_real_enc_ring_stage(const float *rpos_ij_e, const float *tvecs_n, const int64_t *pairs_u, int64_t U,
+                           int64_t K, double dist_max, double wscale, int lattice_range,
+                           double weakest_exponent, void *rings, void *stream);
+int cf_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs_u, int64_t U, int64_t N, int64_t H,
+                          int64_t E, int64_t K, int64_t D, double dist_max, double wscale,
+                          const float *W_k, const void *rings, float *z_ek, float *v_ekd, void *stream);
+/*
+ * cf_real_enc_bwd (below; same arguments, workspace and results) for the fixed cube and one
+ * projection per head, with the rings staged for this geometry, pair list, bin grid and
+ * lattice_range: its pair kernel (K <= 64, D <= 16, gv_ekd given) starts from them; other shapes
+ * run the kernels cf_real_enc_bwd runs, which do not read the rings.
+ */
+int cf_real_enc_bwd_rings(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                          const int64_t *batch_i, const int64_t *edge_ij_e, const int64_t *e_start_i,
+                          const float *z_ek, const float *gz_ek, const float *gv_ekd,
+                          int64_t N, int64_t H, int64_t E, int64_t B, int64_t K, int64_t D,
+                          double dist_max, double wscale, const float *W_k, int lattice_range,
+                          const int64_t *pairs_u, int64_t U, const float *rings, void *workspace,
+                          int64_t workspace_bytes, float *ga_ik, float *gW_k, void *stream);
+
+/*
  * Bytes of device scratch cf_real_enc_bwd needs for the given sizes
  * (pass want_gW != 0 when gW_k will be requested).
  */

@@ -1174,3 +1174,106 @@ def test_fused_encoding_attention_limits(dev):
     hip_funcs.compile_kernels(2, 8, 16, 0, 16, False)
     got = hip_funcs.fused_encoding_attention(a, *args[1:5], *args[6:9])
     assert got is not None and not got.requires_grad
+
+
+# ---- staged rings: the translations of every atom pair staged once, all blocks start from them
+
+def _staged(dev, p, K, lr, weakest=None):
+    rpos, tv = to_dev(dev, p.rpos, p.b.trans_vec)
+    pairs = ops.edge_pairs(p.b.sizes.to(dev))
+    weakest = float(p.a.max()) if weakest is None else weakest
+    return rpos, tv, pairs, ops.staged_rings(rpos, tv, pairs, K, p.dist_max, p.wscale, lr, weakest)
+
+
+@pytest.mark.parametrize("lr", [2, 1])
+@pytest.mark.parametrize("H,K,D", [(8, 64, 16), (4, 16, 8), (1, 7, 3), (2, 100, 4), (16, 32, 8), (8, 64, 32),
+                                   (8, 48, 20), (16, 128, 16)])
+def test_real_enc_fwd_from_staged_rings(dev, H, K, D, lr):
+    p = Problem([1, 3, 9, 2, 17, 1], H=H, K=K, D=D, seed=28)
+    z_ref, v_ref = enc_fwd_ref(p, K, p.W, 0.0, lr, 0)
+    rpos, tv, pairs, rings = _staged(dev, p, K, lr)
+    assert rings is not None and rings.numel() * 4 == lib.load().cf_real_enc_ring_bytes(pairs.shape[0])
+    a, ed, W = to_dev(dev, p.a, p.edges, p.W)
+    z, v = ops.real_enc_fwd_rings(a, ed, pairs, rings, K, p.dist_max, p.wscale, W)
+    assert_close(z, z_ref, "z")
+    assert_close(v, v_ref, "v", atol=v_atol(p, K, p.W, 0.0, lr, 0))
+    # the same geometry again: the staged buffer is found, not rebuilt
+    assert ops.staged_rings(rpos, tv, pairs, K, p.dist_max, p.wscale, lr, float(p.a.max())) is rings
+    # a weaker bound on the exponents keeps more far translations: same result to the last bits
+    _, _, _, rings0 = _staged(dev, p, K, lr, weakest=0.0)
+    z0, v0 = ops.real_enc_fwd_rings(a, ed, pairs, rings0, K, p.dist_max, p.wscale, W)
+    assert rel_err(z0, z) < 1e-6 and rel_err(v0, v) < 1e-6
+
+
+def test_staged_rings_serve_blocks_with_different_exponents(dev):
+    """One staging, several exponent sets (the blocks of a model): each equals the pair kernel's result for its
+    own exponents, on the pair kernel's own bits where no far translation is kept."""
+    p = Problem([5, 11, 2, 30, 1], H=8, K=64, D=16, seed=33)
+    exps = [p.a, p.a * 0.5, p.a * 3.0]
+    rpos, tv, pairs, rings = _staged(dev, p, 64, 2, weakest=float(max(e.max() for e in exps)))
+    bt, ed, W = to_dev(dev, p.b.batch, p.edges, p.W)
+    for a_cpu in exps:
+        a = a_cpu.to(dev)
+        z0, v0 = ops.real_enc_fwd(a, rpos, tv, bt, ed, 64, p.dist_max, p.wscale, W, None, 0.0, 2, 0, pairs_u=pairs)
+        z1, v1 = ops.real_enc_fwd_rings(a, ed, pairs, rings, 64, p.dist_max, p.wscale, W)
+        assert rel_err(z1, z0) < 1e-6 and rel_err(v1, v0) < 1e-6
+        p.a = a_cpu
+        z_ref, v_ref = enc_fwd_ref(p, 64, p.W, 0.0, 2, 0)
+        assert_close(z1, z_ref, "z")
+        assert_close(v1, v_ref, "v", atol=v_atol(p, 64, p.W, 0.0, 2, 0))
+
+
+@pytest.mark.parametrize("lr", [2, 1])
+@pytest.mark.parametrize("H,K,D", [(8, 64, 16), (4, 16, 8), (16, 32, 16), (1, 7, 12)])
+def test_real_enc_bwd_from_staged_rings(dev, H, K, D, lr):
+    p = Problem([1, 3, 9, 2, 14, 1, 1, 1, 1, 20], H=H, K=K, D=D, seed=30)
+    z_ref, v_ref = enc_fwd_ref(p, K, p.W, 0.0, lr, 0)
+    gz, gv = p.randn(p.E, H), p.randn(*v_ref.shape)
+    args = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv)
+    _, _, pairs, rings = _staged(dev, p, K, lr)
+    ga, gW = ops.real_enc_bwd(*args, K, p.dist_max, p.wscale, p.W.to(dev), None, 0.0, lr, 0, pairs_u=pairs,
+                              rings=rings)
+    ga_ref, gW_ref = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv, K,
+                                     p.dist_max, p.wscale, p.W, p.rvlen, 0.0, lr, 0)
+    ga_atol, gW_atol = enc_bwd_atols(p, z_ref, gz, gv, K, p.W, 0.0, lr, 0)
+    assert_close(ga, ga_ref, "ga", atol=ga_atol)
+    assert_close(gW, gW_ref, "gW", atol=gW_atol)
+    ga2, none = ops.real_enc_bwd(*args, K, p.dist_max, p.wscale, p.W.to(dev), None, 0.0, lr, 0, want_gW=False,
+                                 pairs_u=pairs, rings=rings)
+    assert none is None and torch.equal(ga2, ga)
+    # only the value gradient, only the bias gradient
+    for gz_, gv_ in ((None, args[8]), (args[7], None)):
+        ga3, _ = ops.real_enc_bwd(*args[:7], gz_, gv_, K, p.dist_max, p.wscale, p.W.to(dev), None, 0.0, lr, 0,
+                                  want_gW=False, pairs_u=pairs, rings=rings)
+        ga4, _ = ops.real_enc_bwd(*args[:7], gz_, gv_, K, p.dist_max, p.wscale, p.W.to(dev), None, 0.0, lr, 0,
+                                  want_gW=False, pairs_u=pairs)
+        assert rel_err(ga3, ga4) < 1e-6
+
+
+def test_staged_rings_limits(dev):
+    p = Problem([3, 4], H=8, K=64, D=16, seed=34)
+    assert _staged(dev, p, 64, 3)[3] is None                     # 343 translations: beyond the staged kernels
+    assert _staged(dev, p, 0, 2)[3] is None                      # no value bins: nothing to stage for
+    rpos, tv, pairs, rings = _staged(dev, p, 64, 2)
+    a, ed, W = to_dev(dev, p.a, p.edges, p.W)
+    with pytest.raises(lib.CrystalformerHipError, match="too small"):
+        ops.real_enc_fwd_rings(a, ed, pairs, rings[:100], 64, p.dist_max, p.wscale, W)
+    big = torch.zeros(8, 64, 64, device=dev)                     # D = 64: no staged kernel
+    with pytest.raises(lib.CrystalformerHipError):
+        ops.real_enc_fwd_rings(a, ed, pairs, rings, 64, p.dist_max, p.wscale, big)
+    old = ops.STAGED_RINGS_MAX_BYTES
+    ops.STAGED_RINGS_MAX_BYTES = 1000
+    try:
+        ops._ring_cache.clear()
+        assert _staged(dev, p, 64, 2)[3] is None                 # too large to keep: blocks stage for themselves
+    finally:
+        ops.STAGED_RINGS_MAX_BYTES = old
+    # backward: shapes its pair kernel does not take go to the other kernels, rings or not
+    rpos, tv, pairs, rings = _staged(dev, p, 64, 2)
+    z, v = ops.real_enc_fwd_rings(a, ed, pairs, rings, 64, p.dist_max, p.wscale, W)
+    args = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start) + [z, torch.ones_like(z)]
+    W32 = p.randn(8, 32, 64).to(dev)
+    gv32 = p.randn(p.E, 8, 32).to(dev)
+    with_rings = ops.real_enc_bwd(*args, gv32, 64, p.dist_max, p.wscale, W32, None, 0.0, 2, 0, pairs_u=pairs, rings=rings)
+    without = ops.real_enc_bwd(*args, gv32, 64, p.dist_max, p.wscale, W32, None, 0.0, 2, 0, pairs_u=pairs)
+    assert torch.equal(with_rings[0], without[0]) and torch.equal(with_rings[1], without[1])

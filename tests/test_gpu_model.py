@@ -12,7 +12,7 @@ import torch
 
 from crystalformer_amd import global_config, hip_funcs, ops
 from crystalformer_amd.latticeformer import Latticeformer, default_params
-from crystalformer_amd.synthetic import CONFIGS, make_config_batch
+from crystalformer_amd.synthetic import CONFIGS, make_config_batch, select_crystals
 from oracle import kernel_semantics as ks
 from oracle import torch_model as om
 from oracle import torch_path as tp
@@ -695,3 +695,56 @@ def test_other_normalisations_and_dropout_take_the_torch_loop(dev):
     assert_close(y_scaled - attn.out_proj.bias, (y_plain - attn.out_proj.bias) * attn.atten_scale[0], "scaled output",
                  rtol=1e-4)
     attn.params.norm_func_mode = 0
+
+
+def test_blocks_share_one_staging_of_the_translations(dev):
+    """Fixed cube, value bins, shared projection: the translations of every atom pair are staged once per
+    forward pass and all blocks (and their backward passes) start from them.  Same outputs and gradients as
+    with every block staging for itself; one staging launch per pass; graph replays follow new geometry."""
+    from crystalformer_amd.graphs import GraphedForward
+    name = "cfg2_default_b128"
+    b = select_crystals(make_config_batch(name), range(24)).to(dev)
+    cfg, model = build_model(name, adaptive_cutoff_sigma=0.0)
+    model.to(dev).train()
+
+    def step(staged):
+        hip_funcs.KernelManager.STAGED_RINGS = staged
+        try:
+            model.zero_grad(set_to_none=True)
+            log = []
+            ops.set_event_log(log)
+            y = model(b)
+            y.square().sum().backward()
+            ops.set_event_log(None)
+            names = [entry[0] for entry in log]
+            return y.detach().clone(), {k: p.grad.clone() for k, p in model.named_parameters()
+                                        if p.grad is not None}, names
+        finally:
+            hip_funcs.KernelManager.STAGED_RINGS = True
+            ops.set_event_log(None)
+    model(b)                                   # first training pass: stores the batch statistics
+    y1, g1, names1 = step(True)
+    y0, g0, names0 = step(False)
+    layers = len(model.encoder.layers)
+    assert names1.count("real_enc_ring_stage") == 1 and names0.count("real_enc_ring_stage") == 0
+    assert names1.count("real_enc_fwd") == layers and names1.count("real_enc_bwd") == layers
+    assert rel_err(y1, y0) < 1e-6
+    assert set(g1) == set(g0)
+    for k in g1:
+        assert rel_err(g1[k], g0[k]) < 1e-5, k
+    # replays of a captured forward stage again: they follow the geometry of the batch handed in
+    model.eval()
+    with torch.no_grad():
+        y_eager = model(b).clone()
+    graphed = GraphedForward(model, b)
+    b2 = select_crystals(make_config_batch(name), range(24)).to(dev)
+    b2.pos.mul_(1.05)
+    b2.trans_vec.mul_(1.05)
+    with torch.no_grad():
+        y2 = model(b2).clone()
+    assert float((y2 - y_eager).abs().max()) > 1e-6
+    for _ in range(2):
+        assert torch.equal(graphed(b2), y2)
+        torch.cuda.synchronize()
+        assert torch.equal(graphed(b), y_eager)
+        torch.cuda.synchronize()
