@@ -32,7 +32,7 @@ PEAK_FP32_TFLOPS = 157.3          # fp32 on the matrix cores (and packed vector 
 PEAK_FP32_VALU_TFLOPS = 78.6      # one fp32 FMA per lane and cycle: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz x 2
 PEAK_HBM_GBS = 8000.0
 PROFILE_FILE = os.path.join(ROOT, "profiles", "traffic.json")
-KERNEL_SOURCES = {"fwd": ("real_enc_mfma.hip", "real_enc_pair.h", "cf_common.h"),
+KERNEL_SOURCES = {"fwd": ("real_enc_ring.hip", "real_enc_mfma.hip", "real_enc_pair.h", "cf_common.h"),
                   "bwd": ("real_enc_mfma_bwd.hip", "real_enc_pair.h", "cf_common.h")}
 
 
@@ -412,7 +412,9 @@ def main() -> int:
     if args.ingest_counters:
         cfg_name = "cfg4_train_b128" if (args.train and args.config == "cfg2_default_b128") else args.config
         key = args.ingest_key or f"{cfg_name}:{args.rule}:{'bwd' if args.train else 'fwd'}"
-        kernel = args.ingest_kernel or ("real_enc_bwd_pair_kernel" if args.train else "real_enc_fwd_pair_kernel")
+        staged = args.rule == "A" and not args.no_staged_rings     # forward: from the staged rings (fixed cube)
+        kernel = args.ingest_kernel or ("real_enc_bwd_pair_kernel" if args.train else
+                                        "real_enc_fwd_ring_kernel" if staged else "real_enc_fwd_pair_kernel")
         return ingest_counters(args.ingest_counters, key, kernel)
 
     if args.gpus != 1:
@@ -474,13 +476,17 @@ def main() -> int:
         src = torch.ones(64 << 20, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
         captured = {}
-        which = "real_enc_bwd" if args.train else "real_enc_fwd"       # --train: the backward kernel
-        orig = getattr(ops, which)
+        # --train: the backward kernel; otherwise the forward one, pair kernel or from staged rings
+        names = ("real_enc_bwd",) if args.train else ("real_enc_fwd", "real_enc_fwd_rings", "staged_rings")
+        originals = {nm: getattr(ops, nm) for nm in names}
 
-        def spy(*a, **kw):
-            captured.setdefault("args", (a, kw))
-            return orig(*a, **kw)
-        setattr(ops, which, spy)
+        def spy_on(nm):
+            def spy(*a, **kw):
+                captured.setdefault(nm, (a, kw))
+                return originals[nm](*a, **kw)
+            return spy
+        for nm in names:
+            setattr(ops, nm, spy_on(nm))
         if args.train:
             model.train()
             out = model(data)
@@ -488,12 +494,15 @@ def main() -> int:
         else:
             with torch.no_grad():
                 model(data)
-        setattr(ops, which, orig)
-        a, kw = captured["args"]
+        for nm in names:
+            setattr(ops, nm, originals[nm])
         for _ in range(5):
             dst.copy_(src)
-        for _ in range(5):
-            orig(*a, **kw)
+        for nm, (a, kw) in captured.items():
+            for _ in range(5):
+                if nm == "staged_rings":
+                    ops._ring_cache.clear()
+                originals[nm](*a, **kw)
         torch.cuda.synchronize()
         print(json.dumps({"profile_kernel": True, "copy_bytes_read": src.numel() * 4,
                           "copy_bytes_written": src.numel() * 4, "edges": E, "atoms": N}))
@@ -585,7 +594,9 @@ def main() -> int:
                                                                   required=not args.no_counters)
     work = executed_work(counters, enc_avg_ms) if (counters and enc_avg_ms > 0) else None
     roofline = {
-        "kernel": "real_enc_fwd_pair_kernel (periodic encoding forward, projection fused)",
+        "kernel": ("real_enc_fwd_ring_kernel (periodic encoding forward from the staged translations, projection "
+                   "fused)" if calls["real_enc_fwd_rings"] else
+                   "real_enc_fwd_pair_kernel (periodic encoding forward, projection fused)"),
         "bound": "mfma",
         # executed fp32 work (instruction counters of a stored rocprofv3 --pmc run of this kernel
         # on this workload) over the launch time measured in this run

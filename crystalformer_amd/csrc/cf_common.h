@@ -156,6 +156,20 @@ __device__ __forceinline__ int wave_max_i(int v)
     return __builtin_amdgcn_readlane(v, 63);
 }
 
+// Sum over the four rows of 16 lanes (lanes c, c + 16, c + 32, c + 48), left in every lane: two
+// lane-swap instructions of gfx950 (odd rows of one copy against even rows of the other, then the
+// upper half against the lower half) instead of two trips through the LDS permute path.
+typedef unsigned int uint2_cf __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float rows_sum(float v)
+{
+    unsigned int x = (unsigned int)__float_as_int(v);
+    uint2_cf r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+    v = __int_as_float((int)r[0]) + __int_as_float((int)r[1]);
+    x = (unsigned int)__float_as_int(v);
+    r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return __int_as_float((int)r[0]) + __int_as_float((int)r[1]);
+}
+
 // Inclusive prefix sum over the 64 lanes (Hillis-Steele inside each row of 16 lanes on
 // row shifts, then the row totals carried across with the two broadcasts), 6 instructions.
 constexpr int DPP_ROW_SHR1 = 0x111, DPP_ROW_SHR2 = 0x112, DPP_ROW_SHR4 = 0x114, DPP_ROW_SHR8 = 0x118;

@@ -450,8 +450,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
             if (lane == 0) tick[it & 1] = t;
         }
         // column totals: the 4 lanes sharing c hold partial sums
-        sum += __shfl_xor(sum, 16, WAVE);
-        sum += __shfl_xor(sum, 32, WAVE);
+        sum = rows_sum(sum);
         const float inv = __builtin_amdgcn_rcpf(sum);      // 1 ulp, one instruction
         const int64_t e_col = (c < 8) ? e_ij : e_ji;
         if (col_on && q == 0) p.z[e_col * H + h] = log2_hw(sum) * LN2 + d2min * a;
@@ -541,8 +540,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                                 if (k0 + r < K) o = fmaf(Wg[(int64_t)(d0 + dd) * K + k0 + r], acc[m][r], o);
                         }
                     }
-                    o += __shfl_xor(o, 16, WAVE);
-                    o += __shfl_xor(o, 32, WAVE);
+                    o = rows_sum(o);
                     // lane q keeps components 4q .. 4q+3
                     if ((dd >> 2) == q) {
                         if ((dd & 3) == 0) o0 = o;

@@ -91,13 +91,17 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         // lane (q, j) holds gW[d = 4q + r][bin = 16t + j] of head hg_*8 + wave
         const int hw = hg_ * 8 + wave;
         if (p.gW_part && hw < H) {
+            // (the flush sits inside the round loop for the change of head group; its 16 offsets and
+            // masks are worked out here each time, not kept in registers across the rounds)
+            int qq = q, cc = c;
+            asm volatile("" : "+v"(qq), "+v"(cc));
             float *dst = p.gW_part + ((int64_t)blockIdx.x * H + hw) * D * K;
 #pragma unroll
             for (int t = 0; t < NT; t++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const int d = 4 * q + r, k = 16 * t + c;
-                    if (d < D && k < K) dst[d * K + k] = gw_slot[t * WAVE][r];
+                    const int d = 4 * qq + r, k = 16 * t + cc;
+                    if (d < D && k < K) dst[(unsigned)(d * K + k)] = gw_slot[t * WAVE][r];
                 }
         }
     };
@@ -342,8 +346,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         UnitGeom geo_next{};
         if (!RINGS) geo_next = unit_geom(gv_next, !UNIFORM);
         const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane);
-        px += __shfl_xor(px, 16, WAVE);
-        px += __shfl_xor(px, 32, WAVE);
+        px = rows_sum(px);
 
         // ---- exchange: column (dir, head) of unit `wave` -> row ((head*2 + dir)*8 + wave)
         if (q == 0) PXbuf[wave * 16 + c] = px;
@@ -373,14 +376,16 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         }
         // gradient operands of this wave's head for the 16 product columns, requested before
         // the exchange so that they arrive while the columns are parked
-        const int64_t e_out = col_edge;
+        // (edge, head) rows are 32-bit: the launcher refuses E H >= 2^32
+        const int e_out = col_edge;
+        const unsigned row_out = (unsigned)col_edge * (unsigned)H + (unsigned)hw;
         float4_t gv4 = {0.f, 0.f, 0.f, 0.f};
         float gz_out = 0.f;
         float gvk[4] = {0.f, 0.f, 0.f, 0.f};
         if (hw < H) {
-            if (e_out >= 0 && g_gz && q == 0) gz_out = g_gz[e_out * H + hw];
+            if (e_out >= 0 && g_gz && q == 0) gz_out = g_gz[row_out];
             if (e_out >= 0 && g_gv) {
-                const float *gp = g_gv + (e_out * H + hw) * D + 4 * q;
+                const float *gp = g_gv + ((uint64_t)row_out * (unsigned)D + (unsigned)(4 * q));
                 if (4 * q + 3 < D) {
                     gv4 = *reinterpret_cast<const float4_t *>(gp);
                 } else {
@@ -426,19 +431,19 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 }
                 // lane (q, j): components d = 4q + r of W Q' for column j; dot with gv
                 float dot = out[0] * gv4[0] + out[1] * gv4[1] + out[2] * gv4[2] + out[3] * gv4[3];
-                dot += __shfl_xor(dot, 16, WAVE);
-                dot += __shfl_xor(dot, 32, WAVE);
+                dot = rows_sum(dot);
                 if (q == 0 && e_out >= 0 && hw < H) {
                     const float PX = PXbuf[unit_j * 16 + dir_j * 8 + wave];
-                    p.ga_edge[e_out * H + hw] = fmaf(PX, gz_out, dot);
+                    p.ga_edge[row_out] = fmaf(PX, gz_out, dot);
                 }
                 // operands of the gW update of the next pass, requested now so that they arrive
                 // while S is being exchanged
                 if (hw < H && p.gW_part && g_gv) {
 #pragma unroll
                     for (int s4 = 0; s4 < 4; s4++) {
-                        const int64_t e_k = __shfl(col_edge, 4 * s4 + q, WAVE);      // column 4*s4 + q (sign-extended)
-                        if (e_k >= 0 && c < D) gvk[s4] = g_gv[(e_k * H + hw) * D + c];
+                        const int e_k = __builtin_amdgcn_ds_bpermute((4 * s4 + q) << 2, col_edge);   // column 4*s4 + q
+                        const unsigned row_k = (unsigned)e_k * (unsigned)H + (unsigned)hw;
+                        if (e_k >= 0 && c < D) gvk[s4] = g_gv[(uint64_t)row_k * (unsigned)D + (unsigned)c];
                     }
                 }
             } else {
@@ -577,7 +582,7 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
     const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)4 * NT * XPLANE + WPB * 16 +
                                         (size_t)WPB * NT * WAVE * 4) + 16;
     if (((U + WPB - 1) / WPB) * ((H + 7) / 8) >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // 32-bit round positions
-    if (E >= (1ll << 31)) return CF_ERR_UNSUPPORTED;                                        // 32-bit column edge ids
+    if (E >= (1ll << 31) || E * H >= (1ll << 32)) return CF_ERR_UNSUPPORTED;                // 32-bit edge ids and rows
     const int blocks = real_enc_bwd_pairs_blocks(U, H);
 #define CF_BPAIR(NTV)                                                                              \
     do {                                                                                           \

@@ -301,8 +301,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
         }
         wave_mem_sync();
         const UnitIds ids_next2 = unit_ids(dv_next2);
-        sum += __shfl_xor(sum, 16, WAVE);
-        sum += __shfl_xor(sum, 32, WAVE);
+        sum = rows_sum(sum);
         const float inv = __builtin_amdgcn_rcpf(sum);
         const int64_t e_col = (c < 8) ? e_ij : e_ji;
         if (col_on && q == 0) p.z[e_col * H + h] = log2_hw(sum) * LN2 + d2min * a;
