@@ -70,22 +70,24 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         return (rd_ < rounds && u_ < p.U) ? u_ : 0;
     };
     // exponent and forward output of column c of a unit in the head group of a round
+    // (atom and edge rows times H fit 32 bits: checked by the launcher)
     auto load_a = [&](const UnitIds &d, const RoundPos &rp) -> float {
-        const int h_ = min(rp.hg * 8 + (c & 7), H - 1);
-        return g_a[((c < 8) ? d.i : d.j) * H + h_];
+        const unsigned h_ = (unsigned)min(rp.hg * 8 + (c & 7), H - 1);
+        return g_a[((c < 8) ? (unsigned)d.i : (unsigned)d.j) * (unsigned)H + h_];
     };
     auto load_z = [&](const UnitIds &d, const RoundPos &rp) -> float {
-        const int h_ = min(rp.hg * 8 + (c & 7), H - 1);
-        return g_z[((c < 8) ? d.e_ij : d.e_ji) * H + h_];
+        const unsigned h_ = (unsigned)min(rp.hg * 8 + (c & 7), H - 1);
+        return g_z[((c < 8) ? (unsigned)d.e_ij : (unsigned)d.e_ji) * (unsigned)H + h_];
     };
     // edge of product column c of round rd_: direction c/8 of the unit of wave c%8
     // (-1: no such unit, or the reverse of a self edge)
     // (32-bit: the launcher refuses edge counts of 2^31 and more)
     auto load_col_edge = [&](int rd_, const RoundPos &rp) -> int {
-        const int64_t u_ = (int64_t)rp.r * WPB + (c & 7);
-        if (rd_ >= rounds || u_ >= p.U) return -1;
-        const int64_t e0 = g_pairs[u_ * PAIR_FIELDS], e1 = g_pairs[u_ * PAIR_FIELDS + 1];
-        return (int)((c < 8) ? e0 : (e1 != e0 ? e1 : -1));
+        const unsigned u_ = (unsigned)rp.r * WPB + (unsigned)(c & 7);       // (rounds < 2^30)
+        if (rd_ >= rounds || (int64_t)u_ >= p.U) return -1;
+        const int64_t *d_ = g_pairs + (uint64_t)u_ * PAIR_FIELDS;
+        const int e0 = (int)d_[0], e1 = (int)d_[1];
+        return (c < 8) ? e0 : (e1 != e0 ? e1 : -1);
     };
     auto flush_gW = [&](int hg_) {
         // lane (q, j) holds gW[d = 4q + r][bin = 16t + j] of head hg_*8 + wave
@@ -582,7 +584,7 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
     const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)4 * NT * XPLANE + WPB * 16 +
                                         (size_t)WPB * NT * WAVE * 4) + 16;
     if (((U + WPB - 1) / WPB) * ((H + 7) / 8) >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // 32-bit round positions
-    if (E >= (1ll << 31) || E * H >= (1ll << 32)) return CF_ERR_UNSUPPORTED;                // 32-bit edge ids and rows
+    if (E >= (1ll << 31) || E * H >= (1ll << 32) || N * H >= (1ll << 32)) return CF_ERR_UNSUPPORTED;   // 32-bit ids, rows
     const int blocks = real_enc_bwd_pairs_blocks(U, H);
 #define CF_BPAIR(NTV)                                                                              \
     do {                                                                                           \

@@ -191,8 +191,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
         return (rd_ < rounds && u_ < p.U) ? u_ : 0;
     };
     auto load_a = [&](const UnitIds &d, const RoundPos &rp) -> float {
-        const int h_ = min(rp.hg * 8 + (c & 7), H - 1);
-        return g_a[((c < 8) ? d.i : d.j) * H + h_];
+        const unsigned h_ = (unsigned)min(rp.hg * 8 + (c & 7), H - 1);
+        return g_a[((c < 8) ? (unsigned)d.i : (unsigned)d.j) * (unsigned)H + h_];
     };
     using Image = RingImage;
     auto load_image = [&](int64_t u_) -> Image { return load_ring_image(cache, u_, lane); };
@@ -303,8 +303,9 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
         const UnitIds ids_next2 = unit_ids(dv_next2);
         sum = rows_sum(sum);
         const float inv = __builtin_amdgcn_rcpf(sum);
-        const int64_t e_col = (c < 8) ? e_ij : e_ji;
-        if (col_on && q == 0) p.z[e_col * H + h] = log2_hw(sum) * LN2 + d2min * a;
+        // ((edge, head) rows are 32-bit: the launcher refuses E H >= 2^32)
+        const unsigned e_col = (c < 8) ? (unsigned)e_ij : (unsigned)e_ji;
+        if (col_on && q == 0) p.z[e_col * (unsigned)H + (unsigned)h] = log2_hw(sum) * LN2 + d2min * a;
 
         // epilogue: park the column sums, project per head (see the pair kernel)
         float *col = Sbuf + xch_base(q, c & 7, wave, c >> 3);
@@ -344,7 +345,8 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++) {
                     const int dbase = 16 * dt + 4 * q;
-                    float *dst = p.v + (e_out * H + hw) * D + dbase;
+                    float *dst = p.v + ((uint64_t)((unsigned)e_out * (unsigned)H + (unsigned)hw) * (unsigned)D +
+                                        (unsigned)dbase);
                     if (dbase + 3 < D) {
                         *reinterpret_cast<float4_t *>(dst) = out[dt];
                     } else {
@@ -405,6 +407,7 @@ int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U
                               const float *cache, float *z, float *v, hipStream_t st)
 {
     if (K < 1 || K > 128 || !W || D < 1 || D > 32) return CF_ERR_UNSUPPORTED;
+    if (E * H >= (1ll << 32) || N * H >= (1ll << 32)) return CF_ERR_UNSUPPORTED;      // 32-bit rows in the kernel
     PairArgs p{};
     p.a_ik = a_ik; p.pairs = pairs; p.W = W; p.z = z; p.v = v;
     p.N = N; p.E = E; p.U = U; p.W_num = 1;
