@@ -396,34 +396,56 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                 ring_bits[pos] = 0;
             }
             wave_mem_sync();
-            // ---- accumulation over the near block: 4 translations per MFMA; the record of the
-            // next group is loaded while the current one is in use
+            // the tiles any of a group's four records reaches, kept in each record (see
+            // with_group_reach): the four records of a group sit in four adjacent lanes here
+            for (int s4 = 0; s4 < near_cnt; s4 += WAVE) {
+                const bool held = s4 + lane < near_cnt + 8;          // (slots up to near_cnt + 7 hold records)
+                const int marked = with_group_reach(held ? ring_bits[s4 + lane] : 0);
+                if (held) ring_bits[s4 + lane] = marked;
+            }
+            wave_mem_sync();
+            // ---- accumulation over the near block: 4 translations per MFMA, two groups per trip,
+            // each with its own registers for the prefetched records (records beyond the last
+            // group are the neutral padding)
             {
                 const int groups = (near_cnt + 3) >> 2;
-                float d2n = ring_d2[q], sn = ring_s[q];
-                int bitsn = ring_bits[q];
-                for (int g = 0; g < groups; g++) {
-                    const float d2t = d2n, st = sn;
-                    const int bits = bitsn;
-                    const int slot = 4 * (g + 1) + q;
-                    d2n = ring_d2[slot];
-                    sn = ring_s[slot];
-                    bitsn = ring_bits[slot];
-                    float w = exp2_hw(a2 * (d2t - d2min));
+                struct Rec { float d2, s; int bits; };
+                auto fetch = [&](int g_) -> Rec {
+                    const int slot = 4 * g_ + q;
+                    return Rec{ring_d2[slot], ring_s[slot], ring_bits[slot]};
+                };
+                auto group = [&](const Rec &rec) {
+                    float w = exp2_hw(a2 * (rec.d2 - d2min));
                     // (fixed cube: every staged translation is inside every column's box, and the
                     // padding records carry d2 = +inf, i.e. weight 0)
-                    w = (col_on && (UNIFORM || ((bits >> c) & 1))) ? w : 0.f;
+                    w = (col_on && (UNIFORM || ((rec.bits >> c) & 1))) ? w : 0.f;
                     sum += w;
-                    // tiles within reach of any of the group's 4 translations (one record per q)
-                    const int reach = __builtin_amdgcn_readlane(bits, 0) | __builtin_amdgcn_readlane(bits, 16) |
-                                      __builtin_amdgcn_readlane(bits, 32) | __builtin_amdgcn_readlane(bits, 48);
+                    const int reach = group_reach(rec.bits);
 #pragma unroll
                     for (int m = 0; m < NT; m++) {
                         if (reach & (0x10000 << m)) {                             // wave-uniform
-                            float b = ck[m] - st;
+                            float b = ck[m] - rec.s;
                             float gm = exp2_hw(-(b * b));
                             acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, w, acc[m], 0, 0, 0);
                         }
+                    }
+                };
+                Rec ra = fetch(0);
+                if (UNIFORM) {
+                    for (int g = 0; g < groups; g += 2) {
+                        const Rec rb = fetch(g + 1);
+                        group(ra);
+                        if (g + 1 < groups) {
+                            ra = fetch(g + 2);
+                            group(rb);
+                        }
+                    }
+                } else {
+                    // (adaptive boxes: no registers to spare for the second record set)
+                    for (int g = 0; g < groups; g++) {
+                        const Rec rb = fetch(g + 1);
+                        group(ra);
+                        ra = rb;
                     }
                 }
             }

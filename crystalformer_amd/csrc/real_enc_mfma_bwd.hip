@@ -162,7 +162,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             if (near_cnt + 8 > 2 * WAVE || far_cnt > 0)          // slots 128 .. 143 (wave-uniform, rare)
                 copy_ring_tail(p.rings, u, ring_d2, ring_s, ring_bits, lane);
             if (!unit_on && lane < 8) {                          // no unit: an empty near block
-                ring_d2[lane] = __builtin_inff();
+                ring_d2[lane] = RIMG_NEUTRAL_D2;
                 ring_s[lane] = 0.f;
                 ring_bits[lane] = 0;
             }
@@ -301,33 +301,53 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 ring_bits[pos] = 0;
             }
             wave_mem_sync();
+            if (!RINGS) {
+                // the tiles any of a group's four records reaches, kept in each record (an image
+                // gets them on its way into the ring): a group's records sit in adjacent lanes here
+                for (int s4 = 0; s4 < near_cnt; s4 += WAVE) {
+                    const bool held = s4 + lane < near_cnt + 8;      // (slots up to near_cnt + 7 hold records)
+                    const int marked = with_group_reach(held ? ring_bits[s4 + lane] : 0);
+                    if (held) ring_bits[s4 + lane] = marked;
+                }
+                wave_mem_sync();
+            }
             {
+                // two groups per trip, each with its own registers for the prefetched records;
+                // records beyond the last group are the neutral padding
                 const int groups = (near_cnt + 3) >> 2;
-                float d2n = ring_d2[q], sn = ring_s[q];
-                int bitsn = ring_bits[q];
-                for (int g = 0; g < groups; g++) {
-                    const float d2t = d2n, st = sn;
-                    const int bits = bitsn;
-                    const int slot = 4 * (g + 1) + q;
-                    d2n = ring_d2[slot];
-                    sn = ring_s[slot];
-                    bitsn = ring_bits[slot];
-                    const bool on = col_on && ((bits >> c) & 1);
-                    // padding records carry d2 = +inf: keep them out of p*d2
-                    const float w = on ? exp2_hw(a2 * d2t - z2) : 0.f;
-                    const float wd = on ? w * d2t : 0.f;
+                struct Rec { float d2, s; int bits; };
+                auto fetch = [&](int g_) -> Rec {
+                    const int slot = 4 * g_ + q;
+                    return Rec{ring_d2[slot], ring_s[slot], ring_bits[slot]};
+                };
+                auto group = [&](const Rec &rec) {
+                    // padding records carry d2 = +inf: keep them out of p*d2.  (From an image the
+                    // padding has a large finite d2, weight 0 and 0 * d2 = 0, every record is in every
+                    // column's box, and columns that are switched off run with a = -1 and finite
+                    // garbage that is never stored: nothing to mask.)
+                    const bool on = RINGS || (col_on && ((rec.bits >> c) & 1));
+                    const float w = on ? exp2_hw(a2 * rec.d2 - z2) : 0.f;
+                    const float wd = on ? w * rec.d2 : 0.f;
                     px += wd;
                     // tiles within reach of any of the group's 4 translations (one record per q)
-                    const int reach = __builtin_amdgcn_readlane(bits, 0) | __builtin_amdgcn_readlane(bits, 16) |
-                                      __builtin_amdgcn_readlane(bits, 32) | __builtin_amdgcn_readlane(bits, 48);
+                    const int reach = group_reach(rec.bits);
 #pragma unroll
                     for (int m = 0; m < NT; m++) {
                         if (reach & (0x10000 << m)) {
-                            float b = ck[m] - st;
+                            float b = ck[m] - rec.s;
                             float gm = exp2_hw(-(b * b));
                             accS[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, w, accS[m], 0, 0, 0);
                             accQ[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, wd, accQ[m], 0, 0, 0);
                         }
+                    }
+                };
+                Rec ra = fetch(0);
+                for (int g = 0; g < groups; g += 2) {
+                    const Rec rb = fetch(g + 1);
+                    group(ra);
+                    if (g + 1 < groups) {
+                        ra = fetch(g + 2);
+                        group(rb);
                     }
                 }
             }
@@ -337,7 +357,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                     const int slot = BRING_SLOTS - 4 * (g + 1) + q;
                     const float d2t = ring_d2[slot];
                     const int bits = ring_bits[slot];
-                    if (col_on && ((bits >> c) & 1)) px += exp2_hw(a2 * d2t - z2) * d2t;
+                    if (RINGS || (col_on && ((bits >> c) & 1))) px += exp2_hw(a2 * d2t - z2) * d2t;
                 }
             }
             wave_mem_sync();

@@ -230,11 +230,15 @@ __device__ __forceinline__ int proj_bin(int s, int kk) { return 16 * (s >> 2) + 
 // Image of a unit's staged translations (fixed cube of at most RIMG_CAP translations), RIMG_WORDS
 // 32-bit words: d2[RIMG_SLOTS], s[RIMG_SLOTS], bits[RIMG_SLOTS], header {near count, far count,
 // smallest d2, -}.  Near records occupy slots 0 .. near-1 followed by 8 neutral records
-// (d2 = +inf, no bits); far records occupy slots RIMG_SLOTS-1 downwards followed (below) by 4
+// (d2 = RIMG_NEUTRAL_D2, no bits); far records occupy slots RIMG_SLOTS-1 downwards followed (below) by 4
 // neutral records.
 constexpr int RIMG_CAP = 128;
 constexpr int RIMG_SLOTS = RIMG_CAP + 16;
 constexpr int RIMG_WORDS = 3 * RIMG_SLOTS + 4;
+
+// d2 of a neutral record of an image: large and finite, so that a weight exp(a d2) is 0 for every
+// exponent and 0 * d2 is 0 too (no masking of the padding in the loops that run from an image)
+constexpr float RIMG_NEUTRAL_D2 = 1e30f;
 
 // slots lane and 64 + lane of the three arrays, and the header word min(lane, 3)
 struct RingImage { float d2[2], s[2]; int bits[2]; int hdr; };
@@ -253,6 +257,20 @@ __device__ __forceinline__ RingImage load_ring_image(const float *__restrict__ r
     return im;
 }
 
+// The accumulation takes four consecutive slots at a time and needs the tiles any of the four
+// reaches as one wave-uniform value.  The four records sit in four adjacent lanes here (a quad), so
+// the union is formed on the way into LDS (two quad swaps) and kept in bits 24..31 of each record:
+// the loop then reads it from any lane instead of collecting four records' bits.
+__device__ __forceinline__ int with_group_reach(int bits)
+{
+    int t = (bits >> 16) & 0xFF;
+    t |= dpp_i<DPP_QUAD_1032, 0xF>(t, t);
+    t |= dpp_i<DPP_QUAD_2301, 0xF>(t, t);
+    return bits | (t << 24);
+}
+// tiles within reach of the group of a record read back from the ring (wave-uniform, tile m at bit 16 + m)
+__device__ __forceinline__ int group_reach(int bits) { return __builtin_amdgcn_readfirstlane(bits) >> 8; }
+
 __device__ __forceinline__ void store_ring_image(const RingImage &im, float *ring_d2, float *ring_s, int *ring_bits,
                                                  int lane)
 {
@@ -260,7 +278,7 @@ __device__ __forceinline__ void store_ring_image(const RingImage &im, float *rin
     for (int k = 0; k < 2; k++) {
         ring_d2[k * WAVE + lane] = im.d2[k];
         ring_s[k * WAVE + lane] = im.s[k];
-        ring_bits[k * WAVE + lane] = im.bits[k];
+        ring_bits[k * WAVE + lane] = with_group_reach(im.bits[k]);
     }
 }
 
@@ -272,7 +290,7 @@ __device__ __forceinline__ void copy_ring_tail(const float *__restrict__ rings, 
         const float *base = rings + u * RIMG_WORDS;
         ring_d2[2 * WAVE + lane] = base[2 * WAVE + lane];
         ring_s[2 * WAVE + lane] = base[RIMG_SLOTS + 2 * WAVE + lane];
-        ring_bits[2 * WAVE + lane] = __float_as_int(base[2 * RIMG_SLOTS + 2 * WAVE + lane]);
+        ring_bits[2 * WAVE + lane] = with_group_reach(__float_as_int(base[2 * RIMG_SLOTS + 2 * WAVE + lane]));
     }
 }
 

@@ -139,7 +139,7 @@ __global__ __launch_bounds__(256) void ring_stage_kernel(PairArgs p, float weak_
     // neutral records: 8 after the near block (last group + look-ahead), 4 below the far block
     if (lane < 12) {
         const int pos = lane < 8 ? near_cnt + lane : RS - far_cnt - 1 - (lane - 8);
-        ring_d2[pos] = __builtin_inff();
+        ring_d2[pos] = RIMG_NEUTRAL_D2;
         ring_s[pos] = 0.f;
         ring_bits[pos] = 0;
     }
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
         if (near_cnt + 8 > 2 * WAVE || far_cnt > 0)              // slots 128 .. 143 (wave-uniform, rare)
             copy_ring_tail(cache, u, ring_d2, ring_s, ring_bits, lane);
         if (!unit_on && lane < 8) {          // no unit: an empty near block (neutral records)
-            ring_d2[lane] = __builtin_inff();
+            ring_d2[lane] = RIMG_NEUTRAL_D2;
             ring_s[lane] = 0.f;
             ring_bits[lane] = 0;
         }
@@ -263,28 +263,36 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
         wave_mem_sync();
         // ---- accumulation over the near block: 4 translations per MFMA
         {
+            // two groups per trip, each with its own registers for the prefetched records (no
+            // copies from "next" to "current"); records beyond the last group are the neutral padding
             const int groups = (near_cnt + 3) >> 2;
-            float d2n = ring_d2[q], sn = ring_s[q];
-            int bitsn = ring_bits[q];
-            for (int g = 0; g < groups; g++) {
-                const float d2t = d2n, st = sn;
-                const int bits = bitsn;
-                const int slot = 4 * (g + 1) + q;
-                d2n = ring_d2[slot];
-                sn = ring_s[slot];
-                bitsn = ring_bits[slot];
-                float w = exp2_hw(a2 * (d2t - d2min));
-                w = col_on ? w : 0.f;                   // (padding records carry d2 = +inf: weight 0)
+            struct Rec { float d2, s; int bits; };
+            auto fetch = [&](int g_) -> Rec {
+                const int slot = 4 * g_ + q;
+                return Rec{ring_d2[slot], ring_s[slot], ring_bits[slot]};
+            };
+            auto group = [&](const Rec &rec) {
+                // (padding records: weight 0 through their d2; columns that are switched off run
+                // with a = -1 and finite garbage that is never stored)
+                const float w = exp2_hw(a2 * (rec.d2 - d2min));
                 sum += w;
-                const int reach = __builtin_amdgcn_readlane(bits, 0) | __builtin_amdgcn_readlane(bits, 16) |
-                                  __builtin_amdgcn_readlane(bits, 32) | __builtin_amdgcn_readlane(bits, 48);
+                const int reach = group_reach(rec.bits);
 #pragma unroll
                 for (int m = 0; m < NT; m++) {
                     if (reach & (0x10000 << m)) {                             // wave-uniform
-                        float b = ck[m] - st;
+                        float b = ck[m] - rec.s;
                         float gm = exp2_hw(-(b * b));
                         acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(gm, w, acc[m], 0, 0, 0);
                     }
+                }
+            };
+            Rec ra = fetch(0);
+            for (int g = 0; g < groups; g += 2) {
+                const Rec rb = fetch(g + 1);
+                group(ra);
+                if (g + 1 < groups) {
+                    ra = fetch(g + 2);
+                    group(rb);
                 }
             }
         }
@@ -293,10 +301,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
             const int groups = (far_cnt + 3) >> 2;
             for (int g = 0; g < groups; g++) {
                 const int slot = RS - 4 * (g + 1) + q;
-                const float d2t = ring_d2[slot];
-                const int bits = ring_bits[slot];
-                float w = exp2_hw(a2 * (d2t - d2min));
-                sum += (col_on && ((bits >> c) & 1)) ? w : 0.f;
+                sum += exp2_hw(a2 * (ring_d2[slot] - d2min));
             }
         }
         wave_mem_sync();
