@@ -1033,8 +1033,8 @@ extern "C" int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const 
     if (pairs_u) {
         rc = launch_real_enc_fwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, N, H, E, K, D,
                                        p.bin_step, p.s_scale, p.W, W_num, rvlen_n, p.cutoff, lattice_range,
-                                       minimum_range, reinterpret_cast<unsigned int *>(sched_2), z_ek, v_ekd,
-                                       (hipStream_t)stream);
+                                       minimum_range, reinterpret_cast<unsigned int *>(sched_2), nullptr, nullptr,
+                                       z_ek, v_ekd, (hipStream_t)stream);
         if (rc == CF_OK) {
             CF_CHECK_LAUNCH("cf_real_enc_fwd (pairs)");
             return CF_OK;

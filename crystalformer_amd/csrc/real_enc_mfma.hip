@@ -104,11 +104,24 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
     __shared__ int tick[2];
     unsigned int *__restrict__ sched = p.sched;
     const int stride = gridDim.x;
-    int rd_next = blockIdx.x + stride, rd_next2 = blockIdx.x + 2 * stride;
-    RoundPos pos = round_pos(blockIdx.x, rounds_per_hg, p.head_groups);
+    // Adaptive boxes with unit selection (p.unit_flags): this launch takes the units that do not keep
+    // the cube and walks only the rounds that hold one (no tickets then: the launcher passes none).
+    const bool select = !UNIFORM && p.unit_flags != nullptr;
+    int rd_first = blockIdx.x, rd_next = blockIdx.x + stride, rd_next2 = blockIdx.x + 2 * stride;
+    if (select) {
+        const RoundSeq seq = first_active_rounds(p, blockIdx.x, rounds, stride, lane);
+        rd_first = seq.rd[0];
+        rd_next = seq.rd[1];
+        rd_next2 = seq.rd[2];
+    }
+    auto unit_flag = [&](int rd_, const RoundPos &rp) -> int {
+        return select ? load_unit_flag(p, unit_of(rd_, rp), rd_ < rounds ? rp.hg : 0) : 0;
+    };
+    RoundPos pos = round_pos(rd_first, rounds_per_hg, p.head_groups);
     RoundPos pos_next = round_pos(rd_next, rounds_per_hg, p.head_groups);
     // fill the descriptor pipeline: current round complete, next round's ids known
-    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x, pos), lane));
+    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(rd_first, pos), lane));
+    int uflag = unit_flag(rd_first, pos);
     float a_cur;
     UnitGeom geo;
     UnitIds ids_next;
@@ -144,11 +157,14 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         }
     }
     int it = 0;
-    for (int rd = blockIdx.x; rd < rounds; it++) {
+    for (int rd = rd_first; rd < rounds; it++) {
         const int hg = pos.hg;
         const int64_t u = (int64_t)pos.r * WPB + wave;
-        const bool unit_on = u < p.U;
+        const bool unit_on = u < p.U && (!select || unit_selected(p, uflag));
         const RoundPos pos_next2 = round_pos(rd_next2, rounds_per_hg, p.head_groups);
+        // (the round after rd_next2: its candidates' flags are requested here, looked at at the end)
+        bool candidate = false;
+        if (select) candidate = request_round_candidate(p, rd_next2, rounds, stride, lane);
         // ticket for the round after rd_next2 (once past the end, no more draws): requested here,
         // looked at only before the epilogue, like the loads below
         unsigned int ticket_old = 0;
@@ -157,6 +173,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         // loads for the coming rounds, consumed just before this round's epilogue
         const float gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
         const float a_next = load_a(ids_next, pos_next);
+        const int uflag_next = unit_flag(rd_next, pos_next);
         const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd_next2, pos_next2), lane);
         if (PROJ == PROJ_SHARED && hg != wa_hg) {
             const int hw = hg * 8 + wave;
@@ -174,11 +191,15 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
                     }
                 }
             } else {
+                // (taken when the head group changes: its masks and offsets are worked out here,
+                // not kept in registers across the rounds)
+                int qq = q, cc = c;
+                asm volatile("" : "+v"(qq), "+v"(cc));
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                     for (int s = 0; s < 4 * NT; s++) {
-                        const int d = 16 * dt + c, k = proj_bin(s, q);
+                        const int d = 16 * dt + cc, k = proj_bin(s, qq);
                         Wa[dt][s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
                     }
             }
@@ -584,10 +605,11 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
         ids = ids_next;
         geo = geo_next;
         a_cur = a_next;
+        uflag = uflag_next;
         ids_next = ids_next2;
         pos = pos_next;
         pos_next = pos_next2;
-        int rd_next3 = rd_next2 + stride;
+        int rd_next3 = select ? round_after(p, candidate, rd_next2, rounds, stride, lane) : rd_next2 + stride;
         if (sched) {
             if (PROJ != PROJ_SHARED) __syncthreads();     // (the shared projection has its own barriers)
             rd_next3 = tick[it & 1];
@@ -644,9 +666,11 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
                               const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
                               int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
                               int64_t W_num, const float *rvlen, float cutoff, int lattice_range,
-                              int min_range, unsigned int *sched, float *z, float *v, hipStream_t st)
+                              int min_range, unsigned int *sched, const unsigned char *unit_flags,
+                              const unsigned char *round_flags, float *z, float *v, hipStream_t st)
 {
     if (K < 0 || K > 128) return CF_ERR_UNSUPPORTED;
+    if (unit_flags && (cutoff == 0.0f || !round_flags)) return CF_ERR_UNSUPPORTED;   // selection: adaptive boxes only
     if (W && (D < 1 || D > 64)) return CF_ERR_UNSUPPORTED;
     PairArgs p{};
     p.a_ik = a_ik; p.rpos = rpos; p.tvecs = tvecs; p.batch = batch; p.edges = edges; p.pairs = pairs;
@@ -686,6 +710,9 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     // and the fixed stride, which costs nothing, does better (measured: 64.5 against 70 us at
     // 7 rounds per work-group; 1.66 against 1.81 ms at 217).
     if (rounds < 16 * blocks) p.sched = nullptr;
+    // unit selection: the units that do not keep the cube (the others run from the staged rings)
+    p.unit_flags = unit_flags; p.round_flags = round_flags; p.flag_want = 0;
+    if (unit_flags) p.sched = nullptr;
 #define CF_PAIR(NTV, UNI, PRJ, DTV, SR) \
     real_enc_fwd_pair_kernel<NTV, UNI, PRJ, DTV, SR><<<(int)blocks, WPB * WAVE, lds, st>>>(p)
 #define CF_PAIR_MODE(NTV, UNI, SR)                                            \

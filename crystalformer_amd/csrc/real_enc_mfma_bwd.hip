@@ -390,9 +390,12 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 for (int r = 0; r < 4; r++) Wa[4 * t4 + r] = w4[r];
             }
         } else {
+            // (partial tiles: masks and offsets worked out here, not kept in registers across the rounds)
+            int qq = q, cc = c;
+            asm volatile("" : "+v"(qq), "+v"(cc));
 #pragma unroll
             for (int s = 0; s < 4 * NT; s++) {
-                const int d = c, k = proj_bin(s, q);
+                const int d = cc, k = proj_bin(s, qq);
                 Wa[s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
             }
         }

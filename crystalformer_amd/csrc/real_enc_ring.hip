@@ -154,12 +154,55 @@ __global__ __launch_bounds__(256) void ring_stage_kernel(PairArgs p, float weak_
     }
 }
 
+// ---------------------------------------------------------------- unit selection
+// Adaptive boxes: which units keep the fixed cube in all their active columns (the range rule of
+// every (atom, head) of the unit yields lattice_range on the three axes).  Those are evaluated from
+// the staged rings, on the bits the pair kernel's own shortcut for such units produces; the others
+// go to the pair kernel.  One wavefront per round (8 units) and head group: lane = (unit, head),
+// each lane applies the rule to its head of atoms i and j.
+__global__ __launch_bounds__(256) void unit_floor_kernel(PairArgs p, unsigned char *__restrict__ unit_flags,
+                                                         unsigned char *__restrict__ round_flags)
+{
+    const int lane = threadIdx.x & 63;
+    const int rounds_per_hg = (int)((p.U + WPB - 1) / WPB);
+    const int64_t rounds = (int64_t)rounds_per_hg * p.head_groups;
+    const int64_t rd = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (rd >= rounds) return;
+    const RoundPos rp = round_pos((int)rd, rounds_per_hg, p.head_groups);
+    const int w = lane >> 3, hh = lane & 7;
+    const int64_t u = (int64_t)rp.r * WPB + w;
+    const bool exists = u < p.U;
+    bool keeps = true;
+    if (exists) {
+        const int64_t *d = p.pairs + u * PAIR_FIELDS;
+        const int64_t e_ij = d[0], e_ji = d[1], n = d[4];
+        const int h = rp.hg * 8 + hh;
+        if (h < p.H) {
+            const float rvl[3] = {p.rvlen[n * 3 + 0], p.rvlen[n * 3 + 1], p.rvlen[n * 3 + 2]};
+#pragma unroll
+            for (int side = 0; side < 2; side++) {
+                if (side == 1 && e_ji == e_ij) continue;         // a self pair has one direction
+                int R1, R2, R3;
+                range_rule(p.a_ik[d[2 + side] * p.H + h], p.cutoff, rvl, p.lattice_range, p.min_range, R1, R2, R3);
+                keeps = keeps && R1 == p.lattice_range && R2 == p.lattice_range && R3 == p.lattice_range;
+            }
+        }
+    }
+    const unsigned long long km = __ballot(keeps);
+    const bool unit_keeps = exists && ((km >> (8 * w)) & 0xFFull) == 0xFFull;
+    if (exists && hh == 0) unit_flags[(int64_t)rp.hg * p.U + u] = unit_keeps ? 1 : 0;
+    const unsigned long long any_keep = __ballot(unit_keeps), any_other = __ballot(exists && !unit_keeps);
+    if (lane == 0) round_flags[rd] = (unsigned char)((any_keep != 0ull ? 1 : 0) | (any_other != 0ull ? 2 : 0));
+}
+
 // ---------------------------------------------------------------- consumer
 // Work-group of 8 wavefronts, one unit per wavefront and round, as in the pair kernel.  The image
 // of the next round's unit (its address follows from the round number alone) is requested a round
 // ahead into registers and copied to the wavefront's LDS ring at the top of its round.
 // LDS: per wave 3 x RS words, exchange buffer 4 NT x XPLANE, 8 x 2 edge ids, 8 x 16 reciprocals.
-template <int NT, int DT>
+// SELECT: only the units picked by p.unit_flags / p.flag_want are evaluated, and only the rounds
+// that hold one are walked (p.round_flags).
+template <int NT, int DT, bool SELECT>
 __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, const float *__restrict__ cache)
 {
     extern __shared__ __align__(16) float lds[];
@@ -197,18 +240,38 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
     using Image = RingImage;
     auto load_image = [&](int64_t u_) -> Image { return load_ring_image(cache, u_, lane); };
 
-    RoundPos pos = round_pos(blockIdx.x, rounds_per_hg, p.head_groups);
-    RoundPos pos_next = round_pos(blockIdx.x + stride, rounds_per_hg, p.head_groups);
-    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x, pos), lane));
+    // rounds of this work-group: blockIdx.x, + grid, + 2 grid, ...; with SELECT those of them that
+    // hold a unit of this launch, known three rounds ahead
+    int rd, rd_next, rd_next2;
+    if (SELECT) {
+        const RoundSeq seq = first_active_rounds(p, blockIdx.x, rounds, stride, lane);
+        rd = seq.rd[0];
+        rd_next = seq.rd[1];
+        rd_next2 = seq.rd[2];
+    } else {
+        rd = blockIdx.x;
+        rd_next = rd + stride;
+        rd_next2 = rd + 2 * stride;
+    }
+    auto unit_flag = [&](int rd_, const RoundPos &rp) -> int {
+        return SELECT ? load_unit_flag(p, unit_of(rd_, rp), rd_ < rounds ? rp.hg : 0) : 0;
+    };
+    RoundPos pos = round_pos(rd, rounds_per_hg, p.head_groups);
+    RoundPos pos_next = round_pos(rd_next, rounds_per_hg, p.head_groups);
+    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(rd, pos), lane));
     float a_cur = load_a(ids, pos);
-    Image img = load_image(unit_of(blockIdx.x, pos));
-    UnitIds ids_next = unit_ids(load_unit_ids(g_pairs, unit_of(blockIdx.x + stride, pos_next), lane));
+    Image img = load_image(unit_of(rd, pos));
+    int uflag = unit_flag(rd, pos);
+    UnitIds ids_next = unit_ids(load_unit_ids(g_pairs, unit_of(rd_next, pos_next), lane));
 
-    for (int rd = blockIdx.x; rd < rounds; rd += stride) {
+    while (rd < rounds) {
         const int hg = pos.hg;
         const int64_t u = (int64_t)pos.r * WPB + wave;
-        const bool unit_on = u < p.U;
-        const RoundPos pos_next2 = round_pos(rd + 2 * stride, rounds_per_hg, p.head_groups);
+        const bool unit_on = u < p.U && (!SELECT || unit_selected(p, uflag));
+        const RoundPos pos_next2 = round_pos(rd_next2, rounds_per_hg, p.head_groups);
+        // (the round after rd_next2: its candidates' flags are requested here, looked at at the end)
+        bool candidate = false;
+        if (SELECT) candidate = request_round_candidate(p, rd_next2, rounds, stride, lane);
         // this round's image into the ring (the previous round's readers of the ring are done:
         // same wavefront, and the epilogue's barriers lie in between)
         const int near_cnt = unit_on ? __builtin_amdgcn_readlane(img.hdr, 0) : 0;
@@ -223,9 +286,10 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
             ring_bits[lane] = 0;
         }
         // loads for the coming rounds
-        const Image img_next = load_image(unit_of(rd + stride, pos_next));
+        const Image img_next = load_image(unit_of(rd_next, pos_next));
         const float a_next = load_a(ids_next, pos_next);
-        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane);
+        const int uflag_next = unit_flag(rd_next, pos_next);
+        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd_next2, pos_next2), lane);
         if (hg != wa_hg) {
             const int hw = hg * 8 + wave;
             if (hw < H && K == 16 * NT && D == 16 * DT) {
@@ -240,11 +304,15 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
                     }
                 }
             } else {
+                // (taken when the head group changes: its masks and offsets are worked out here,
+                // not kept in registers across the rounds)
+                int qq = q, cc = c;
+                asm volatile("" : "+v"(qq), "+v"(cc));
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                     for (int s = 0; s < 4 * NT; s++) {
-                        const int d = 16 * dt + c, k = proj_bin(s, q);
+                        const int d = 16 * dt + cc, k = proj_bin(s, qq);
                         Wa[dt][s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
                     }
             }
@@ -366,9 +434,15 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
         ids = ids_next;
         a_cur = a_next;
         img = img_next;
+        uflag = uflag_next;
         ids_next = ids_next2;
         pos = pos_next;
         pos_next = pos_next2;
+        const int rd_next3 = SELECT ? round_after(p, candidate, rd_next2, rounds, stride, lane)
+                                    : rd_next2 + stride;
+        rd = rd_next;
+        rd_next = rd_next2;
+        rd_next2 = rd_next3;
     }
 }
 
@@ -406,10 +480,32 @@ int launch_ring_stage(const float *rpos, const float *tvecs, const int64_t *pair
     return CF_OK;
 }
 
+// Flags for the two launches of the adaptive rule (see unit_floor_kernel): unit_flags holds
+// head_groups x U bytes, round_flags one byte per round.
+int64_t real_enc_round_count(int64_t U, int64_t H) { return ((U + WPB - 1) / WPB) * ((H + 7) / 8); }
+
+int launch_unit_floor(const float *a_ik, const float *rvlen, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
+                      float cutoff, int lattice_range, int min_range, unsigned char *unit_flags,
+                      unsigned char *round_flags, hipStream_t st)
+{
+    PairArgs p{};
+    p.a_ik = a_ik; p.rvlen = rvlen; p.pairs = pairs;
+    p.N = N; p.U = U; p.H = (int)H;
+    p.head_groups = (int)((H + 7) / 8);
+    p.cutoff = cutoff; p.lattice_range = lattice_range; p.min_range = min_range;
+    const int64_t rounds = real_enc_round_count(U, H);
+    if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;
+    if (rounds < 1) return CF_OK;
+    unit_floor_kernel<<<(int)((rounds + 3) / 4), 256, 0, st>>>(p, unit_flags, round_flags);
+    return CF_OK;
+}
+
 // Forward from staged rings (shared projection, D <= 32).  CF_ERR_UNSUPPORTED otherwise.
+// With unit flags only the units that keep the cube are evaluated.
 int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U, int64_t N, int64_t H, int64_t E,
                               int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
-                              const float *cache, float *z, float *v, hipStream_t st)
+                              const float *cache, const unsigned char *unit_flags, const unsigned char *round_flags,
+                              float *z, float *v, hipStream_t st)
 {
     if (K < 1 || K > 128 || !W || D < 1 || D > 32) return CF_ERR_UNSUPPORTED;
     if (E * H >= (1ll << 32) || N * H >= (1ll << 32)) return CF_ERR_UNSUPPORTED;      // 32-bit rows in the kernel
@@ -420,6 +516,8 @@ int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U
     p.head_groups = (int)((H + 7) / 8);
     p.bin_step = bin_step; p.s_scale = s_scale; p.inv_bin_step = 1.0f / bin_step;
     p.window = sqrtf(40.0f) / bin_step;
+    p.unit_flags = unit_flags; p.round_flags = round_flags; p.flag_want = 1;      // units that keep the cube
+    const bool select = unit_flags != nullptr;
     const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
     const int DT = D > 16 ? 2 : 1;
     size_t lds = sizeof(float) * ((size_t)WPB * 3 * RS + (size_t)4 * NT * XPLANE + WPB * 16) +
@@ -430,7 +528,11 @@ int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U
     const int64_t cap = persistent_grid_cap(2);
     if (blocks > cap) blocks = cap;
     if (blocks < 1) return CF_OK;
-#define CF_RING(NTV, DTV) real_enc_fwd_ring_kernel<NTV, DTV><<<(int)blocks, WPB * WAVE, lds, st>>>(p, cache)
+#define CF_RING(NTV, DTV)                                                                               \
+    do {                                                                                                \
+        if (select) real_enc_fwd_ring_kernel<NTV, DTV, true><<<(int)blocks, WPB * WAVE, lds, st>>>(p, cache);   \
+        else real_enc_fwd_ring_kernel<NTV, DTV, false><<<(int)blocks, WPB * WAVE, lds, st>>>(p, cache);         \
+    } while (0)
 #define CF_RING_NT(NTV) do { if (DT == 1) CF_RING(NTV, 1); else CF_RING(NTV, 2); } while (0)
     switch (NT) {
         case 1: CF_RING_NT(1); break;
@@ -480,9 +582,19 @@ extern "C" int cf_real_enc_ring_stage(const float *rpos_ij_e, const float *tvecs
     return CF_OK;
 }
 
-extern "C" int cf_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs_u, int64_t U, int64_t N, int64_t H,
-                                     int64_t E, int64_t K, int64_t D, double dist_max, double wscale,
-                                     const float *W_k, const void *rings, float *z_ek, float *v_ekd, void *stream)
+extern "C" int64_t cf_real_enc_flag_bytes(int64_t U, int64_t H)
+{
+    if (U < 0 || H < 1) return 0;
+    return ((H + 7) / 8) * U + cf::real_enc_round_count(U, H);
+}
+
+extern "C" int cf_real_enc_fwd_rings(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                                     const int64_t *batch_i, const int64_t *edge_ij_e, const int64_t *pairs_u,
+                                     int64_t U, int64_t N, int64_t H, int64_t E, int64_t K, int64_t D,
+                                     double dist_max, double wscale, const float *W_k, const float *rvlen_n,
+                                     double cutoff_radius, int lattice_range, int minimum_range,
+                                     const void *rings, void *flags, int64_t flag_bytes, float *z_ek,
+                                     float *v_ekd, void *stream)
 {
     CF_REQUIRE(N >= 0 && E >= 0 && U >= 0, CF_ERR_INVALID_ARGUMENT, "cf_real_enc_fwd_rings: negative size");
     CF_REQUIRE(H == 1 || H == 2 || H == 4 || H == 8 || H == 16, CF_ERR_UNSUPPORTED,
@@ -495,11 +607,44 @@ extern "C" int cf_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs_u, 
                "cf_real_enc_fwd_rings: null pointer");
     CF_REQUIRE(K >= 1 && K <= 128 && D >= 1 && D <= 32 && dist_max > 0 && wscale > 0, CF_ERR_UNSUPPORTED,
                "cf_real_enc_fwd_rings: needs 1 <= K <= 128, 1 <= D <= 32");
+    const int edge = 2 * lattice_range + 1;
+    CF_REQUIRE(lattice_range >= 0 && edge * edge * edge <= RC, CF_ERR_UNSUPPORTED,
+               "cf_real_enc_fwd_rings: lattice_range %d outside what the rings hold", lattice_range);
     float bin_step, s_scale;
     bin_scales(K, dist_max, wscale, bin_step, s_scale);
-    int rc = cf::launch_real_enc_fwd_rings(a_ik, pairs_u, U, N, H, E, K, D, bin_step, s_scale, W_k,
-                                           (const float *)rings, z_ek, v_ekd, (hipStream_t)stream);
+    hipStream_t st = (hipStream_t)stream;
+    const float cutoff = rvlen_n ? (float)cutoff_radius : 0.0f;
+    if (cutoff == 0.0f) {
+        int rc = cf::launch_real_enc_fwd_rings(a_ik, pairs_u, U, N, H, E, K, D, bin_step, s_scale, W_k,
+                                               (const float *)rings, nullptr, nullptr, z_ek, v_ekd, st);
+        CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported shape");
+        CF_CHECK_LAUNCH("cf_real_enc_fwd_rings");
+        return CF_OK;
+    }
+    // Adaptive boxes: the units whose columns all keep the cube from the rings, the rest by the
+    // pair kernel; both write their own edges of z and v.
+    CF_REQUIRE(minimum_range >= 0 && minimum_range <= MAX_RANGE, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_fwd_rings: minimum_range %d outside 0..%d", minimum_range, MAX_RANGE);
+    CF_REQUIRE(rpos_ij_e && tvecs_n && batch_i && edge_ij_e, CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_fwd_rings: adaptive boxes need rpos_ij_e, tvecs_n, batch_i and edge_ij_e");
+    CF_REQUIRE(flags && flag_bytes >= cf_real_enc_flag_bytes(U, H), CF_ERR_INVALID_ARGUMENT,
+               "cf_real_enc_fwd_rings: adaptive boxes need %lld bytes of flags, %lld given",
+               (long long)cf_real_enc_flag_bytes(U, H), (long long)flag_bytes);
+    unsigned char *unit_flags = (unsigned char *)flags;
+    unsigned char *round_flags = unit_flags + ((H + 7) / 8) * U;
+    int rc = cf::launch_unit_floor(a_ik, rvlen_n, pairs_u, U, N, H, cutoff, lattice_range, minimum_range, unit_flags,
+                                   round_flags, st);
+    CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported size");
+    // (Tried: the pair kernel's launch on a second stream between two events, beside the ring
+    // launch.  The fork and join cost more than the overlap wins, eagerly and in a captured graph:
+    // 62.5 against 60.4 us per block, 0.31 against 0.26 ms per step with four forwards in flight.)
+    rc = cf::launch_real_enc_fwd_rings(a_ik, pairs_u, U, N, H, E, K, D, bin_step, s_scale, W_k, (const float *)rings,
+                                       unit_flags, round_flags, z_ek, v_ekd, st);
     CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported shape");
-    CF_CHECK_LAUNCH("cf_real_enc_fwd_rings");
+    rc = cf::launch_real_enc_fwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, N, H, E, K, D,
+                                       bin_step, s_scale, W_k, 1, rvlen_n, cutoff, lattice_range, minimum_range,
+                                       nullptr, unit_flags, round_flags, z_ek, v_ekd, st);
+    CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported shape");
+    CF_CHECK_LAUNCH("cf_real_enc_fwd_rings (adaptive boxes)");
     return CF_OK;
 }

@@ -161,12 +161,17 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         pairs_u = _pairs(batch_i, edge_ij_e, tvecs_n, K)
         rings = None
         fixed_cube = rvlen_n is None or cutoff_radius is None or float(cutoff_radius) == 0.0
+        # (adaptive boxes too: atom pairs whose half-widths all come out as LATTICE_RANGE have exactly
+        # the cube and start from the rings, the others are staged by the pair kernel)
         if (KernelManager.STAGED_RINGS and KernelManager.WEAKEST_EXPONENT is not None and pairs_u is not None
-                and fixed_cube and K > 0 and W_k is not None and _w_leading(W_k) == 1 and W_k.shape[-2] <= 32):
+                and K > 0 and W_k is not None and _w_leading(W_k) == 1 and W_k.shape[-2] <= 32):
             rings = ops.staged_rings(rpos_ij_e, tvecs_n, pairs_u, K, dist_max, wscale, KernelManager.LATTICE_RANGE,
                                      KernelManager.WEAKEST_EXPONENT)
         if rings is not None:
-            z_ek, v_ekd = ops.real_enc_fwd_rings(a_ik, edge_ij_e, pairs_u, rings, K, dist_max, wscale, W_k)
+            z_ek, v_ekd = ops.real_enc_fwd_rings(
+                a_ik, edge_ij_e, pairs_u, rings, K, dist_max, wscale, W_k, KernelManager.LATTICE_RANGE,
+                rpos_ij_e, tvecs_n, batch_i, None if fixed_cube else rvlen_n, None if fixed_cube else cutoff_radius,
+                KernelManager.MINIMUM_RANGE)
         else:
             z_ek, v_ekd = ops.real_enc_fwd(
                 a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, W_k, rvlen_n,
@@ -176,7 +181,7 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         ctx.ranges = (KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
         ctx.adaptive_args = rvlen_n is not None
         # the backward's pair kernel (K <= 64, D <= 16) starts from the same staged translations
-        ctx.rings = rings if (rings is not None and K <= 64 and W_k.shape[-2] <= 16) else None
+        ctx.rings = rings if (rings is not None and fixed_cube and K <= 64 and W_k.shape[-2] <= 16) else None
         if K <= 0:
             return (z_ek,)
         return z_ek, v_ekd

@@ -35,8 +35,9 @@ SIGNATURES = {
                                                          _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
     "cf_real_enc_ring_bytes": (_i64, [_i64]),
     "cf_real_enc_ring_stage": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _dbl, _dbl, _int, _dbl, _ptr, _ptr]),
-    "cf_real_enc_fwd_rings": (_int, [_ptr, _ptr, _i64, _i64, _i64, _i64, _i64, _i64, _dbl, _dbl, _ptr, _ptr, _ptr,
-                                     _ptr, _ptr]),
+    "cf_real_enc_flag_bytes": (_i64, [_i64, _i64]),
+    "cf_real_enc_fwd_rings": (_int, [_ptr] * 6 + [_i64] * 6 + [_dbl, _dbl, _ptr, _ptr, _dbl, _int, _int, _ptr, _ptr,
+                                                               _i64, _ptr, _ptr, _ptr]),
     "cf_real_enc_bwd_workspace": (_i64, [_i64] * 6 + [_int]),
     "cf_real_enc_bwd": (_int, [_ptr] * 9 + [_i64] * 6 + [_dbl, _dbl, _ptr, _i64, _ptr, _dbl, _int, _int,
                                                          _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),

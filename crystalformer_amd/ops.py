@@ -271,35 +271,55 @@ def staged_rings(rpos_ij_e: Tensor, tvecs_n: Tensor, pairs_u: Tensor, K: int, di
 
 
 def real_enc_fwd_rings(a_ik: Tensor, edge_ij_e: Tensor, pairs_u: Tensor, rings: Tensor, K: int, dist_max: float,
-                       wscale: float, W_k: Tensor) -> Tuple[Tensor, Tensor]:
-    """:func:`real_enc_fwd` for a shared projection and the fixed cube, from the staged rings."""
-    dev = require_device(a_ik, edge_ij_e, pairs_u, rings, W_k)
+                       wscale: float, W_k: Tensor, lattice_range: int = 2, rpos_ij_e: Optional[Tensor] = None,
+                       tvecs_n: Optional[Tensor] = None, batch_i: Optional[Tensor] = None,
+                       rvlen_n: Optional[Tensor] = None, cutoff_radius: Optional[float] = None,
+                       minimum_range: int = 0) -> Tuple[Tensor, Tensor]:
+    """:func:`real_enc_fwd` for a shared projection from the staged rings (``lattice_range`` the one
+    they were staged for).  Fixed cube: every atom pair starts from its ring.  Adaptive boxes
+    (``rvlen_n`` and a non-zero ``cutoff_radius``; needs ``rpos_ij_e``, ``tvecs_n`` and ``batch_i`` too):
+    the pairs whose half-widths all come out as ``lattice_range`` start from their rings, the others are
+    staged by the pair kernel in a second launch."""
+    dev = require_device(a_ik, edge_ij_e, pairs_u, rings, W_k, rpos_ij_e, tvecs_n, batch_i, rvlen_n)
     a_ik, W_k = _f32(a_ik, "a_ik"), _f32(W_k, "W_k")
-    pairs_u = _i64(pairs_u, "pairs_u")
+    pairs_u, edge_ij_e = _i64(pairs_u, "pairs_u"), _i64(edge_ij_e, "edge_ij_e")
     N, H = a_ik.shape
     E = edge_ij_e.shape[1]
+    U = pairs_u.shape[0]
     W_num, D = _w_shape(W_k, H, int(K))
+    L = _lib.load()
     if W_num != 1:
         raise _lib.CrystalformerHipError("real_enc_fwd_rings: one projection per head only")
-    if rings.dtype != torch.float32 or rings.numel() * 4 < int(_lib.load().cf_real_enc_ring_bytes(pairs_u.shape[0])):
+    if rings.dtype != torch.float32 or rings.numel() * 4 < int(L.cf_real_enc_ring_bytes(U)):
         raise _lib.CrystalformerHipError("real_enc_fwd_rings: rings buffer too small for this pair list")
+    cutoff = 0.0 if (cutoff_radius is None or rvlen_n is None) else float(cutoff_radius)
+    flags, flag_bytes = None, 0
+    if cutoff != 0.0:
+        if rpos_ij_e is None or tvecs_n is None or batch_i is None:
+            raise _lib.CrystalformerHipError("real_enc_fwd_rings: adaptive boxes need rpos_ij_e, tvecs_n and batch_i")
+        rpos_ij_e, tvecs_n, rvlen_n = _f32(rpos_ij_e, "rpos_ij_e"), _f32(tvecs_n, "tvecs_n"), _f32(rvlen_n, "rvlen_n")
+        batch_i = _i64(batch_i, "batch_i")
+        if rpos_ij_e.shape != (E, 3) or batch_i.shape != (N,) or rvlen_n.shape != (tvecs_n.shape[0], 3):
+            raise _lib.CrystalformerHipError("real_enc_fwd_rings: inconsistent input shapes")
+        flag_bytes = int(L.cf_real_enc_flag_bytes(U, H))
+        flags = torch.empty(max(flag_bytes, 1), dtype=torch.uint8, device=dev)
     z = torch.empty((E, H), dtype=torch.float32, device=dev)
     v = torch.empty((E, H, D), dtype=torch.float32, device=dev)
     if _eval_counter is not None:
-        _eval_counter.append(float(E) * (2 * _ring_lattice_range(rings, pairs_u) + 1) ** 3)
+        if cutoff == 0.0:
+            _eval_counter.append(float(E) * (2 * int(lattice_range) + 1) ** 3)
+        else:
+            _eval_counter.append(count_translation_evals(a_ik, rvlen_n, batch_i, edge_ij_e, cutoff, int(lattice_range),
+                                                         int(minimum_range)))
     with device_guard(dev), _timed("real_enc_fwd", E=E, H=H, K=K, D=D, proj=True):
-        rc = _lib.load().cf_real_enc_fwd_rings(ptr(a_ik), ptr(pairs_u), pairs_u.shape[0], N, H, E, int(K), D,
-                                               float(dist_max), float(wscale), ptr(W_k), ptr(rings), ptr(z), ptr(v),
-                                               stream_handle(dev))
+        rc = L.cf_real_enc_fwd_rings(
+            ptr(a_ik), ptr(rpos_ij_e if cutoff != 0.0 else None), ptr(tvecs_n if cutoff != 0.0 else None),
+            ptr(batch_i if cutoff != 0.0 else None), ptr(edge_ij_e), ptr(pairs_u), U, N, H, E, int(K), D,
+            float(dist_max), float(wscale), ptr(W_k), ptr(rvlen_n if cutoff != 0.0 else None), cutoff,
+            int(lattice_range), int(minimum_range), ptr(rings), ptr(flags), flag_bytes, ptr(z), ptr(v),
+            stream_handle(dev))
     check(rc, "cf_real_enc_fwd_rings")
     return z, v
-
-
-def _ring_lattice_range(rings: Tensor, pairs_u: Tensor) -> int:
-    for entry in _ring_cache:
-        if entry[2] is rings:
-            return entry[0][-2]
-    return 2
 
 
 def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor,

@@ -116,14 +116,25 @@ int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvec
  *                     -gauss_lb / (2 r0^2): translations that reach no bin are kept only if
  *                     exp(weakest_exponent (d^2 - d^2_min)) > 2^-40.  Exponents above the bound
  *                     make the lattice sums drop terms they should hold; 0 keeps every translation.
+ * Adaptive boxes (rvlen_n given and cutoff_radius != 0, the rule of
+ * models/kernels/real_enc_fwd.cu:58-85): atom pairs whose (atom, head) half-widths all come out as
+ * lattice_range have exactly the cube and are evaluated from the rings; the others are staged and
+ * evaluated as cf_real_enc_fwd does.  Three launches (selection, rings, rest) that share `flags`,
+ * cf_real_enc_flag_bytes(U, H) bytes of device scratch written and read by the call.  With the fixed
+ * cube rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n and flags may be NULL.
  */
 int64_t cf_real_enc_ring_bytes(int64_t U);
+int64_t cf_real_enc_flag_bytes(int64_t U, int64_t H);
 int cf_real_enc_ring_stage(const float *rpos_ij_e, const float *tvecs_n, const int64_t *pairs_u, int64_t U,
                            int64_t K, double dist_max, double wscale, int lattice_range,
                            double weakest_exponent, void *rings, void *stream);
-int cf_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs_u, int64_t U, int64_t N, int64_t H,
-                          int64_t E, int64_t K, int64_t D, double dist_max, double wscale,
-                          const float *W_k, const void *rings, float *z_ek, float *v_ekd, void *stream);
+int cf_real_enc_fwd_rings(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
+                          const int64_t *batch_i, const int64_t *edge_ij_e, const int64_t *pairs_u,
+                          int64_t U, int64_t N, int64_t H, int64_t E, int64_t K, int64_t D,
+                          double dist_max, double wscale, const float *W_k, const float *rvlen_n,
+                          double cutoff_radius, int lattice_range, int minimum_range,
+                          const void *rings, void *flags, int64_t flag_bytes, float *z_ek,
+                          float *v_ekd, void *stream);
 /*
  * cf_real_enc_bwd (below; same arguments, workspace and results) for the fixed cube and one
  * projection per head, with the rings staged for this geometry, pair list, bin grid and

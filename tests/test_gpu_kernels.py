@@ -1194,14 +1194,14 @@ def test_real_enc_fwd_from_staged_rings(dev, H, K, D, lr):
     rpos, tv, pairs, rings = _staged(dev, p, K, lr)
     assert rings is not None and rings.numel() * 4 == lib.load().cf_real_enc_ring_bytes(pairs.shape[0])
     a, ed, W = to_dev(dev, p.a, p.edges, p.W)
-    z, v = ops.real_enc_fwd_rings(a, ed, pairs, rings, K, p.dist_max, p.wscale, W)
+    z, v = ops.real_enc_fwd_rings(a, ed, pairs, rings, K, p.dist_max, p.wscale, W, lr)
     assert_close(z, z_ref, "z")
     assert_close(v, v_ref, "v", atol=v_atol(p, K, p.W, 0.0, lr, 0))
     # the same geometry again: the staged buffer is found, not rebuilt
     assert ops.staged_rings(rpos, tv, pairs, K, p.dist_max, p.wscale, lr, float(p.a.max())) is rings
     # a weaker bound on the exponents keeps more far translations: same result to the last bits
     _, _, _, rings0 = _staged(dev, p, K, lr, weakest=0.0)
-    z0, v0 = ops.real_enc_fwd_rings(a, ed, pairs, rings0, K, p.dist_max, p.wscale, W)
+    z0, v0 = ops.real_enc_fwd_rings(a, ed, pairs, rings0, K, p.dist_max, p.wscale, W, lr)
     assert rel_err(z0, z) < 1e-6 and rel_err(v0, v) < 1e-6
 
 
@@ -1277,3 +1277,36 @@ def test_staged_rings_limits(dev):
     with_rings = ops.real_enc_bwd(*args, gv32, 64, p.dist_max, p.wscale, W32, None, 0.0, 2, 0, pairs_u=pairs, rings=rings)
     without = ops.real_enc_bwd(*args, gv32, 64, p.dist_max, p.wscale, W32, None, 0.0, 2, 0, pairs_u=pairs)
     assert torch.equal(with_rings[0], without[0]) and torch.equal(with_rings[1], without[1])
+
+
+@pytest.mark.parametrize("cutoff,lr,mr", [(-3.5, 2, 2), (-3.5, 1, 1), (-2.0, 2, 2), (5.0, 1, 1), (-3.5, 2, 0)])
+@pytest.mark.parametrize("H,K,D", [(8, 64, 16), (4, 16, 8), (16, 32, 8), (2, 100, 4), (8, 64, 32)])
+def test_real_enc_fwd_from_staged_rings_with_adaptive_boxes(dev, H, K, D, cutoff, lr, mr):
+    """Adaptive boxes in two launches: atom pairs whose half-widths all come out as lattice_range start from
+    the staged rings, the others are staged by the pair kernel.  Against the oracle and against the pair
+    kernel alone; the problems hold pairs of both kinds."""
+    p = Problem([1, 3, 9, 2, 17, 1, 6], H=H, K=K, D=D, seed=41)
+    z_ref, v_ref = enc_fwd_ref(p, K, p.W, cutoff, lr, mr)
+    rpos, tv, pairs, rings = _staged(dev, p, K, lr)
+    a, bt, ed, W, rv = to_dev(dev, p.a, p.b.batch, p.edges, p.W, p.rvlen)
+    z, v = ops.real_enc_fwd_rings(a, ed, pairs, rings, K, p.dist_max, p.wscale, W, lr, rpos, tv, bt, rv, cutoff, mr)
+    assert_close(z, z_ref, "z")
+    assert_close(v, v_ref, "v", atol=v_atol(p, K, p.W, cutoff, lr, mr))
+    z1, v1 = ops.real_enc_fwd(a, rpos, tv, bt, ed, K, p.dist_max, p.wscale, W, rv, cutoff, lr, mr, pairs_u=pairs)
+    assert rel_err(z, z1) < 1e-6 and rel_err(v, v1) < 1e-6
+    # how the pairs split (the rule's integers are bit-exact on the device)
+    R = ops.translation_ranges(a, rv, bt, cutoff, lr, mr)
+    at_floor = (R == lr).all(-1).all(-1)
+    both = at_floor[pairs[:, 2]] & at_floor[pairs[:, 3]]
+    print("pairs from the rings:", int(both.sum()), "of", both.numel())
+
+
+def test_adaptive_boxes_split_covers_both_kinds(dev):
+    """The problems of the test above do hold atom pairs of both kinds for the default rule."""
+    p = Problem([1, 3, 9, 2, 17, 1, 6], H=8, K=64, D=16, seed=41)
+    a, bt, rv = to_dev(dev, p.a, p.b.batch, p.rvlen)
+    pairs = ops.edge_pairs(p.b.sizes.to(dev))
+    R = ops.translation_ranges(a, rv, bt, -3.5, 2, 2)
+    at_floor = (R == 2).all(-1).all(-1)
+    both = at_floor[pairs[:, 2]] & at_floor[pairs[:, 3]]
+    assert 0 < int(both.sum()) < both.numel()
