@@ -32,7 +32,7 @@ PEAK_FP32_TFLOPS = 157.3          # fp32 on the matrix cores (and packed vector 
 PEAK_FP32_VALU_TFLOPS = 78.6      # one fp32 FMA per lane and cycle: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz x 2
 PEAK_HBM_GBS = 8000.0
 PROFILE_FILE = os.path.join(ROOT, "profiles", "traffic.json")
-KERNEL_SOURCES = {"fwd": ("real_enc_ring.hip", "real_enc_mfma.hip", "real_enc_pair.h", "cf_common.h"),
+KERNEL_SOURCES = {"fwd": ("real_enc_ring.hip", "real_enc_mfma.hip", "real_enc_pair_fwd.h", "real_enc_pair.h", "cf_common.h"),
                   "bwd": ("real_enc_mfma_bwd.hip", "real_enc_pair.h", "cf_common.h")}
 
 

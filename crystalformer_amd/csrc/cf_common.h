@@ -52,6 +52,12 @@ int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U
                               const float *cache, const unsigned char *unit_flags, const unsigned char *round_flags,
                               float *z, float *v, hipStream_t st);
 int64_t real_enc_round_count(int64_t U, int64_t H);
+int launch_real_enc_fwd_two_role(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,
+                                 const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
+                                 int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
+                                 const float *rvlen, float cutoff, int lattice_range, int min_range,
+                                 const float *cache, const unsigned char *unit_flags,
+                                 const unsigned char *round_flags, float *z, float *v, hipStream_t st);
 int launch_unit_floor(const float *a_ik, const float *rvlen, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
                       float cutoff, int lattice_range, int min_range, unsigned char *unit_flags,
                       unsigned char *round_flags, hipStream_t st);

@@ -16,7 +16,7 @@
 // records occupy slots RS-1 downwards followed (below) by 4 neutral records.  (Keeping d2 alone and
 // recomputing s and the bits in every launch makes the image three times smaller and the staging
 // faster, but costs each launch 5% more instructions: 46.4 against 43.8 us on 128 crystals.)
-#include "real_enc_pair.h"
+#include "real_enc_pair_fwd.h"
 
 namespace {
 
@@ -203,7 +203,8 @@ __global__ __launch_bounds__(256) void unit_floor_kernel(PairArgs p, unsigned ch
 // SELECT: only the units picked by p.unit_flags / p.flag_want are evaluated, and only the rounds
 // that hold one are walked (p.round_flags).
 template <int NT, int DT, bool SELECT>
-__global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, const float *__restrict__ cache)
+__device__ __forceinline__ void real_enc_fwd_ring_body(const PairArgs &p, const float *__restrict__ cache,
+                                                       const int block_id, const int grid_size)
 {
     extern __shared__ __align__(16) float lds[];
     const int lane = threadIdx.x & 63;
@@ -228,7 +229,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
 
     const int rounds_per_hg = (int)((p.U + WPB - 1) / WPB);
     const int rounds = rounds_per_hg * p.head_groups;
-    const int stride = gridDim.x;
+    const int stride = grid_size;
     auto unit_of = [&](int rd_, const RoundPos &rp) -> int64_t {
         const int64_t u_ = (int64_t)rp.r * WPB + wave;
         return (rd_ < rounds && u_ < p.U) ? u_ : 0;
@@ -240,16 +241,16 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
     using Image = RingImage;
     auto load_image = [&](int64_t u_) -> Image { return load_ring_image(cache, u_, lane); };
 
-    // rounds of this work-group: blockIdx.x, + grid, + 2 grid, ...; with SELECT those of them that
+    // rounds of this work-group: block_id, + grid, + 2 grid, ...; with SELECT those of them that
     // hold a unit of this launch, known three rounds ahead
     int rd, rd_next, rd_next2;
     if (SELECT) {
-        const RoundSeq seq = first_active_rounds(p, blockIdx.x, rounds, stride, lane);
+        const RoundSeq seq = first_active_rounds(p, block_id, rounds, stride, lane);
         rd = seq.rd[0];
         rd_next = seq.rd[1];
         rd_next2 = seq.rd[2];
     } else {
-        rd = blockIdx.x;
+        rd = block_id;
         rd_next = rd + stride;
         rd_next2 = rd + 2 * stride;
     }
@@ -446,6 +447,29 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, c
     }
 }
 
+template <int NT, int DT, bool SELECT>
+__global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, const float *__restrict__ cache)
+{
+    real_enc_fwd_ring_body<NT, DT, SELECT>(p, cache, (int)blockIdx.x, (int)gridDim.x);
+}
+
+// Adaptive boxes in one launch: the first pair_blocks work-groups run the pair kernel's body over the
+// rounds that hold an atom pair which does not keep the cube (few, long rounds; a work-group
+// without such a round leaves at once and frees its place), the others the ring body over the
+// rounds that hold one which does.  Two independent sets of work-groups, each with its own
+// numbering; they write different edges.
+template <int NT, int DT>
+__global__ __launch_bounds__(512, 4) void real_enc_fwd_two_role_kernel(PairArgs p_ring, PairArgs p_pair,
+                                                                       const float *__restrict__ cache,
+                                                                       int pair_blocks)
+{
+    if ((int)blockIdx.x < pair_blocks)
+        real_enc_fwd_pair_body<NT, false, PROJ_SHARED, DT, false>(p_pair, (int)blockIdx.x, pair_blocks);
+    else
+        real_enc_fwd_ring_body<NT, DT, true>(p_ring, cache, (int)blockIdx.x - pair_blocks,
+                                             (int)gridDim.x - pair_blocks);
+}
+
 }  // namespace
 
 namespace cf {
@@ -497,6 +521,58 @@ int launch_unit_floor(const float *a_ik, const float *rvlen, const int64_t *pair
     if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;
     if (rounds < 1) return CF_OK;
     unit_floor_kernel<<<(int)((rounds + 3) / 4), 256, 0, st>>>(p, unit_flags, round_flags);
+    return CF_OK;
+}
+
+// Adaptive boxes, one launch for both kinds of atom pairs (real_enc_fwd_two_role_kernel).
+int launch_real_enc_fwd_two_role(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,
+                                 const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
+                                 int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
+                                 const float *rvlen, float cutoff, int lattice_range, int min_range,
+                                 const float *cache, const unsigned char *unit_flags,
+                                 const unsigned char *round_flags, float *z, float *v, hipStream_t st)
+{
+    if (K < 1 || K > 128 || !W || D < 1 || D > 32 || cutoff == 0.0f || !unit_flags || !round_flags)
+        return CF_ERR_UNSUPPORTED;
+    if (E * H >= (1ll << 32) || N * H >= (1ll << 32)) return CF_ERR_UNSUPPORTED;      // 32-bit rows in the ring body
+    PairArgs pp{};
+    pp.a_ik = a_ik; pp.rpos = rpos; pp.tvecs = tvecs; pp.batch = batch; pp.edges = edges; pp.pairs = pairs;
+    pp.W = W; pp.rvlen = rvlen; pp.z = z; pp.v = v; pp.sched = nullptr;
+    pp.N = N; pp.E = E; pp.U = U; pp.W_num = 1;
+    pp.H = (int)H; pp.K = (int)K; pp.D = (int)D;
+    pp.head_groups = (int)((H + 7) / 8);
+    pp.cutoff = cutoff; pp.lattice_range = lattice_range; pp.min_range = min_range;
+    pp.bin_step = bin_step; pp.s_scale = s_scale; pp.inv_bin_step = 1.0f / bin_step;
+    pp.window = sqrtf(40.0f) / bin_step;
+    pp.unit_flags = unit_flags; pp.round_flags = round_flags; pp.flag_want = 0;       // pairs that leave the cube
+    PairArgs pr = pp;                                                                   // pairs that keep it
+    pr.rpos = nullptr; pr.tvecs = nullptr; pr.batch = nullptr; pr.edges = nullptr; pr.rvlen = nullptr;
+    pr.cutoff = 0.f; pr.flag_want = 1;
+    const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
+    const int DT = D > 16 ? 2 : 1;
+    const size_t shared_proj = sizeof(float) * ((size_t)4 * NT * XPLANE + WPB * 16) + sizeof(int64_t) * WPB * 2 + 8;
+    const size_t lds_ring = sizeof(float) * (size_t)WPB * 3 * RS + shared_proj;
+    const size_t lds_pair = sizeof(float) * (size_t)WPB * 3 * (RING_CAP + 16) + shared_proj;
+    const size_t lds = lds_ring > lds_pair ? lds_ring : lds_pair;
+    const int64_t rounds = ((U + WPB - 1) / WPB) * pp.head_groups;
+    if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;
+    if (rounds < 1) return CF_OK;
+    const int64_t cap = persistent_grid_cap(2);
+    const int64_t ring_blocks = rounds < cap ? rounds : cap;
+    int64_t pair_blocks = cap / 8 < 1 ? 1 : cap / 8;       // few long rounds: an eighth of the places, freed at once where idle
+    if (pair_blocks > rounds) pair_blocks = rounds;
+    const int grid = (int)(ring_blocks + pair_blocks);
+#define CF_TWO(NTV, DTV) \
+    real_enc_fwd_two_role_kernel<NTV, DTV><<<grid, WPB * WAVE, lds, st>>>(pr, pp, cache, (int)pair_blocks)
+#define CF_TWO_NT(NTV) do { if (DT == 1) CF_TWO(NTV, 1); else CF_TWO(NTV, 2); } while (0)
+    switch (NT) {
+        case 1: CF_TWO_NT(1); break;
+        case 2: CF_TWO_NT(2); break;
+        case 4: CF_TWO_NT(4); break;
+        default: CF_TWO_NT(8); break;
+    }
+#undef CF_TWO_NT
+#undef CF_TWO
     return CF_OK;
 }
 
@@ -635,15 +711,14 @@ extern "C" int cf_real_enc_fwd_rings(const float *a_ik, const float *rpos_ij_e, 
     int rc = cf::launch_unit_floor(a_ik, rvlen_n, pairs_u, U, N, H, cutoff, lattice_range, minimum_range, unit_flags,
                                    round_flags, st);
     CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported size");
-    // (Tried: the pair kernel's launch on a second stream between two events, beside the ring
-    // launch.  The fork and join cost more than the overlap wins, eagerly and in a captured graph:
-    // 62.5 against 60.4 us per block, 0.31 against 0.26 ms per step with four forwards in flight.)
-    rc = cf::launch_real_enc_fwd_rings(a_ik, pairs_u, U, N, H, E, K, D, bin_step, s_scale, W_k, (const float *)rings,
-                                       unit_flags, round_flags, z_ek, v_ekd, st);
-    CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported shape");
-    rc = cf::launch_real_enc_fwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, N, H, E, K, D,
-                                       bin_step, s_scale, W_k, 1, rvlen_n, cutoff, lattice_range, minimum_range,
-                                       nullptr, unit_flags, round_flags, z_ek, v_ekd, st);
+    // One launch for both kinds of atom pairs.  (Tried before: the two kernels one after the other,
+    // 60.4 us per block at 128 crystals, the pair kernel's part being one long round of a few
+    // work-groups; and that launch on a second stream between two events beside the ring launch, where
+    // fork and join cost more than the overlap won, 62.5 us and 0.31 against 0.26 ms per step with
+    // four forwards in flight.)
+    rc = cf::launch_real_enc_fwd_two_role(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, N, H, E, K, D,
+                                          bin_step, s_scale, W_k, rvlen_n, cutoff, lattice_range, minimum_range,
+                                          (const float *)rings, unit_flags, round_flags, z_ek, v_ekd, st);
     CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported shape");
     CF_CHECK_LAUNCH("cf_real_enc_fwd_rings (adaptive boxes)");
     return CF_OK;
