@@ -392,6 +392,8 @@ def main() -> int:
     ap.add_argument("--no-staged-rings", action="store_true",
                     help="every block stages its translations itself (pair kernel) instead of starting from the "
                          "rings staged once per forward")
+    ap.add_argument("--adaptive-rings", action="store_true",
+                    help="with --rule B: atom pairs that keep the cube start from the staged rings (off by default)")
     ap.add_argument("--no-fresh", action="store_true", help="skip the fresh-batch (layout rebuilt every step) figure")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--train", action="store_true",
@@ -437,6 +439,8 @@ def main() -> int:
         hip_funcs.KernelManager.FUSE_ENCODING_ATTENTION = False
     if args.no_staged_rings:
         hip_funcs.KernelManager.STAGED_RINGS = False
+    if args.adaptive_rings:
+        hip_funcs.KernelManager.ADAPTIVE_RINGS = True
     dev = torch.device("cuda:0")
     if args.train and args.config == "cfg2_default_b128":
         args.config = "cfg4_train_b128"

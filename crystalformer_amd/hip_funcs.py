@@ -83,8 +83,12 @@ class KernelManager:
     # attention module sets around its call (-gauss_lb / (2 r0^2)); None: every launch stages for itself.
     STAGED_RINGS: bool = True
     WEAKEST_EXPONENT: Optional[float] = None
-    # adaptive boxes, eager launches: atom pairs from which the staged rings are used (see the encoding Function)
-    ADAPTIVE_RINGS_MIN_PAIRS = 60000
+    # Adaptive boxes from the staged rings (forward): atom pairs whose half-widths all come out as
+    # LATTICE_RANGE start from their rings, the others are staged by the pair kernel's body in the same
+    # launch.  Off by default: it pays where nearly all pairs keep the cube (default model, inference, 128
+    # crystals: 0.426 against 0.471 ms per forward) and costs where many do not (the split of the
+    # work-groups between the two kinds is fixed, and a round that holds both kinds is walked twice).
+    ADAPTIVE_RINGS = False
     compiled: bool = False
 
 
@@ -165,10 +169,8 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         fixed_cube = rvlen_n is None or cutoff_radius is None or float(cutoff_radius) == 0.0
         # (adaptive boxes too: atom pairs whose half-widths all come out as LATTICE_RANGE have exactly
         # the cube and start from the rings, the others are staged by the pair kernel)
-        # (three launches instead of one: taken where launches are cheap or the kernels dominate, i.e. under
-        # stream capture and for large batches; an eager forward over a small batch is bound by its launches)
-        worth_it = fixed_cube or pairs_u is None or pairs_u.shape[0] >= KernelManager.ADAPTIVE_RINGS_MIN_PAIRS \
-            or (a_ik.is_cuda and torch.cuda.is_current_stream_capturing())
+        # (adaptive boxes: on request only, see KernelManager.ADAPTIVE_RINGS)
+        worth_it = fixed_cube or KernelManager.ADAPTIVE_RINGS
         if (KernelManager.STAGED_RINGS and KernelManager.WEAKEST_EXPONENT is not None and pairs_u is not None
                 and worth_it and K > 0 and W_k is not None and _w_leading(W_k) == 1 and W_k.shape[-2] <= 32):
             rings = ops.staged_rings(rpos_ij_e, tvecs_n, pairs_u, K, dist_max, wscale, KernelManager.LATTICE_RANGE,

@@ -750,21 +750,19 @@ def test_blocks_share_one_staging_of_the_translations(dev):
         torch.cuda.synchronize()
 
 
-def test_adaptive_boxes_take_the_staged_rings_where_pairs_keep_the_cube(dev):
-    """The reference kernels' default rule (adaptive boxes, floor at lattice_range): with the staged rings the
-    forward runs as selection + rings + pair kernel on the rest; outputs and gradients equal those of the pair
-    kernel alone.  Eager launches over a small batch keep the single launch (ADAPTIVE_RINGS_MIN_PAIRS)."""
+def test_adaptive_boxes_take_the_staged_rings_on_request(dev):
+    """The reference kernels' default rule (adaptive boxes, floor at lattice_range): with ADAPTIVE_RINGS the
+    forward runs as selection + one launch in which the pairs that keep the cube start from the staged rings and
+    the others are staged; outputs and gradients equal those of the pair kernel alone.  Off by default."""
     name = "cfg2_default_b128"
     b = select_crystals(make_config_batch(name), range(40)).to(dev)
     cfg, model = build_model(name)                     # adaptive_cutoff_sigma = -3.5, minimum_range on
-    assert cfg.adaptive_cutoff_sigma < 0
+    assert cfg.adaptive_cutoff_sigma < 0 and not hip_funcs.KernelManager.ADAPTIVE_RINGS
     model.to(dev).train()
     model(b)                                           # first training pass: stores the batch statistics
 
-    def step(min_pairs, staged=True):
-        old = hip_funcs.KernelManager.ADAPTIVE_RINGS_MIN_PAIRS
-        hip_funcs.KernelManager.ADAPTIVE_RINGS_MIN_PAIRS = min_pairs
-        hip_funcs.KernelManager.STAGED_RINGS = staged
+    def step(adaptive_rings):
+        hip_funcs.KernelManager.ADAPTIVE_RINGS = adaptive_rings
         try:
             model.zero_grad(set_to_none=True)
             log = []
@@ -774,14 +772,11 @@ def test_adaptive_boxes_take_the_staged_rings_where_pairs_keep_the_cube(dev):
             return y.detach().clone(), {k: p.grad.clone() for k, p in model.named_parameters()
                                         if p.grad is not None}, [entry[0] for entry in log]
         finally:
-            hip_funcs.KernelManager.ADAPTIVE_RINGS_MIN_PAIRS = old
-            hip_funcs.KernelManager.STAGED_RINGS = True
+            hip_funcs.KernelManager.ADAPTIVE_RINGS = False
             ops.set_event_log(None)
-    y1, g1, names1 = step(0)
-    y0, g0, names0 = step(0, staged=False)
-    _, _, names_small = step(10 ** 9)
+    y1, g1, names1 = step(True)
+    y0, g0, names0 = step(False)
     assert names1.count("real_enc_ring_stage") == 1 and names0.count("real_enc_ring_stage") == 0
-    assert names_small.count("real_enc_ring_stage") == 0
     assert rel_err(y1, y0) < 1e-6
     for k in g1:
         assert rel_err(g1[k], g0[k]) < 1e-5, k
