@@ -157,6 +157,15 @@ __device__ __forceinline__ float row16_min(float v)
     return v;
 }
 
+__device__ __forceinline__ int row16_max_i(int v)
+{
+    v = max(v, dpp_i<DPP_QUAD_1032, 0xF>(v, v));
+    v = max(v, dpp_i<DPP_QUAD_2301, 0xF>(v, v));
+    v = max(v, dpp_i<DPP_ROW_ROR4, 0xF>(v, v));
+    v = max(v, dpp_i<DPP_ROW_ROR8, 0xF>(v, v));
+    return v;
+}
+
 __device__ __forceinline__ int wave_max_i(int v)
 {
     v = max(v, dpp_i<DPP_QUAD_1032, 0xF>(v, v));

@@ -35,7 +35,9 @@ using namespace cfpair;
 template <int NT, bool UNIFORM, int PROJ, int DT, bool SHORT_RING>
 __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
 {
-    real_enc_fwd_pair_body<NT, UNIFORM, PROJ, DT, SHORT_RING>(p, (int)blockIdx.x, (int)gridDim.x);
+    // (p is the kernel's first argument: it lies at the start of the kernel-argument segment)
+    const cfpair::PairArgsSeg seg = (cfpair::PairArgsSeg)__builtin_amdgcn_kernarg_segment_ptr();
+    real_enc_fwd_pair_body<NT, UNIFORM, PROJ, DT, SHORT_RING>(p, seg, (int)blockIdx.x, (int)gridDim.x);
 }
 
 // Unit descriptors: the (i <= j) edges of every crystal's dense block, their reverses,

@@ -16,6 +16,7 @@
 // that head's D x K block of gW, which stays in registers for the whole kernel
 // and is written once per work-group; a second kernel adds the per-work-group
 // blocks in a fixed order.  No atomics.
+#include <type_traits>
 #include "real_enc_pair.h"
 
 namespace {
@@ -170,7 +171,11 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         }
         // loads for the coming rounds, consumed just before this round's exchange
         float gv_next = 0.f;
-        if (!RINGS) gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
+        // (adaptive boxes: the lane parts of the once-a-round addresses are formed in the round, not
+        // kept in registers across the rounds)
+        int lane_r = lane, q_r = q, c_r = c;
+        if (!UNIFORM) asm volatile("" : "+v"(lane_r), "+v"(q_r), "+v"(c_r));
+        if (!RINGS) gv_next = load_unit_geom(ids_next, lane_r, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
         const float a_next = load_a(ids_next, pos_next);
         const float z_next = load_z(ids_next, pos_next);
         const int col_edge_next = load_col_edge(rd + stride, pos_next);
@@ -196,13 +201,14 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 
         BoxDims bx;
         bx.U1 = bx.U2 = bx.U3 = p.lattice_range;
-        int R1 = bx.U1, R2 = bx.U1, R3 = bx.U1;
+        // (lane (q, c) works out axis q of column c; the row maxima are the union box)
+        int Rq = 0, Uq = 0;
         if (!UNIFORM) {
-            range_rule(a, p.cutoff, geo.rvl, p.lattice_range, p.min_range, R1, R2, R3);
-            if (!col_on) R1 = R2 = R3 = 0;
-            bx.U1 = __builtin_amdgcn_readfirstlane(wave_max_int(R1));
-            bx.U2 = __builtin_amdgcn_readfirstlane(wave_max_int(R2));
-            bx.U3 = __builtin_amdgcn_readfirstlane(wave_max_int(R3));
+            Rq = column_axis_range(a, p.cutoff, geo.rvl, p.lattice_range, p.min_range, q, col_on);
+            Uq = row16_max_i(Rq);
+            bx.U1 = __builtin_amdgcn_readlane(Uq, 0);
+            bx.U2 = __builtin_amdgcn_readlane(Uq, 16);
+            bx.U3 = __builtin_amdgcn_readlane(Uq, 32);
         }
         bx.S3 = 2 * bx.U3 + 1;
         bx.S2 = 2 * bx.U2 + 1;
@@ -214,14 +220,17 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         // all active columns have the cube [-lattice_range, lattice_range]^3 (wave-uniform): under
         // the adaptive rule with its floor switched on that is most units, and they skip the
         // per-column box tables and lookups
-        bool cube = UNIFORM;
+        // ... and so do units whose active columns all have the same box, whatever it is: every
+        // translation of the union box then counts for every column
+        bool cube = UNIFORM, same_box = UNIFORM;
         if (!UNIFORM) {
             const int lr = p.lattice_range;
-            const bool other = col_on && (R1 != lr || R2 != lr || R3 != lr);
-            cube = bx.U1 == lr && bx.U2 == lr && bx.U3 == lr && __ballot(other) == 0ull;
+            const bool other = col_on && q < 3 && Rq != Uq;
+            same_box = __ballot(other) == 0ull;
+            cube = same_box && bx.U1 == lr && bx.U2 == lr && bx.U3 == lr;
         }
         ColumnBoxes cbox{0, 0, 0};
-        if (!cube) cbox = column_boxes(R1, R2, R3, bx, lane);
+        if (!same_box) cbox = column_boxes_rows(Rq, bx, lane);
 
         // p_t <= 2^-40 in every column when a2_weak d2 - z2_floor <= -40
         // (every row of 16 lanes holds the 16 columns, so a reduction over a row is complete)
@@ -248,7 +257,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 }
                 const float d2 = dist2(cell, (float)n1, (float)n2, (float)n3);
                 int bits = 0;
-                if (cube) {
+                if (same_box) {
                     bits = valid ? 0xFFFF : 0;
                 } else {
                     bits = column_bits(cbox, n1, n2, n3);     // all lanes take part in the lookup
@@ -296,7 +305,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             }
             if (!RINGS && lane < 12) {
                 const int pos = lane < 8 ? near_cnt + lane : BRING_SLOTS - far_cnt - 1 - (lane - 8);
-                ring_d2[pos] = __builtin_inff();
+                ring_d2[pos] = RIMG_NEUTRAL_D2;          // (finite: weight 0 and 0 * d2 = 0, as in an image)
                 ring_s[pos] = 0.f;
                 ring_bits[pos] = 0;
             }
@@ -320,12 +329,13 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                     const int slot = 4 * g_ + q;
                     return Rec{ring_d2[slot], ring_s[slot], ring_bits[slot]};
                 };
-                auto group = [&](const Rec &rec) {
-                    // padding records carry d2 = +inf: keep them out of p*d2.  (From an image the
-                    // padding has a large finite d2, weight 0 and 0 * d2 = 0, every record is in every
-                    // column's box, and columns that are switched off run with a = -1 and finite
-                    // garbage that is never stored: nothing to mask.)
-                    const bool on = RINGS || (col_on && ((rec.bits >> c) & 1));
+                // PLAIN (staged rings; boxes that are the same for all columns): every record is in every
+                // column's box, the padding has a large finite d2, i.e. weight 0 and 0 * d2 = 0, and columns
+                // that are switched off run with a = -1 and finite garbage that is never stored: nothing
+                // to mask.
+                auto group = [&](const Rec &rec, auto plain) {
+                    constexpr bool PLAIN = decltype(plain)::value;
+                    const bool on = PLAIN || (col_on && ((rec.bits >> c) & 1));
                     const float w = on ? exp2_hw(a2 * rec.d2 - z2) : 0.f;
                     const float wd = on ? w * rec.d2 : 0.f;
                     px += wd;
@@ -342,12 +352,21 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                     }
                 };
                 Rec ra = fetch(0);
-                for (int g = 0; g < groups; g += 2) {
-                    const Rec rb = fetch(g + 1);
-                    group(ra);
-                    if (g + 1 < groups) {
-                        ra = fetch(g + 2);
-                        group(rb);
+                if (RINGS || same_box) {
+                    for (int g = 0; g < groups; g += 2) {
+                        const Rec rb = fetch(g + 1);
+                        group(ra, std::true_type{});
+                        if (g + 1 < groups) {
+                            ra = fetch(g + 2);
+                            group(rb, std::true_type{});
+                        }
+                    }
+                } else {
+                    // (columns with boxes of their own: no registers to spare for the second record set)
+                    for (int g = 0; g < groups; g++) {
+                        const Rec rb = fetch(g + 1);
+                        group(ra, std::false_type{});
+                        ra = rb;
                     }
                 }
             }
@@ -357,7 +376,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                     const int slot = BRING_SLOTS - 4 * (g + 1) + q;
                     const float d2t = ring_d2[slot];
                     const int bits = ring_bits[slot];
-                    if (RINGS || (col_on && ((bits >> c) & 1))) px += exp2_hw(a2 * d2t - z2) * d2t;
+                    if (RINGS || same_box || (col_on && ((bits >> c) & 1))) px += exp2_hw(a2 * d2t - z2) * d2t;
                 }
             }
             wave_mem_sync();
@@ -367,11 +386,11 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         // registers through the whole accumulation)
         UnitGeom geo_next{};
         if (!RINGS) geo_next = unit_geom(gv_next, !UNIFORM);
-        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane);
+        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd + 2 * stride, pos_next2), lane_r);
         px = rows_sum(px);
 
         // ---- exchange: column (dir, head) of unit `wave` -> row ((head*2 + dir)*8 + wave)
-        if (q == 0) PXbuf[wave * 16 + c] = px;
+        if (q == 0) PXbuf[wave * 16 + c_r] = px;
         const int hw = hg * 8 + wave;
         const int jcol = c, unit_j = jcol & 7, dir_j = jcol >> 3;    // product column j = dir*8 + unit
         const float *src = Sbuf + xch_base(q, wave, unit_j, dir_j);
@@ -382,7 +401,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
             // (proj_bin(s, q) = 16 (s / 4) + 4 q + s % 4)
             // (wave-uniform base + 32-bit lane offset: no 64-bit address per lane kept across rounds)
             const float *wbase = p.W + (int64_t)hw * D * K;
-            const unsigned woff = (unsigned)(c * K + 4 * q);
+            const unsigned woff = (unsigned)(c_r * K + 4 * q_r);
 #pragma unroll
             for (int t4 = 0; t4 < NT; t4++) {
                 const float4_t w4 = *reinterpret_cast<const float4_t *>(wbase + (woff + 16u * t4));
@@ -410,7 +429,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         if (hw < H) {
             if (e_out >= 0 && g_gz && q == 0) gz_out = g_gz[row_out];
             if (e_out >= 0 && g_gv) {
-                const float *gp = g_gv + ((uint64_t)row_out * (unsigned)D + (unsigned)(4 * q));
+                const float *gp = g_gv + ((uint64_t)row_out * (unsigned)D + (unsigned)(4 * q_r));
                 if (4 * q + 3 < D) {
                     gv4 = *reinterpret_cast<const float4_t *>(gp);
                 } else {
@@ -458,7 +477,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                 float dot = out[0] * gv4[0] + out[1] * gv4[1] + out[2] * gv4[2] + out[3] * gv4[3];
                 dot = rows_sum(dot);
                 if (q == 0 && e_out >= 0 && hw < H) {
-                    const float PX = PXbuf[unit_j * 16 + dir_j * 8 + wave];
+                    const float PX = PXbuf[(c_r & 7) * 16 + (c_r >> 3) * 8 + wave];      // (unit_j, dir_j)
                     p.ga_edge[row_out] = fmaf(PX, gz_out, dot);
                 }
                 // operands of the gW update of the next pass, requested now so that they arrive
@@ -468,7 +487,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                     for (int s4 = 0; s4 < 4; s4++) {
                         const int e_k = __builtin_amdgcn_ds_bpermute((4 * s4 + q) << 2, col_edge);   // column 4*s4 + q
                         const unsigned row_k = (unsigned)e_k * (unsigned)H + (unsigned)hw;
-                        if (e_k >= 0 && c < D) gvk[s4] = g_gv[(uint64_t)row_k * (unsigned)D + (unsigned)c];
+                        if (e_k >= 0 && c < D) gvk[s4] = g_gv[(uint64_t)row_k * (unsigned)D + (unsigned)c_r];
                     }
                 }
             } else {

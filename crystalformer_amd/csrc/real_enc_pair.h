@@ -48,6 +48,30 @@ struct PairArgs {
     int flag_want;
 };
 
+// The arguments where the launch put them, in the kernel-argument segment.  A pointer that a
+// kernel uses once a round is read from there when it is needed (a scalar load that hits the
+// constant cache) instead of occupying two scalar registers through the whole kernel: the pair
+// kernels need more scalar registers than there are, and every value the compiler parks in a
+// vector register's lanes costs a vector instruction to get back.
+typedef const PairArgs __attribute__((address_space(4))) *PairArgsSeg;
+
+// (the reads through the returned pointer stay behind this point and are not kept across rounds)
+__device__ __forceinline__ PairArgsSeg reread(PairArgsSeg seg)
+{
+    int off = 0;
+    asm volatile("" : "+s"(off));
+    return reinterpret_cast<PairArgsSeg>(reinterpret_cast<const char __attribute__((address_space(4))) *>(seg) + off);
+}
+
+// A pointer field of the segment, read as a 64-bit word (hipcc of ROCm 7.2 stops with an internal
+// error on a lane-dependent choice between pointers that were loaded as pointers from there).
+template <typename T>
+__device__ __forceinline__ T *seg_pointer(T *const __attribute__((address_space(4))) *field)
+{
+    typedef const unsigned long long __attribute__((address_space(4))) *Word;
+    return reinterpret_cast<T *>(*reinterpret_cast<Word>(field));
+}
+
 struct Cell {
     float rx, ry, rz;
     float t[9];
@@ -109,6 +133,50 @@ __device__ __forceinline__ ColumnBoxes column_boxes(int R1, int R2, int R3, cons
     cb.m2 = axis_table(R2, bx.U2, lane);
     cb.m3 = axis_table(R3, bx.U3, lane);
     return cb;
+}
+
+// The same tables from half-widths laid out one axis per row of 16 lanes (lane 16 q + c: axis q of
+// column c; 0 in row 3): one ballot per |n| serves the three axes.
+__device__ __forceinline__ ColumnBoxes column_boxes_rows(int Rq, const BoxDims &bx, int lane)
+{
+    ColumnBoxes cb{0, 0, 0};
+    const int top = max(bx.U1, max(bx.U2, bx.U3));       // wave-uniform
+    for (int r = 1; r <= top; r++) {
+        const unsigned long long m = __ballot(Rq >= r);
+        const bool mine = lane == r - 1;
+        cb.m1 = mine ? (int)(m & 0xFFFFull) : cb.m1;
+        cb.m2 = mine ? (int)((m >> 16) & 0xFFFFull) : cb.m2;
+        cb.m3 = mine ? (int)((m >> 32) & 0xFFFFull) : cb.m3;
+    }
+    return cb;
+}
+
+// Half-width of column c along axis q for the lanes of row q < 3 (0 in row 3 and for columns that
+// are off): cf::range_rule, one axis per lane instead of three.
+__device__ __forceinline__ int column_axis_range(float a, float cutoff, const float *rvl, int lattice_range,
+                                                 int minimum_range, int q, bool col_on)
+{
+    int R = lattice_range;
+    if (cutoff != 0.0f) {
+        const float rv = q == 0 ? rvl[0] : (q == 1 ? rvl[1] : rvl[2]);
+        const bool counts = col_on && q < 3;
+        if (cutoff < 0.0f) {
+            // First with the one-ulp reciprocal and square root: the quotient that is rounded up
+            // comes out within 1e-6 of the exact rule's (relative), so unless it lies within 1e-4
+            // of a whole number (or is not finite, not below 1e6) both give the same half-width.
+            const float cut = __builtin_amdgcn_sqrtf(-0.5f * __builtin_amdgcn_rcpf(a)) * (-cutoff);
+            const float qf = (cut + 0.01f) * rv * (float)(1.0 / (2.0 * (double)PI_F));
+            const bool clear = fabsf(qf - rintf(qf)) > 1.0e-4f * fmaxf(fabsf(qf), 1.0f) && fabsf(qf) < 1.0e6f;
+            if (__ballot(counts && !clear) == 0ull) {             // (wave-uniform; nearly always)
+                const float up = ceilf(qf);
+                const int r = up <= 0.f ? 0 : (up > (float)MAX_RANGE ? MAX_RANGE : (int)up);
+                return counts ? max(r, minimum_range) : 0;
+            }
+            cutoff = sqrtf(-0.5f / a) * (-cutoff);
+        }
+        R = range_axis(cutoff, rv, minimum_range);
+    }
+    return (col_on && q < 3) ? R : 0;
 }
 
 // columns whose box contains translation (n1,n2,n3); |n| <= 64 on every axis

@@ -28,6 +28,8 @@
 //                that head (8 units x 2 directions) and stores 16-byte rows of v.
 #pragma once
 
+#include <type_traits>
+
 #include "real_enc_pair.h"
 
 namespace cfpair {
@@ -48,7 +50,8 @@ constexpr int PROJ_INDEXED = 2;          // W per edge or per atom: read from gl
 // (layout in real_enc_pair.h), WPB x 2 edge ids and WPB x 16 reciprocal column totals.
 // block_id / grid_size: this work-group's position among the work-groups that share the rounds.
 template <int NT, bool UNIFORM, int PROJ, int DT, bool SHORT_RING>
-__device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const int block_id, const int grid_size)
+__device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const PairArgsSeg seg, const int block_id,
+                                                       const int grid_size)
 {
     extern __shared__ __align__(16) float lds[];
     constexpr int SPLANE = XPLANE;      // exchange buffer of the shared-projection epilogue
@@ -57,12 +60,8 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
     const int q = lane >> 4;
     const int c = lane & 15;
     const int H = p.H, K = p.K, D = p.D;
-    // read-only inputs: plain restrict pointers let per-unit descriptors use scalar loads
-    const int64_t *__restrict__ g_pairs = p.pairs;
-    const float *__restrict__ g_rpos = p.rpos;
-    const float *__restrict__ g_tvecs = p.tvecs;
-    const float *__restrict__ g_a = p.a_ik;
-    const float *__restrict__ g_rvlen = p.rvlen;
+    // (p: the arguments as the compiler holds them; seg: the same in the kernel-argument segment, for
+    // the pointers that are fetched when they are needed, see real_enc_pair.h)
     // SHORT_RING (a fixed cube of at most 128 translations, the default cube has 125): the ring
     // holds 128 translations per pass, no more than the cube needs.  Fewer distances cached in
     // registers across the staging passes and less LDS per work-group than with a ring of 256:
@@ -94,7 +93,7 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
         return (rd_ < rounds && u_ < p.U) ? u_ : 0;
     };
     // exponent of column c of a unit in the head group of a round
-    auto load_a = [&](const UnitIds &d, const RoundPos &rp) -> float {
+    auto load_a = [&](const float *g_a, const UnitIds &d, const RoundPos &rp) -> float {
         const int h_ = min(rp.hg * 8 + (c & 7), H - 1);
         return g_a[((c < 8) ? d.i : d.j) * H + h_];
     };
@@ -121,15 +120,15 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
     RoundPos pos = round_pos(rd_first, rounds_per_hg, p.head_groups);
     RoundPos pos_next = round_pos(rd_next, rounds_per_hg, p.head_groups);
     // fill the descriptor pipeline: current round complete, next round's ids known
-    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(rd_first, pos), lane));
+    UnitIds ids = unit_ids(load_unit_ids(p.pairs, unit_of(rd_first, pos), lane));
     int uflag = unit_flag(rd_first, pos);
     float a_cur;
     UnitGeom geo;
     UnitIds ids_next;
     {
-        const float gv0 = load_unit_geom(ids, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
-        a_cur = load_a(ids, pos);
-        const int64_t dv1 = load_unit_ids(g_pairs, unit_of(rd_next, pos_next), lane);
+        const float gv0 = load_unit_geom(ids, lane, p.rpos, p.tvecs, UNIFORM ? nullptr : p.rvlen);
+        a_cur = load_a(p.a_ik, ids, pos);
+        const int64_t dv1 = load_unit_ids(p.pairs, unit_of(rd_next, pos_next), lane);
         geo = unit_geom(gv0, !UNIFORM);
         ids_next = unit_ids(dv1);
     }
@@ -164,26 +163,35 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
         const bool unit_on = u < p.U && (!select || unit_selected(p, uflag));
         const RoundPos pos_next2 = round_pos(rd_next2, rounds_per_hg, p.head_groups);
         // (the round after rd_next2: its candidates' flags are requested here, looked at at the end)
+        // (adaptive boxes: the addresses of the once-a-round loads are formed here, not kept in
+        // registers across the rounds)
+        int lane_r = lane;
+        if (!UNIFORM) asm volatile("" : "+v"(lane_r));
         bool candidate = false;
-        if (select) candidate = request_round_candidate(p, rd_next2, rounds, stride, lane);
+        if (select) candidate = request_round_candidate(p, rd_next2, rounds, stride, lane_r);
         // ticket for the round after rd_next2 (once past the end, no more draws): requested here,
         // looked at only before the epilogue, like the loads below
         unsigned int ticket_old = 0;
         const bool draw = sched && wave == 0 && rd_next2 < rounds;
         if (draw && lane == 0) ticket_old = atomicAdd(sched, 1u);
         // loads for the coming rounds, consumed just before this round's epilogue
-        const float gv_next = load_unit_geom(ids_next, lane, g_rpos, g_tvecs, UNIFORM ? nullptr : g_rvlen);
-        const float a_next = load_a(ids_next, pos_next);
+        const PairArgsSeg in = reread(seg);
+        const float *__restrict__ g_rvlen = UNIFORM ? nullptr : seg_pointer(&in->rvlen);
+        const float gv_next = load_unit_geom(ids_next, lane_r, seg_pointer(&in->rpos), seg_pointer(&in->tvecs), g_rvlen);
+        const float a_next = load_a(in->a_ik, ids_next, pos_next);
         const int uflag_next = unit_flag(rd_next, pos_next);
-        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd_next2, pos_next2), lane);
+        const int64_t dv_next2 = load_unit_ids(in->pairs, unit_of(rd_next2, pos_next2), lane_r);
         if (PROJ == PROJ_SHARED && hg != wa_hg) {
             const int hw = hg * 8 + wave;
+            const float *__restrict__ g_W = reread(seg)->W;
             if (hw < H && K == 16 * NT && D == 16 * DT) {
                 // full tiles: one base address per lane, 16-byte loads at fixed offsets
                 // (proj_bin(s, q) = 16 (s / 4) + 4 q + s % 4)
+                int qw = q, cw = c;
+                if (!UNIFORM) asm volatile("" : "+v"(qw), "+v"(cw));
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++) {
-                    const float *wrow = p.W + ((int64_t)hw * D + 16 * dt + c) * K + 4 * q;
+                    const float *wrow = g_W + ((int64_t)hw * D + 16 * dt + cw) * K + 4 * qw;
 #pragma unroll
                     for (int t4 = 0; t4 < NT; t4++) {
                         const float4_t w4 = *reinterpret_cast<const float4_t *>(wrow + 16 * t4);
@@ -201,7 +209,7 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
 #pragma unroll
                     for (int s = 0; s < 4 * NT; s++) {
                         const int d = 16 * dt + cc, k = proj_bin(s, qq);
-                        Wa[dt][s] = (hw < H && d < D && k < K) ? p.W[((int64_t)hw * D + d) * K + k] : 0.f;
+                        Wa[dt][s] = (hw < H && d < D && k < K) ? g_W[((int64_t)hw * D + d) * K + k] : 0.f;
                     }
             }
             wa_hg = hg;
@@ -224,13 +232,14 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
         // translation box: union over the 16 columns; per-column boxes when they differ
         BoxDims bx;
         bx.U1 = bx.U2 = bx.U3 = p.lattice_range;
-        int R1 = bx.U1, R2 = bx.U1, R3 = bx.U1;
+        // (lane (q, c) works out axis q of column c; the row maxima are the union box)
+        int Rq = 0, Uq = 0;
         if (!UNIFORM) {
-            range_rule(a, p.cutoff, geo.rvl, p.lattice_range, p.min_range, R1, R2, R3);
-            if (!col_on) R1 = R2 = R3 = 0;
-            bx.U1 = __builtin_amdgcn_readfirstlane(wave_max_int(R1));
-            bx.U2 = __builtin_amdgcn_readfirstlane(wave_max_int(R2));
-            bx.U3 = __builtin_amdgcn_readfirstlane(wave_max_int(R3));
+            Rq = column_axis_range(a, p.cutoff, geo.rvl, p.lattice_range, p.min_range, q, col_on);
+            Uq = row16_max_i(Rq);
+            bx.U1 = __builtin_amdgcn_readlane(Uq, 0);
+            bx.U2 = __builtin_amdgcn_readlane(Uq, 16);
+            bx.U3 = __builtin_amdgcn_readlane(Uq, 32);
         }
         bx.S3 = 2 * bx.U3 + 1;
         bx.S2 = 2 * bx.U2 + 1;
@@ -240,15 +249,18 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
         bx.inv_S3 = __builtin_amdgcn_rcpf((float)bx.S3);
         const int T = bx.T;
         // all active columns of this unit have the box [-lattice_range, lattice_range]^3 (wave-uniform)
-        bool cube = UNIFORM;
+        // ... or at least all the same box, the union (wave-uniform as well): then every translation of
+        // the box counts for every column and the per-column tables, lookups and minima are not needed
+        bool cube = UNIFORM, same_box = UNIFORM;
         if (!UNIFORM) {
             const int lr = p.lattice_range;
-            const bool other = col_on && (R1 != lr || R2 != lr || R3 != lr);
-            cube = bx.U1 == lr && bx.U2 == lr && bx.U3 == lr && NPRE * WAVE >= T && __ballot(other) == 0ull;
+            const bool other = col_on && q < 3 && Rq != Uq;
+            same_box = __ballot(other) == 0ull;
+            cube = same_box && bx.U1 == lr && bx.U2 == lr && bx.U3 == lr && NPRE * WAVE >= T;
         }
 
         ColumnBoxes cbox{0, 0, 0};
-        if (!UNIFORM && !cube) cbox = column_boxes(R1, R2, R3, bx, lane);
+        if (!UNIFORM && !same_box) cbox = column_boxes_rows(Rq, bx, lane);
         // geometry of one translation: d^2 and the in-box bits of the 16 columns
         auto geometry = [&](int idx, bool valid, float &d2, int &colbits) {
             int n1, n2, n3;
@@ -257,7 +269,8 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
             if (UNIFORM) {
                 colbits = valid ? 0xFFFF : 0;
             } else {
-                colbits = column_bits(cbox, n1, n2, n3);     // all lanes take part in the lookup
+                colbits = 0xFFFF;
+                if (!same_box) colbits = column_bits(cbox, n1, n2, n3);     // all lanes take part in the lookup
                 if (!valid) colbits = 0;
             }
         };
@@ -271,13 +284,35 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
                 best_idx = idx;
             }
         };
-        constexpr int NCACHE = RCAP / WAVE;
+        // (adaptive boxes: only the cube's distances are kept; other boxes are evaluated again by the
+        // staging passes, their minimum coming from the cube where it can, see below)
+        constexpr int NCACHE = UNIFORM ? RCAP / WAVE : NPRE;
         float d2c[NCACHE];
-        int bitsc[UNIFORM ? 1 : NCACHE];
-        const bool cached = T <= RCAP;
+        const bool cached = UNIFORM ? T <= RCAP : cube;
         // chunks of 64 translations in the box; kept opaque so that the chunk guards below stay
         // real (wave-uniform) branches instead of being folded into lane predicates
         const int nchunk = __builtin_amdgcn_readfirstlane((T + WAVE - 1) / WAVE);
+        // Boxes too large to keep: where the box of every active column holds the pre-decoded cube,
+        // the smallest d^2 over the cube stands in for the minimum over the box and the first pass
+        // is left out.  It is an upper bound of every column's own minimum, so the weights
+        // exp(a (d^2 - d^2ref)) of closer images exceed 1 (bounded by 2^100, see the test) and the
+        // 2^-40 drop below stays on the safe side; z = log(sum) + a d^2ref holds for any d^2ref.
+        bool quick_min = false;
+        if (!UNIFORM && !cached) {
+            const int lr = p.lattice_range;
+            const int side = 2 * lr + 1;
+            const bool short_col = col_on && q < 3 && Rq < lr;
+            if (NPRE * WAVE >= side * side * side && __ballot(short_col) == 0ull) {
+                float m = 1e10f;
+#pragma unroll
+                for (int ch = 0; ch < NPRE; ch++)        // (lanes past the cube repeat its last translation)
+                    m = fminf(m, dist2(cell, npre[ch][0], npre[ch][1], npre[ch][2]));
+                m = wave_min(m);
+                const float a2_strong = row16_max(col_on ? -a2 : 0.f);
+                quick_min = __builtin_amdgcn_readfirstlane((int)(a2_strong * m <= 100.0f)) != 0;
+                if (quick_min) best = m;
+            }
+        }
         if (cached) {
 #pragma unroll
             for (int ch = 0; ch < NCACHE; ch++) {
@@ -292,10 +327,9 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
                         geometry(ch * WAVE + lane, ch * WAVE + lane < T, d2c[ch], cb);
                     }
                     track_min(d2c[ch], cb, ch * WAVE + lane);
-                    if (!UNIFORM) bitsc[ch] = cb;
                 }
             }
-        } else {
+        } else if (!quick_min) {
             for (int c0 = 0; c0 < T; c0 += WAVE) {
                 float d2;
                 int cb;
@@ -307,7 +341,7 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
         // nearest image lies inside the column's box (nearly always); otherwise a pass that
         // tracks the 16 columns separately.
         float d2min = wave_min(best);
-        if (!UNIFORM && !cube) {
+        if (!UNIFORM && !same_box && !quick_min) {
             const unsigned long long holders = __ballot(best == d2min);
             const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)holders) - 1);
             const int idx_star = __builtin_amdgcn_readlane(best_idx, src);
@@ -400,8 +434,7 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
             if (cached) {
 #pragma unroll
                 for (int ch = 0; ch < NCACHE; ch++)
-                    if (ch < nchunk) stage(d2c[ch], UNIFORM ? (ch * WAVE + lane < T ? 0xFFFF : 0) : bitsc[UNIFORM ? 0 : ch],
-                                             ch * WAVE + lane < T);
+                    if (ch < nchunk) stage(d2c[ch], ch * WAVE + lane < T ? 0xFFFF : 0, ch * WAVE + lane < T);
             } else {
                 for (int c0 = 0; c0 < cnt; c0 += WAVE) {
                     float d2;
@@ -436,11 +469,14 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
                     const int slot = 4 * g_ + q;
                     return Rec{ring_d2[slot], ring_s[slot], ring_bits[slot]};
                 };
-                auto group = [&](const Rec &rec) {
+                // PLAIN: every staged translation counts for every column (fixed cube, or adaptive
+                // boxes that came out the same for all columns)
+                auto group = [&](const Rec &rec, auto plain) {
+                    constexpr bool PLAIN = decltype(plain)::value;
                     float w = exp2_hw(a2 * (rec.d2 - d2min));
                     // (fixed cube: every staged translation is inside every column's box, and the
                     // padding records carry d2 = +inf, i.e. weight 0)
-                    w = (col_on && (UNIFORM || ((rec.bits >> c) & 1))) ? w : 0.f;
+                    w = (col_on && (PLAIN || ((rec.bits >> c) & 1))) ? w : 0.f;
                     sum += w;
                     const int reach = group_reach(rec.bits);
 #pragma unroll
@@ -453,20 +489,19 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
                     }
                 };
                 Rec ra = fetch(0);
-                if (UNIFORM) {
+                if (UNIFORM || same_box) {
                     for (int g = 0; g < groups; g += 2) {
                         const Rec rb = fetch(g + 1);
-                        group(ra);
+                        group(ra, std::true_type{});
                         if (g + 1 < groups) {
                             ra = fetch(g + 2);
-                            group(rb);
+                            group(rb, std::true_type{});
                         }
                     }
                 } else {
-                    // (adaptive boxes: no registers to spare for the second record set)
                     for (int g = 0; g < groups; g++) {
                         const Rec rb = fetch(g + 1);
-                        group(ra);
+                        group(ra, std::false_type{});
                         ra = rb;
                     }
                 }
@@ -479,7 +514,7 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
                     const float d2t = ring_d2[slot];
                     const int bits = ring_bits[slot];
                     float w = exp2_hw(a2 * (d2t - d2min));
-                    sum += (col_on && ((bits >> c) & 1)) ? w : 0.f;
+                    sum += (col_on && (same_box || ((bits >> c) & 1))) ? w : 0.f;
                 }
             }
             wave_mem_sync();
@@ -497,7 +532,10 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
         sum = rows_sum(sum);
         const float inv = __builtin_amdgcn_rcpf(sum);      // 1 ulp, one instruction
         const int64_t e_col = (c < 8) ? e_ij : e_ji;
-        if (col_on && q == 0) p.z[e_col * H + h] = log2_hw(sum) * LN2 + d2min * a;
+        const PairArgsSeg outp = reread(seg);
+        float *__restrict__ g_z = outp->z;
+        float *__restrict__ g_v = outp->v;
+        if (col_on && q == 0) g_z[e_col * H + h] = log2_hw(sum) * LN2 + d2min * a;
 
         // epilogue: lane (q,c) holds S[bin = 16m + 4q + r][column c] in acc[m][r]
         if (PROJ == PROJ_NONE) {
@@ -505,7 +543,7 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
 #pragma unroll
                 for (int m = 0; m < NT; m++) {
                     int k0 = 16 * m + 4 * q;
-                    float *dst = p.v + (e_col * H + h) * K + k0;
+                    float *dst = g_v + (e_col * H + h) * K + k0;
 #pragma unroll
                     for (int r = 0; r < 4; r++)
                         if (k0 + r < K) dst[r] = acc[m][r] * inv;
@@ -553,7 +591,7 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
 #pragma unroll
                     for (int dt = 0; dt < DT; dt++) {
                         const int dbase = 16 * dt + 4 * q;
-                        float *dst = p.v + (e_out * H + hw) * D + dbase;
+                        float *dst = g_v + (e_out * H + hw) * D + dbase;
                         if (dbase + 3 < D) {
                             *reinterpret_cast<float4_t *>(dst) = out[dt];
                         } else {
@@ -569,7 +607,7 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
             int64_t w_ind = 0;
             if (p.W_num == p.E) w_ind = e_col;
             else if (p.W_num == p.N) w_ind = atom;
-            const float *Wg = p.W + (w_ind * H + (col_on ? h : 0)) * (int64_t)D * K;
+            const float *Wg = reread(seg)->W + (w_ind * H + (col_on ? h : 0)) * (int64_t)D * K;
             for (int d0 = 0; d0 < D; d0 += 16) {
                 float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;   // this lane's 4 output components
 #pragma unroll
@@ -595,7 +633,7 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
                 }
                 if (col_on) {
                     const int dbase = d0 + 4 * q;
-                    float *dst = p.v + (e_col * H + h) * D + dbase;
+                    float *dst = g_v + (e_col * H + h) * D + dbase;
                     if (dbase + 0 < D) dst[0] = o0 * inv;
                     if (dbase + 1 < D) dst[1] = o1 * inv;
                     if (dbase + 2 < D) dst[2] = o2 * inv;

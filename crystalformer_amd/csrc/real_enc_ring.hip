@@ -463,11 +463,15 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_two_role_kernel(PairArgs 
                                                                        const float *__restrict__ cache,
                                                                        int pair_blocks)
 {
-    if ((int)blockIdx.x < pair_blocks)
-        real_enc_fwd_pair_body<NT, false, PROJ_SHARED, DT, false>(p_pair, (int)blockIdx.x, pair_blocks);
-    else
+    if ((int)blockIdx.x < pair_blocks) {
+        // (p_pair is the kernel's second argument, behind p_ring in the kernel-argument segment)
+        static_assert(sizeof(PairArgs) % 8 == 0, "the second argument follows the first without padding");
+        const PairArgsSeg seg = (PairArgsSeg)__builtin_amdgcn_kernarg_segment_ptr() + 1;
+        real_enc_fwd_pair_body<NT, false, PROJ_SHARED, DT, false>(p_pair, seg, (int)blockIdx.x, pair_blocks);
+    } else {
         real_enc_fwd_ring_body<NT, DT, true>(p_ring, cache, (int)blockIdx.x - pair_blocks,
                                              (int)gridDim.x - pair_blocks);
+    }
 }
 
 }  // namespace

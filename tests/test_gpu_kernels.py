@@ -104,6 +104,40 @@ def test_real_enc_pair_kernel_large_boxes_and_indexed_projection(dev):
         assert_close(v, v_ref, "v", atol=v_atol(pm, 16, pm.W, -3.5, 2, 2))
 
 
+def test_real_enc_pair_kernels_where_the_sigma_rule_hits_whole_numbers(dev):
+    """Exponents chosen so that (3.5 sigma + 0.01) |b| / 2 pi of one axis is a whole number to within a
+    few float ulps, per (atom, head): the pair kernels work the half-widths out with one-ulp
+    reciprocals and square roots and must fall back to the exact rule there.  A half-width that is off
+    by one adds or drops a shell of translations at 3.5 sigma, 2e-3 of the leading term."""
+    p = Problem([3, 6, 2], H=8, K=64, D=16, seed=41)
+    g = torch.Generator().manual_seed(3)
+    two_pi = 2.0 * float(torch.tensor(3.141592654, dtype=torch.float32))
+    rv = p.rvlen[p.b.batch].double()                                    # (N, 3)
+    axis = torch.randint(0, 3, (p.N, 8), generator=g)
+    k = torch.randint(2, 5, (p.N, 8), generator=g).double()
+    sigma = (k * two_pi / rv.gather(1, axis) - float(torch.tensor(0.01, dtype=torch.float32))) / 3.5
+    a = (-0.5 / (sigma * sigma)).float()
+    for _ in range(int(torch.randint(0, 3, (1,), generator=g))):        # a few ulps either way for some
+        a = torch.where(torch.rand(p.N, 8, generator=g) < 0.5, torch.nextafter(a, torch.zeros(())), a)
+    p.a = a
+    R = ks.translation_ranges(p.a, p.rvlen, p.b.batch, -3.5, 2, 0)
+    on_axis = R.gather(2, axis[:, :, None]).squeeze(2).double()
+    assert float(((on_axis - k).abs() <= 1).float().mean()) == 1.0 and len(set(on_axis.flatten().tolist())) >= 3
+    z_ref, v_ref = enc_fwd_ref(p, 64, p.W, -3.5, 2, 0)
+    z, v = enc_fwd_gpu(dev, p, 64, p.W, -3.5, 2, 0, pairs=True)
+    assert_close(z, z_ref, "z")
+    assert_close(v, v_ref, "v", atol=v_atol(p, 64, p.W, -3.5, 2, 0))
+    gz, gv = p.randn(p.E, 8), p.randn(p.E, 8, 16)
+    args = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv)
+    ga, gW = ops.real_enc_bwd(*args, 64, p.dist_max, p.wscale, p.W.to(dev), p.rvlen.to(dev), -3.5, 2, 0,
+                              pairs_u=ops.edge_pairs(p.b.sizes.to(dev)))
+    ga_ref, gW_ref = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv, 64,
+                                     p.dist_max, p.wscale, p.W, p.rvlen, -3.5, 2, 0)
+    ga_atol, gW_atol = enc_bwd_atols(p, z_ref, gz, gv, 64, p.W, -3.5, 2, 0)
+    assert_close(ga, ga_ref, "ga", atol=ga_atol)
+    assert_close(gW, gW_ref, "gW", atol=gW_atol)
+
+
 @pytest.mark.parametrize("cutoff,mr", [(-3.5, 0), (-1.0, 0), (2.0, 0), (-3.5, 1)])
 def test_real_enc_pair_kernel_atoms_outside_the_home_cell(dev, cutoff, mr):
     """Atoms displaced by whole lattice vectors: the nearest image of an edge is then a
