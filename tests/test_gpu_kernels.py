@@ -104,6 +104,33 @@ def test_real_enc_pair_kernel_large_boxes_and_indexed_projection(dev):
         assert_close(v, v_ref, "v", atol=v_atol(pm, 16, pm.W, -3.5, 2, 2))
 
 
+@pytest.mark.parametrize("scale,mr", [(0.05, 2), (0.05, 0), (0.3, 2), (1.0, 3)])
+def test_real_enc_pair_kernels_one_box_for_all_columns(dev, scale, mr):
+    """The same exponent for every (atom, head): all 16 columns of an atom pair have one box, which
+    is not the cube (wide Gaussians: several staging passes per pair; floor above lattice_range:
+    one pass).  The kernels then skip the per-column tables and masks and, for boxes of several
+    passes, take the reference distance from the cube."""
+    p = Problem([4, 7, 1, 2], H=8, K=64, D=16, seed=43)
+    p.a = torch.full_like(p.a, float(p.a.mean()) * scale)
+    R = ks.translation_ranges(p.a, p.rvlen, p.b.batch, -3.5, 2, mr)
+    assert bool((R == R[:, :1, :]).all())                               # one box per crystal
+    T = (2 * R[:, 0, :] + 1).prod(dim=1)
+    assert int(T.max()) > (192 if scale < 0.1 else 125)
+    z_ref, v_ref = enc_fwd_ref(p, 64, p.W, -3.5, 2, mr)
+    z, v = enc_fwd_gpu(dev, p, 64, p.W, -3.5, 2, mr, pairs=True)
+    assert_close(z, z_ref, "z")
+    assert_close(v, v_ref, "v", atol=v_atol(p, 64, p.W, -3.5, 2, mr))
+    gz, gv = p.randn(p.E, 8), p.randn(p.E, 8, 16)
+    args = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv)
+    ga, gW = ops.real_enc_bwd(*args, 64, p.dist_max, p.wscale, p.W.to(dev), p.rvlen.to(dev), -3.5, 2, mr,
+                              pairs_u=ops.edge_pairs(p.b.sizes.to(dev)))
+    ga_ref, gW_ref = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z_ref, gz, gv, 64,
+                                     p.dist_max, p.wscale, p.W, p.rvlen, -3.5, 2, mr)
+    ga_atol, gW_atol = enc_bwd_atols(p, z_ref, gz, gv, 64, p.W, -3.5, 2, mr)
+    assert_close(ga, ga_ref, "ga", atol=ga_atol)
+    assert_close(gW, gW_ref, "gW", atol=gW_atol)
+
+
 def test_real_enc_pair_kernels_where_the_sigma_rule_hits_whole_numbers(dev):
     """Exponents chosen so that (3.5 sigma + 0.01) |b| / 2 pi of one axis is a whole number to within a
     few float ulps, per (atom, head): the pair kernels work the half-widths out with one-ulp
