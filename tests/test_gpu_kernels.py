@@ -104,6 +104,30 @@ def test_real_enc_pair_kernel_large_boxes_and_indexed_projection(dev):
         assert_close(v, v_ref, "v", atol=v_atol(pm, 16, pm.W, -3.5, 2, 2))
 
 
+@pytest.mark.parametrize("scale,mr", [(0.03, 2), (0.3, 2), (1.0, 3)])
+def test_real_enc_pair_kernel_large_boxes_with_the_nearest_image_outside_the_cube(dev, scale, mr):
+    """Atoms displaced by whole lattice vectors under the floored rule: every box holds the cube, but the
+    nearest image of an edge lies up to four cells away, outside it.  Boxes of several staging passes
+    take their reference distance from the cube: weights above 1 (wide Gaussians) or, where that would
+    go too far (narrow Gaussians in boxes that a floor of 3 makes large: |a| d2 of the cube's nearest
+    image beyond the kernel's limit for many pairs), the pass over the whole box."""
+    p = Problem([5, 2, 8, 1], H=8, K=64, D=16, seed=47)
+    g = torch.Generator().manual_seed(78)
+    shift = torch.randint(-2, 3, (p.N, 3), generator=g).float()
+    p.b.pos = p.b.pos + (shift[:, None, :] @ p.b.trans_vec[p.b.batch]).squeeze(1)
+    p.rpos = tp.relative_positions(p.b.pos, p.edges)
+    p.a = p.a * scale
+    R = ks.translation_ranges(p.a, p.rvlen, p.b.batch, -3.5, 2, mr)
+    assert int((2 * R.max(dim=1).values + 1).prod(dim=1).max()) > 192
+    z_ref, v_ref = enc_fwd_ref(p, 64, p.W, -3.5, 2, mr)
+    z, v = enc_fwd_gpu(dev, p, 64, p.W, -3.5, 2, mr, pairs=True)
+    ok = torch.isfinite(z_ref)
+    assert ok.float().mean() > 0.5
+    okv = ok[:, :, None].expand_as(v_ref)
+    assert_close(torch.where(ok, z.cpu(), torch.zeros(())), torch.where(ok, z_ref, torch.zeros(())), "z")
+    assert_close(torch.where(okv, v.cpu(), torch.zeros(())), torch.where(okv, v_ref, torch.zeros(())), "v")
+
+
 @pytest.mark.parametrize("scale,mr", [(0.05, 2), (0.05, 0), (0.3, 2), (1.0, 3)])
 def test_real_enc_pair_kernels_one_box_for_all_columns(dev, scale, mr):
     """The same exponent for every (atom, head): all 16 columns of an atom pair have one box, which
