@@ -499,10 +499,13 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
                         }
                     }
                 } else {
-                    for (int g = 0; g < groups; g++) {
+                    for (int g = 0; g < groups; g += 2) {
                         const Rec rb = fetch(g + 1);
                         group(ra, std::false_type{});
-                        ra = rb;
+                        if (g + 1 < groups) {
+                            ra = fetch(g + 2);
+                            group(rb, std::false_type{});
+                        }
                     }
                 }
             }
