@@ -26,6 +26,13 @@
 //                wavefront w multiplies head w's D x K matrix (held in registers
 //                as MFMA A operands for the whole kernel) with the 16 columns of
 //                that head (8 units x 2 directions) and stores 16-byte rows of v.
+//
+// Adaptive boxes (UNIFORM = false): the 16 columns of a unit have half-widths of their own
+// (models/kernels/real_enc_fwd.cu:58-85), worked out one axis per lane.  Three kinds of unit,
+// told apart with one ballot each: all columns have the cube [-lattice_range, lattice_range]^3
+// (the cube's shortcuts: translations decoded once per kernel, no column masks); all columns
+// have the same box (no per-column tables, lookups, minima or masks); otherwise per-axis
+// tables of column sets and a 16-bit column mask per translation.
 #pragma once
 
 #include <type_traits>
