@@ -25,6 +25,13 @@ int device_cu_count();
 // Work-groups a persistent kernel may launch at `per_cu` per CU, scaled by the calling
 // thread's launch share (cf_set_launch_share).
 int persistent_grid_cap(int per_cu);
+// Live sizes on the device (cf_set_size_header).  Each returns the header word that holds the
+// live count when the calling thread has a header set and the argument is the capacity that
+// word goes with (atoms, edges, atom pairs), else NULL: the size argument is then the size.
+const int64_t *live_atoms(int64_t N);
+const int64_t *live_edges(int64_t E);
+const int64_t *live_units(int64_t U);
+int64_t *size_header_for_layout(int64_t N, int64_t E);
 
 // real_enc_mfma.hip
 int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,
@@ -78,6 +85,19 @@ int launch_unit_floor(const float *a_ik, const float *rvlen, const int64_t *pair
 
 // ---- device helpers --------------------------------------------------------
 #if defined(__HIPCC__)
+
+// The live count behind a size argument: *live (clamped to the capacity, so that no value the
+// header can hold sends a kernel outside its buffers) when a header word is given, else the
+// argument itself.  Wave-uniform.
+__device__ __forceinline__ int64_t live_count(const int64_t *live, int64_t capacity)
+{
+    if (!live) return capacity;
+    const int64_t n = *live;
+    const int64_t c = n < 0 ? 0 : (n > capacity ? capacity : n);
+    const int lo = __builtin_amdgcn_readfirstlane((int)(c & 0xFFFFFFFFll));
+    const int hi = __builtin_amdgcn_readfirstlane((int)(c >> 32));
+    return ((int64_t)hi << 32) | (unsigned int)lo;
+}
 
 __device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float log2_hw(float x) { return __builtin_amdgcn_logf(x); }

@@ -46,9 +46,42 @@ int persistent_grid_cap(int per_cu)
     return (int)(cap < 1 ? 1 : cap);
 }
 
+// Live sizes on the device (cf_set_size_header): the header and the capacities it goes with.
+static thread_local const int64_t *g_size_header = nullptr;
+static thread_local int64_t g_cap_atoms = -1, g_cap_edges = -1;
+
+const int64_t *live_atoms(int64_t N) { return (g_size_header && N == g_cap_atoms) ? g_size_header : nullptr; }
+const int64_t *live_edges(int64_t E) { return (g_size_header && E == g_cap_edges) ? g_size_header + 1 : nullptr; }
+const int64_t *live_units(int64_t U)
+{
+    return (g_size_header && 2 * U == g_cap_atoms + g_cap_edges) ? g_size_header + 2 : nullptr;
+}
+int64_t *size_header_for_layout(int64_t N, int64_t E)
+{
+    return (g_size_header && N == g_cap_atoms && E == g_cap_edges) ? const_cast<int64_t *>(g_size_header) : nullptr;
+}
+
 }  // namespace cf
 
-extern "C" int cf_version(void) { return 100; }
+extern "C" int cf_version(void) { return 101; }
+
+extern "C" int cf_set_size_header(int64_t *header_4, int64_t N_cap, int64_t E_cap)
+{
+    if (!header_4) {
+        cf::g_size_header = nullptr;
+        cf::g_cap_atoms = cf::g_cap_edges = -1;
+        return CF_OK;
+    }
+    CF_REQUIRE(N_cap >= 1 && E_cap >= 1 && (N_cap + E_cap) % 2 == 0, CF_ERR_INVALID_ARGUMENT,
+               "cf_set_size_header: capacities must be positive with an even sum (got %lld atoms, %lld edges)",
+               (long long)N_cap, (long long)E_cap);
+    cf::g_size_header = header_4;
+    cf::g_cap_atoms = N_cap;
+    cf::g_cap_edges = E_cap;
+    return CF_OK;
+}
+
+extern "C" const int64_t *cf_get_size_header(void) { return cf::g_size_header; }
 
 extern "C" int cf_set_launch_share(double share)
 {

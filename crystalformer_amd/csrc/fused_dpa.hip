@@ -25,6 +25,7 @@ struct DpaArgs {
     float *gque, *gkey, *gval, *gaij, *gbij;
     int64_t N, E;
     int H, Dk, Dv;
+    const int64_t *live_N;   // forward only, nullable: live atom count on the device (N is then the capacity)
 };
 
 constexpr int MAXH = 16;
@@ -35,7 +36,7 @@ __global__ __launch_bounds__(256) void fused_dpa_fwd_kernel(DpaArgs p)
 {
     const int lane = threadIdx.x & 63;
     const int64_t i = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (i >= p.N) return;   // whole wave exits together
+    if (i >= live_count(p.live_N, p.N)) return;   // whole wave exits together
     const int Dk = p.Dk, Dv = p.Dv;
     const int64_t e0 = p.e_start[i], e1 = p.e_start[i + 1];
     const int64_t *dst = p.edges + p.E;
@@ -182,6 +183,7 @@ __global__ __launch_bounds__(256, (PREFETCH ? 6 : 7)) void fused_dpa_fwd_stream_
     const uint32_t h = piece / DV4;
     const bool lead = (piece % DV4) == 0;      // first piece of its head: owns the logit
     const uint32_t e0 = (uint32_t)p.e_start[i], e1 = (uint32_t)p.e_start[i + 1];
+    if (p.live_N && (int64_t)i >= live_count(p.live_N, p.N)) return;   // beyond the live atoms (whole work-group)
     if (e0 >= e1) {                            // an atom without edges yields zeros (whole work-group)
         if (threadIdx.x < HD4)
             reinterpret_cast<float4_v *>(p.out)[i * HD4 + threadIdx.x] = float4_v{0.f, 0.f, 0.f, 0.f};
@@ -642,6 +644,7 @@ extern "C" int cf_fused_dpa_fwd(const float *que, const float *key, const float 
     p.edges = edge_ij_e; p.e_start = e_start_i;
     p.prob = prob_eh; p.out = out;
     p.N = N; p.E = E; p.H = (int)H; p.Dk = (int)Dk; p.Dv = (int)Dv;
+    p.live_N = cf::live_atoms(N);
     hipStream_t st = (hipStream_t)stream;
     // streaming kernel when a head's components split into 16-byte pieces that tile a wavefront
     const int64_t dv4 = Dv / 4, lpe = H * dv4;

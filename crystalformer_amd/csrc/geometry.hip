@@ -66,7 +66,21 @@ struct GaussArgs {
     float *part;       // (blocks, 3): count, mean, sum of squared deviations; then (scale, shift) used and stored
     int blocks;
     float *alpha_n, *a, *q_scaled;
+    const int64_t *live_N;   // nullable: the live atom count on the device (N is then the capacity)
 };
+
+// Live element count and the number of blocks that hold an element (the statistics are merged over
+// exactly those, so a launch sized for a capacity gives the bits of a launch sized for the live count).
+__device__ __forceinline__ int64_t live_total(const GaussArgs &p, int &blocks)
+{
+    if (!p.live_N) {
+        blocks = p.blocks;
+        return p.total;
+    }
+    const int64_t total = live_count(p.live_N, p.N) * p.H;
+    blocks = (int)((total + GE_THREADS - 1) / GE_THREADS);
+    return total;
+}
 
 __device__ __forceinline__ float positive_map(float x, int func, float beta, float lb)
 {
@@ -96,7 +110,10 @@ __global__ __launch_bounds__(GE_THREADS) void gauss_exponents_alpha_kernel(Gauss
 {
     __shared__ float red[GE_THREADS / WAVE][2];
     const int64_t t = (int64_t)blockIdx.x * GE_THREADS + threadIdx.x;
-    const bool live = t < p.total;
+    int live_blocks;
+    const int64_t total = live_total(p, live_blocks);
+    if ((int)blockIdx.x >= live_blocks) return;
+    const bool live = t < total;
     float alpha = 0.f;
     if (live) {
         const int64_t h = t % p.H;
@@ -129,7 +146,7 @@ __global__ __launch_bounds__(GE_THREADS) void gauss_exponents_alpha_kernel(Gauss
     // block statistics: mean first, then squared deviations from it
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int64_t first = (int64_t)blockIdx.x * GE_THREADS;
-    const float cnt = (float)min((int64_t)GE_THREADS, p.total - first);
+    const float cnt = (float)min((int64_t)GE_THREADS, total - first);
     float s = wave_sum(live ? alpha : 0.f);
     if (lane == 0) red[wave][0] = s;
     __syncthreads();
@@ -160,10 +177,13 @@ __global__ __launch_bounds__(GE_THREADS) void gauss_exponents_alpha_kernel(Gauss
 __global__ __launch_bounds__(GE_THREADS) void gauss_exponents_final_kernel(GaussArgs p)
 {
     __shared__ float sh[2];
+    int live_blocks;
+    const int64_t total = live_total(p, live_blocks);
+    if ((int)blockIdx.x >= live_blocks) return;
     if (threadIdx.x < WAVE) {
         const int lane = threadIdx.x;
         float n = 0.f, mean = 0.f, m2 = 0.f;
-        for (int b = lane; b < p.blocks; b += WAVE)
+        for (int b = lane; b < live_blocks; b += WAVE)
             stat_merge(n, mean, m2, p.part[3 * b], p.part[3 * b + 1], p.part[3 * b + 2]);
 #pragma unroll
         for (int off = 1; off < WAVE; off <<= 1) {
@@ -195,7 +215,7 @@ __global__ __launch_bounds__(GE_THREADS) void gauss_exponents_final_kernel(Gauss
     __syncthreads();
     const float scale = sh[0], shift = sh[1];
     const int64_t t = (int64_t)blockIdx.x * GE_THREADS + threadIdx.x;
-    if (t >= p.total) return;
+    if (t >= total) return;
     const float x = (p.a[t] + shift) * scale;
     if (p.alpha_n) p.alpha_n[t] = x;
     p.a[t] = positive_map(x, p.func, p.beta, p.lb) * p.coef;
@@ -420,6 +440,7 @@ extern "C" int cf_gauss_exponents(const float *q, const float *w, float *gauss_s
     p.beta = beta; p.lb = lower_bound; p.coef = coef; p.q_scale = q_scale;
     p.part = (float *)workspace; p.blocks = (int)blocks;
     p.alpha_n = alpha_n; p.a = a; p.q_scaled = q_scaled;
+    p.live_N = cf::live_atoms(N);
     gauss_exponents_alpha_kernel<<<(int)blocks, GE_THREADS, 0, stream>>>(p);
     CF_CHECK_LAUNCH("cf_gauss_exponents: alpha");
     if (normalize) {

@@ -20,6 +20,7 @@ struct LinArgs {
     float *y[3];               // each (N, C)
     int64_t N;
     int K, C, nw, relu;
+    const int64_t *live_N;     // nullable: live row count on the device (N is then the capacity)
 };
 
 // LDS-tiled: a work-group of 4 wavefronts (WR x WC) owns TM rows x TN columns; every KC-wide
@@ -46,15 +47,18 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(LinArgs p)
     const int wave = threadIdx.x >> 6;
     const int q = lane >> 4, c = lane & 15;
     const int wr = wave / WC, wc = wave - wr * WC;
-    const int64_t row0 = (int64_t)blockIdx.x * TM;
+    const int64_t N = live_count(p.live_N, p.N);
     const int col0 = blockIdx.y * TN;                           // column over all weights
+    // (one row tile per work-group unless the grid was cut short: with a live row count the launch
+    // covers a capacity, and a work-group then strides over the row tiles that exist)
+    for (int64_t row0 = (int64_t)blockIdx.x * TM; row0 < N; row0 += (int64_t)gridDim.x * TM) {
     const int total_cols = p.nw * p.C;
     // staging role: thread -> (row t / PPR (+RPP u), 16-byte piece t % PPR) of a tile
     const int srow = threadIdx.x / PPR, spiece = threadIdx.x % PPR;
     const float *xg[XL];
     const float *wg[WL];
 #pragma unroll
-    for (int u = 0; u < XL; u++) xg[u] = p.x + min(row0 + srow + RPP * u, p.N - 1) * p.K + 4 * spiece;
+    for (int u = 0; u < XL; u++) xg[u] = p.x + min(row0 + srow + RPP * u, N - 1) * p.K + 4 * spiece;
 #pragma unroll
     for (int u = 0; u < WL; u++) {
         const int col = min(col0 + srow + RPP * u, total_cols - 1);
@@ -118,12 +122,13 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(LinArgs p)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int64_t row = row0 + (wr * MT + mt) * 16 + 4 * q + r;
-                if (row >= p.N) continue;
+                if (row >= N) continue;
                 float v = acc[mt][nt][r] + bv;
                 if (p.res) v += p.res[row * p.C + lc];
-                if (p.relu) v = fmaxf(v, 0.f);
+                if (p.relu) v = v < 0.f ? 0.f : v;              // (a NaN stays one, as in torch.relu)
                 y[row * p.C + lc] = v;
             }
+    }
     }
 }
 
@@ -462,12 +467,16 @@ extern "C" int cf_linear_rows(const float *x, int64_t N, int64_t K, const float 
     }
     p.bias = bias; p.res = residual;
     p.N = N; p.K = (int)K; p.C = (int)C; p.nw = n_weights; p.relu = relu;
+    p.live_N = cf::live_atoms(N);      // (rows are atoms when N is the atom capacity of a size header)
     // few rows (a tile grid that leaves CUs idle): 32 x 32 tiles, four to eight times the work-groups;
     // otherwise wide outputs take 64-column tiles (2 x 2 wavefronts), narrow ones 32-column tiles
     const int64_t total_cols = (int64_t)n_weights * C;
     const bool small = N <= 8192;
     const bool wide = !small && total_cols >= 256;
-    const int64_t gx = (N + (small ? 31 : 63)) / (small ? 32 : 64);
+    int64_t gx = (N + (small ? 31 : 63)) / (small ? 32 : 64);
+    // a capacity: most row tiles are beyond the live rows, so launch a bounded number of work-groups
+    // per column tile and let them stride (empty work-groups cost a few microseconds per thousand)
+    if (p.live_N && gx > 128) gx = 128;
     const int64_t gy = (total_cols + (wide ? 63 : 31)) / (wide ? 64 : 32);
     CF_REQUIRE(gx < (1ll << 31) && gy < 65536, CF_ERR_UNSUPPORTED, "cf_linear_rows: too large");
     const dim3 grid((unsigned)gx, (unsigned)gy);

@@ -1041,6 +1041,9 @@ extern "C" int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const 
         }
         if (rc != CF_ERR_UNSUPPORTED) return rc;   // otherwise: shape not instantiated, use the per-edge kernel
     }
+    CF_REQUIRE(!cf::live_edges(E), CF_ERR_UNSUPPORTED,
+               "cf_real_enc_fwd: with a size header set only the pair-evaluated kernels are served "
+               "(pair list, K <= 128, shared projection with D <= 32)");
     rc = CF_DISPATCH_H(H, launch_fwd, p, (hipStream_t)stream);
     if (rc) return rc;
     CF_CHECK_LAUNCH("cf_real_enc_fwd");

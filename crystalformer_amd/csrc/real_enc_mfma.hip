@@ -33,9 +33,11 @@ using namespace cf;
 using namespace cfpair;
 
 template <int NT, bool UNIFORM, int PROJ, int DT, bool SHORT_RING>
-__global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
+__global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p_)
 {
-    // (p is the kernel's first argument: it lies at the start of the kernel-argument segment)
+    const PairArgs p = with_live_units(p_);
+    if (p.U == 0) return;          // (an empty list: not even the descriptor of unit 0 may be read)
+    // (p_ is the kernel's first argument: it lies at the start of the kernel-argument segment)
     const cfpair::PairArgsSeg seg = (cfpair::PairArgsSeg)__builtin_amdgcn_kernarg_segment_ptr();
     real_enc_fwd_pair_body<NT, UNIFORM, PROJ, DT, SHORT_RING>(p, seg, (int)blockIdx.x, (int)gridDim.x);
 }
@@ -43,10 +45,11 @@ __global__ __launch_bounds__(512, 4) void real_enc_fwd_pair_kernel(PairArgs p)
 // Unit descriptors: the (i <= j) edges of every crystal's dense block, their reverses,
 // the two atoms and the crystal.
 __global__ void edge_pairs_kernel(const int64_t *atom_start, const int64_t *edge_start,
-                                  const int64_t *unit_start, int64_t B, int64_t E, int64_t *pairs)
+                                  const int64_t *unit_start, int64_t B, int64_t E, const int64_t *live_E,
+                                  int64_t *pairs)
 {
     int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= E) return;
+    if (e >= live_count(live_E, E)) return;
     int64_t lo = 0, hi = B;
     while (hi - lo > 1) {
         int64_t mid = (lo + hi) >> 1;
@@ -126,6 +129,8 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     // unit selection: the units that do not keep the cube (the others run from the staged rings)
     p.unit_flags = unit_flags; p.round_flags = round_flags; p.flag_want = 0;
     if (unit_flags) p.sched = nullptr;
+    p.live_U = live_units(U);
+    if (p.live_U && unit_flags) return CF_ERR_UNSUPPORTED;   // (the flags are laid out for a known U)
 #define CF_PAIR(NTV, UNI, PRJ, DTV, SR) \
     real_enc_fwd_pair_kernel<NTV, UNI, PRJ, DTV, SR><<<(int)blocks, WPB * WAVE, lds, st>>>(p)
 #define CF_PAIR_MODE(NTV, UNI, SR)                                            \
@@ -164,7 +169,8 @@ extern "C" int cf_edge_pairs(const int64_t *atom_start_n, const int64_t *edge_st
     CF_REQUIRE(B > 0 && atom_start_n && edge_start_n && unit_start_n && pairs_u, CF_ERR_INVALID_ARGUMENT,
                "cf_edge_pairs: null pointer or no crystals");
     edge_pairs_kernel<<<(int)((E + 255) / 256), 256, 0, (hipStream_t)stream>>>(atom_start_n, edge_start_n,
-                                                                              unit_start_n, B, E, pairs_u);
+                                                                              unit_start_n, B, E, cf::live_edges(E),
+                                                                              pairs_u);
     CF_CHECK_LAUNCH("cf_edge_pairs");
     return CF_OK;
 }

@@ -46,7 +46,21 @@ struct PairArgs {
     const unsigned char *unit_flags;
     const unsigned char *round_flags;
     int flag_want;
+    // Live unit count on the device, nullable (forward and staging kernels): U is then the capacity
+    // of the unit list -- what the grid and the buffers are sized for -- and the kernel walks the
+    // first *live_U units only.
+    const int64_t *live_U;
 };
+
+#if defined(__HIPCC__)
+// The arguments a kernel body works with: U replaced by the live count when there is one.
+__device__ __forceinline__ PairArgs with_live_units(const PairArgs &p)
+{
+    PairArgs q = p;
+    q.U = live_count(p.live_U, p.U);
+    return q;
+}
+#endif
 
 // The arguments where the launch put them, in the kernel-argument segment.  A pointer that a
 // kernel uses once a round is read from there when it is needed (a scalar load that hits the

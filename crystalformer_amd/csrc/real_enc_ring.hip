@@ -54,8 +54,9 @@ __device__ __forceinline__ int slot_record(const PairArgs &p, float d2, float &s
 struct StageIds { int64_t e_ij, n; };
 
 template <int NT>
-__global__ __launch_bounds__(256) void ring_stage_kernel(PairArgs p, float weak_a2, float *__restrict__ cache)
+__global__ __launch_bounds__(256) void ring_stage_kernel(PairArgs p_, float weak_a2, float *__restrict__ cache)
 {
+    const PairArgs p = with_live_units(p_);
     const int lane = threadIdx.x & 63;
     const int64_t waves = (int64_t)gridDim.x * (blockDim.x >> 6);
     const int64_t first = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)));
@@ -448,8 +449,10 @@ __device__ __forceinline__ void real_enc_fwd_ring_body(const PairArgs &p, const 
 }
 
 template <int NT, int DT, bool SELECT>
-__global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p, const float *__restrict__ cache)
+__global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p_, const float *__restrict__ cache)
 {
+    const PairArgs p = with_live_units(p_);
+    if (p.U == 0) return;          // (an empty list: not even the descriptor of unit 0 may be read)
     real_enc_fwd_ring_body<NT, DT, SELECT>(p, cache, (int)blockIdx.x, (int)gridDim.x);
 }
 
@@ -493,6 +496,7 @@ int launch_ring_stage(const float *rpos, const float *tvecs, const int64_t *pair
     p.lattice_range = lattice_range;
     p.bin_step = bin_step; p.s_scale = s_scale; p.inv_bin_step = 1.0f / bin_step;
     p.window = sqrtf(40.0f) / bin_step;
+    p.live_U = live_units(U);
     const float weak_a2 = weak_a * LOG2E;
     const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
     int64_t blocks64 = (U + 3) / 4;
@@ -598,6 +602,8 @@ int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U
     p.window = sqrtf(40.0f) / bin_step;
     p.unit_flags = unit_flags; p.round_flags = round_flags; p.flag_want = 1;      // units that keep the cube
     const bool select = unit_flags != nullptr;
+    p.live_U = live_units(U);
+    if (p.live_U && select) return CF_ERR_UNSUPPORTED;       // (the flags are laid out for a known U)
     const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
     const int DT = D > 16 ? 2 : 1;
     size_t lds = sizeof(float) * ((size_t)WPB * 3 * RS + (size_t)4 * NT * XPLANE + WPB * 16) +
@@ -703,6 +709,9 @@ extern "C" int cf_real_enc_fwd_rings(const float *a_ik, const float *rpos_ij_e, 
     }
     // Adaptive boxes: the units whose columns all keep the cube from the rings, the rest by the
     // pair kernel; both write their own edges of z and v.
+    CF_REQUIRE(!cf::live_units(U), CF_ERR_UNSUPPORTED,
+               "cf_real_enc_fwd_rings: adaptive boxes from the rings need sizes known on the host "
+               "(a size header is set): use cf_real_enc_fwd");
     CF_REQUIRE(minimum_range >= 0 && minimum_range <= MAX_RANGE, CF_ERR_INVALID_ARGUMENT,
                "cf_real_enc_fwd_rings: minimum_range %d outside 0..%d", minimum_range, MAX_RANGE);
     CF_REQUIRE(rpos_ij_e && tvecs_n && batch_i && edge_ij_e, CF_ERR_INVALID_ARGUMENT,

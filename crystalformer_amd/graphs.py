@@ -11,7 +11,8 @@ kernels clear what they need themselves.
 """
 from __future__ import annotations
 
-from typing import Optional
+import contextlib
+from typing import Optional, Tuple
 
 import torch
 
@@ -38,8 +39,19 @@ def _same_layout(owner, batch: CrystalBatch) -> None:
 class GraphedForward:
     """Capture ``model(batch)`` (inference, no autograd) and replay it.
 
-    ``batch`` fixes the layout: later calls may pass a batch with different
-    positions, lattices or species but identical ``sizes``.
+    Without ``capacity``, ``batch`` fixes the layout: later calls may pass a batch with
+    different positions, lattices or species but identical ``sizes``.
+
+    With ``capacity = (crystals, atoms, edges)`` one graph serves ANY batch within those
+    bounds (edges = sum of squared crystal sizes): the buffers and launch grids have the
+    capacity's size, a call copies the batch into their front, and the graph itself works
+    out the index structure and the counts from the crystal sizes on the device
+    (:class:`crystalformer_amd.ops.live_sizes`); nothing is read back to the host, so a new
+    batch costs five small device copies and one submission.  Results are those of an eager
+    forward over the same batch, bit for bit.  A batch with more edges than the capacity
+    cannot be detected without a read-back: the layout kernels turn it into a batch of empty
+    crystals, whose pooled features -- means over no atoms -- and outputs are NaN, and
+    :meth:`overflowed` reports it.
 
     ``launch_share`` (0 < share <= 1) is for several graphs replayed concurrently on
     different streams: the periodic-encoding launches of this graph then take that share
@@ -48,30 +60,82 @@ class GraphedForward:
     """
 
     def __init__(self, model: torch.nn.Module, batch: CrystalBatch, warmup: int = 3,
-                 launch_share: float = 1.0):
+                 launch_share: float = 1.0, capacity: Optional[Tuple[int, int, int]] = None):
         if not batch.pos.is_cuda:
             raise ValueError("GraphedForward needs a batch on the GPU")
         self.model = model
-        self.static = CrystalBatch(batch.x.clone(), batch.pos.clone(), batch.batch.clone(),
-                                   batch.trans_vec.clone(), batch.sizes.clone(),
-                                   None if batch.y is None else batch.y.clone())
-        self._sizes_host = batch.sizes.tolist()
+        self.capacity = None
         self._checked: dict = {}
+        if capacity is None:
+            self.static = CrystalBatch(batch.x.clone(), batch.pos.clone(), batch.batch.clone(),
+                                       batch.trans_vec.clone(), batch.sizes.clone(),
+                                       None if batch.y is None else batch.y.clone())
+            self._sizes_host = batch.sizes.tolist()
+            self._live = contextlib.nullcontext()
+        else:
+            B, N, E = (int(c) for c in capacity)
+            if B < 1 or N < B or E < N:
+                raise ValueError("capacity is (crystals, atoms, edges) with crystals <= atoms <= edges")
+            E += (N + E) % 2                    # (atoms + edges is even for any batch)
+            self.capacity = (B, N, E)
+            dev = batch.pos.device
+            eye = torch.eye(3, dtype=batch.trans_vec.dtype, device=dev)
+            self.static = CrystalBatch(
+                torch.zeros((N,) + tuple(batch.x.shape[1:]), dtype=batch.x.dtype, device=dev),
+                torch.zeros((N, 3), dtype=batch.pos.dtype, device=dev),
+                torch.zeros(N, dtype=torch.int64, device=dev),
+                eye.repeat(B, 1, 1),            # unused slots hold a valid lattice
+                torch.zeros(B, dtype=torch.int64, device=dev), None)
+            self.header = torch.zeros(4, dtype=torch.int64, device=dev)
+            self._live = ops.live_sizes(self.header, N, E)
+            self.crystals = 0
+            self._load(batch)
         self.graph = torch.cuda.CUDAGraph()
         stream = torch.cuda.Stream()            # default priority
         stream.wait_stream(torch.cuda.current_stream())
-        with torch.no_grad(), torch.cuda.stream(stream):
+        with torch.no_grad(), torch.cuda.stream(stream), self._live:
             for _ in range(max(warmup, 1)):     # primes index caches and library workspaces
                 model(self.static)
         torch.cuda.current_stream().wait_stream(stream)
         torch.cuda.synchronize()
-        with torch.no_grad(), ops.launch_share(launch_share), torch.cuda.graph(self.graph):
+        with torch.no_grad(), ops.launch_share(launch_share), self._live, torch.cuda.graph(self.graph):
             self.output = model(self.static)
         # the graph holds raw addresses of the cached index tensors of this layout
         self._keepalive = ops.index_cache_snapshot()
         torch.cuda.synchronize()
 
+    def _load(self, batch: CrystalBatch) -> None:
+        """Copy a batch into the front of the capacity buffers (device copies, no read-back)."""
+        Bc, Nc, _ = self.capacity
+        B, N = batch.sizes.numel(), batch.pos.shape[0]
+        if B > Bc or N > Nc or B < 1:
+            raise ValueError(f"batch of {B} crystals / {N} atoms exceeds the capacity {Bc} / {Nc}")
+        if batch.x.shape[0] != N or batch.batch.numel() != N or batch.trans_vec.shape[0] != B:
+            raise ValueError("inconsistent batch")
+        st = self.static
+        # (the crystal index per atom is not copied: inside the graph the layout kernels write it)
+        moves = [(st.x[:N], batch.x), (st.pos[:N], batch.pos), (st.trans_vec[:B], batch.trans_vec),
+                 (st.sizes[:B], batch.sizes)]
+        if B < self.crystals:                   # slots the previous batch used and this one does not
+            moves.append((st.sizes[B:self.crystals], None))
+        if all(s is None or (s.is_cuda and s.is_contiguous() and s.dtype == d.dtype) for d, s in moves):
+            ops.copy_segments(moves)            # one launch
+        else:
+            for d, s in moves:
+                d.zero_() if s is None else d.copy_(s, non_blocking=True)
+        self.crystals = B
+
+    def overflowed(self) -> bool:
+        """Whether the batch of the last call exceeded the edge capacity (reads the status word
+        back: a host synchronisation, for when the caller has one anyway)."""
+        return self.capacity is not None and bool(self.header[3].item())
+
     def __call__(self, batch: Optional[CrystalBatch] = None) -> torch.Tensor:
+        if self.capacity is not None:
+            if batch is not None and batch is not self.static:
+                self._load(batch)
+            self.graph.replay()
+            return self.output[:self.crystals]
         if batch is not None and batch is not self.static:
             _same_layout(self, batch)
             self.static.x.copy_(batch.x)

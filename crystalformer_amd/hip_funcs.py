@@ -170,7 +170,7 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         # (adaptive boxes too: atom pairs whose half-widths all come out as LATTICE_RANGE have exactly
         # the cube and start from the rings, the others are staged by the pair kernel)
         # (adaptive boxes: on request only, see KernelManager.ADAPTIVE_RINGS)
-        worth_it = fixed_cube or KernelManager.ADAPTIVE_RINGS
+        worth_it = fixed_cube or (KernelManager.ADAPTIVE_RINGS and ops.current_live_sizes() is None)
         if (KernelManager.STAGED_RINGS and KernelManager.WEAKEST_EXPONENT is not None and pairs_u is not None
                 and worth_it and K > 0 and W_k is not None and _w_leading(W_k) == 1 and W_k.shape[-2] <= 32):
             rings = ops.staged_rings(rpos_ij_e, tvecs_n, pairs_u, K, dist_max, wscale, KernelManager.LATTICE_RANGE,
@@ -299,6 +299,8 @@ def fused_encoding_attention(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, que_i
     rows too long for it, row lengths unknown under stream capture): the caller then runs the two
     operators."""
     if not KernelManager.FUSE_ENCODING_ATTENTION or not a_ik.is_cuda:
+        return None
+    if ops.current_live_sizes() is not None:          # (its row bound would have to be read back)
         return None
     if torch.cuda.is_current_stream_capturing() and not KernelManager.FUSE_ENCODING_ATTENTION_IN_GRAPHS:
         return None

@@ -31,6 +31,8 @@ SIGNATURES = {
     "cf_max_translation_range": (_int, []),
     "cf_set_launch_share": (_int, [_dbl]),
     "cf_get_launch_share": (_dbl, []),
+    "cf_set_size_header": (_int, [_ptr, _i64, _i64]),
+    "cf_get_size_header": (_ptr, []),
     "cf_real_enc_fwd": (_int, [_ptr] * 5 + [_i64] * 6 + [_dbl, _dbl, _ptr, _i64, _ptr, _dbl, _int, _int,
                                                          _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
     "cf_real_enc_ring_bytes": (_i64, [_i64]),
@@ -72,7 +74,8 @@ SIGNATURES = {
     "cf_adamw_step": (_int, [_int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _f32, _f32, _f32, _f32, _f32, _f32, _ptr,
                              _ptr, _i64, _ptr]),
     "cf_l1_mean_loss": (_int, [_ptr, _ptr, _i64, _i64, _ptr, _ptr, _ptr]),
-    "cf_batch_layout": (_int, [_ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "cf_batch_layout": (_int, [_ptr, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "cf_copy_segments": (_int, [_int, _ptr, _ptr, _ptr, _ptr]),
     "cf_lattice_geometry": (_int, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
     "cf_gauss_exponents_workspace": (_i64, [_i64, _i64]),
     "cf_gauss_exponents": (_int, [_ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _int, _int, _f32, _f32, _f32, _f32,

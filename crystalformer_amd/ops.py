@@ -4,6 +4,7 @@ torch, pass raw device pointers and torch's current stream.  No autograd here
 """
 from __future__ import annotations
 
+import threading
 from typing import Optional, Tuple
 
 import torch
@@ -65,6 +66,45 @@ class launch_share:
     def __exit__(self, *exc):
         check(_lib.load().cf_set_launch_share(self.previous), "cf_set_launch_share")
         return False
+
+
+class live_sizes:
+    """Context manager: within it the operators of this thread take the atom, edge and pair counts
+    of a batch from ``header`` (4 int64 words on the device: atoms, edges, atom pairs, status) instead
+    of from their arguments, whose sizes are then capacities (``cf_set_size_header``).  For one set
+    of buffers -- one captured graph -- served to batches whose crystal sizes differ:
+    :func:`batch_layout` called inside fills the header from ``sizes`` as it finds it when its
+    kernels run, without reading anything back to the host, and every tensor downstream has the
+    capacity's shape with the live items in front.  A captured graph keeps the header's address."""
+
+    def __init__(self, header: Tensor, atom_capacity: int, edge_capacity: int):
+        if header.dtype != torch.int64 or header.numel() != 4 or not header.is_cuda or not header.is_contiguous():
+            raise _lib.CrystalformerHipError("live_sizes: the header is 4 contiguous int64 words on the GPU")
+        self.header, self.atoms, self.edges = header, int(atom_capacity), int(edge_capacity)
+        self.units = (self.atoms + self.edges) // 2
+        self.previous = None
+
+    def __enter__(self):
+        self.previous = getattr(_live, "current", None)
+        check(_lib.load().cf_set_size_header(ptr(self.header), self.atoms, self.edges), "cf_set_size_header")
+        _live.current = self
+        return self
+
+    def __exit__(self, *exc):
+        prev = self.previous
+        _live.current = prev
+        if prev is None:
+            check(_lib.load().cf_set_size_header(None, 0, 0), "cf_set_size_header")
+        else:
+            check(_lib.load().cf_set_size_header(ptr(prev.header), prev.atoms, prev.edges), "cf_set_size_header")
+        return False
+
+
+_live = threading.local()
+
+
+def current_live_sizes() -> Optional[live_sizes]:
+    return getattr(_live, "current", None)
 
 
 class _timed:
@@ -687,6 +727,9 @@ def batch_layout(sizes: Tensor, batch_i: Tensor) -> BatchLayout:
     """Layout for ``sizes`` (B,) / ``batch_i`` (N,), cached on the identity and version
     of both tensors.  ``layout.batch`` is ``batch_i`` renumbered from 0.  The derived
     tensors are also entered in the index caches under the keys the operators use."""
+    live = current_live_sizes()
+    if live is not None:
+        return _live_batch_layout(sizes, batch_i, live)
     sig, hit = _cache_lookup("layout", sizes, batch_i)
     if hit is not None:
         return hit
@@ -719,22 +762,82 @@ def batch_layout(sizes: Tensor, batch_i: Tensor) -> BatchLayout:
         lay.pairs = torch.empty(((E + N) // 2, PAIR_FIELDS), dtype=torch.int64, device=dev)
         with device_guard(dev):
             rc = _lib.load().cf_batch_layout(ptr(sizes), B, N, E, ptr(starts[0]), ptr(starts[1]), ptr(starts[2]),
-                                             ptr(lay.e_start), ptr(lay.edges), ptr(lay.pairs), stream_handle(dev))
+                                             ptr(lay.e_start), ptr(lay.edges), ptr(lay.pairs), None,
+                                             stream_handle(dev))
         check(rc, "cf_batch_layout")
+    _enter_layout(lay, max(sizes_host) if sizes_host else 0)
+    return _cache_store(sig, (sizes, batch_i), lay)
+
+
+def _enter_layout(lay: BatchLayout, max_row: Optional[int]) -> None:
+    """The derived tensors of a layout under the keys the operators look them up with."""
     s_, _ = _cache_lookup("e_start", lay.edges)
     _cache_store(s_, (lay.edges,), lay.e_start)
     if lay.pairs is not None:
         s_, _ = _cache_lookup("pairs", lay.batch, lay.edges)
         _cache_store(s_, (lay.batch, lay.edges), lay.pairs)
-    s_, _ = _cache_lookup("max_row", lay.edges)                # a row has as many edges as its crystal atoms
-    _cache_store(s_, (lay.edges,), max(sizes_host) if sizes_host else 0)
+    if max_row is not None:
+        s_, _ = _cache_lookup("max_row", lay.edges)            # a row has as many edges as its crystal atoms
+        _cache_store(s_, (lay.edges,), max_row)
     s_, _ = _cache_lookup("dense", lay.batch, lay.edges)       # dense by construction
-    _cache_store(s_, (lay.batch, lay.edges), (sizes,))
+    _cache_store(s_, (lay.batch, lay.edges), (lay.sizes,))
     s_, _ = _cache_lookup("offsets", lay.batch)
     _cache_store(s_, (lay.batch,), (lay.atom_start, lay.edge_start))
-    s_, _ = _cache_lookup("mean_start", sizes)
-    _cache_store(s_, (sizes,), lay.atom_start)
-    return _cache_store(sig, (sizes, batch_i), lay)
+    s_, _ = _cache_lookup("mean_start", lay.sizes)
+    _cache_store(s_, (lay.sizes,), lay.atom_start)
+
+
+def _live_batch_layout(sizes: Tensor, batch_i: Tensor, live: "live_sizes") -> BatchLayout:
+    """:func:`batch_layout` inside :class:`live_sizes`: every tensor has the capacity's shape, the
+    kernels work out the counts from ``sizes`` (crystals past the live ones hold 0) and leave them
+    in the header.  Nothing is read back and nothing is cached on ``sizes``, whose contents change
+    from one use of the buffers to the next."""
+    dev = require_device(sizes, batch_i, live.header)
+    sizes = _i64(sizes, "sizes")
+    N, E = live.atoms, live.edges
+    B = sizes.numel()
+    if batch_i.numel() != N:
+        raise _lib.CrystalformerHipError(
+            f"live sizes: batch has {batch_i.numel()} entries, the atom capacity is {N}")
+    if B < 1:
+        raise _lib.CrystalformerHipError("live sizes: no crystal slots")
+    lay = BatchLayout()
+    lay.sizes = sizes
+    lay.batch = torch.empty(N, dtype=torch.int64, device=dev)      # written by the layout kernels
+    lay.num_atoms, lay.num_edges = N, E
+    starts = torch.empty((3, B + 1), dtype=torch.int64, device=dev)
+    lay.atom_start, lay.edge_start = starts[0], starts[1]
+    lay.e_start = torch.empty(N + 1, dtype=torch.int64, device=dev)
+    lay.edges = torch.empty((2, E), dtype=torch.int64, device=dev)
+    lay.pairs = torch.empty((live.units, PAIR_FIELDS), dtype=torch.int64, device=dev)
+    with device_guard(dev):
+        rc = _lib.load().cf_batch_layout(ptr(sizes), B, N, E, ptr(starts[0]), ptr(starts[1]), ptr(starts[2]),
+                                         ptr(lay.e_start), ptr(lay.edges), ptr(lay.pairs), ptr(lay.batch),
+                                         stream_handle(dev))
+    check(rc, "cf_batch_layout")
+    _enter_layout(lay, None)
+    return lay
+
+
+def copy_segments(pairs) -> None:
+    """``dst.copy_(src)`` for up to eight ``(dst, src)`` pairs of contiguous tensors on one GPU in a
+    single launch; ``src`` None fills ``dst`` with zeros.  Element counts and types must agree."""
+    import ctypes
+    pairs = [(d, s) for d, s in pairs if d.numel() > 0]
+    if not pairs:
+        return
+    dev = require_device(*[t for pr in pairs for t in pr if t is not None])
+    for d, s in pairs:
+        if not d.is_contiguous() or (s is not None and (not s.is_contiguous() or s.dtype != d.dtype
+                                                         or s.numel() != d.numel())):
+            raise _lib.CrystalformerHipError("copy_segments: contiguous tensors of equal type and size expected")
+    n = len(pairs)
+    src = (ctypes.c_void_p * n)(*[None if s is None else s.data_ptr() for _, s in pairs])
+    dst = (ctypes.c_void_p * n)(*[d.data_ptr() for d, _ in pairs])
+    nbytes = (ctypes.c_int64 * n)(*[d.numel() * d.element_size() for d, _ in pairs])
+    with device_guard(dev):
+        rc = _lib.load().cf_copy_segments(n, src, dst, nbytes, stream_handle(dev))
+    check(rc, "cf_copy_segments")
 
 
 def relative_positions(layout: BatchLayout, pos: Tensor) -> Tensor:

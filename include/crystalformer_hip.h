@@ -54,6 +54,31 @@ int cf_set_launch_share(double share);
 double cf_get_launch_share(void);
 
 /*
+ * Batch sizes that only the device knows, for the calling thread.  For callers that replay ONE
+ * captured graph (or keep one set of buffers) over batches whose crystal sizes differ: buffers
+ * and launch grids are sized for capacities, and the live counts are read on the device.  No
+ * counterpart in the reference, whose wrappers read the sizes back to the host on every call
+ * (models/cuda_funcs/fused_dpa.py:73,137; models/cuda_funcs/irregular_mean.py:29-36).
+ *
+ *   header_4  DEVICE, four int64 words: live atoms N, live edges E, live atom pairs U, status.
+ *             cf_batch_layout writes them from `sizes_n` as it finds it when its kernels run
+ *             (status 1 and N = E = U = 0 when a size is negative or the totals exceed the
+ *             capacities: every kernel below then does nothing).  NULL switches the mode off.
+ *   N_cap, E_cap  the capacities; their sum must be even (U_cap = (N_cap + E_cap) / 2).
+ * While a header is set, an entry point listed here that is called with N == N_cap (E == E_cap,
+ * U == U_cap) takes that argument as the capacity -- array strides, launch grid -- and works on
+ * the first live N (E, U) items only; results for those are bit-identical to a call with the
+ * live sizes as arguments.  Entry points: cf_batch_layout, cf_edge_index, cf_edge_pairs,
+ * cf_gauss_exponents, cf_linear_rows (rows = atoms), cf_real_enc_ring_stage,
+ * cf_real_enc_fwd_rings (fixed cube), cf_real_enc_fwd (pair list), cf_fused_dpa_fwd.  The other
+ * entry points ignore the header (per-crystal ones run over all B lattices handed in; crystals
+ * beyond the live ones must have size 0).  Read at launch: a captured graph keeps the header
+ * address it was captured with.
+ */
+int cf_set_size_header(int64_t *header_4, int64_t N_cap, int64_t E_cap);
+const int64_t *cf_get_size_header(void);
+
+/*
  * Real-space periodic encoding, forward.
  * Replaces the launches of real_enc_fwd / real_enc_proj_fwd
  * (models/cuda_funcs/real_space_enc.py:96-113,
@@ -509,10 +534,25 @@ int cf_adamw_step(int n_tensors, float *const *params, const float *const *grads
  *   atom_start_n, edge_start_n, unit_start_n (B+1): leading-zero cumulative sums of n, n^2,
  *       n (n + 1) / 2
  *   e_start_i (N+1), edge_ij_e (2,E), pairs_u ((E+N)/2, 5) or NULL
+ *   batch_i (N) or NULL: crystal of each atom, numbered from 0 (what the data loader's `batch`
+ *       holds after the rebasing of models/indexed_latticeformer_encoder.py:436,722)
+ * With a size header set for (N, E) (cf_set_size_header) N and E are capacities, `sizes_n` may hold
+ * zeros past the live crystals, and the header is written here.
  */
 int cf_batch_layout(const int64_t *sizes_n, int64_t B, int64_t N, int64_t E, int64_t *atom_start_n,
                     int64_t *edge_start_n, int64_t *unit_start_n, int64_t *e_start_i, int64_t *edge_ij_e,
-                    int64_t *pairs_u, void *stream);
+                    int64_t *pairs_u, int64_t *batch_i, void *stream);
+
+/*
+ * Up to 8 device-to-device copies in one launch: dst[s][0..bytes[s]) = src[s][0..bytes[s]), or
+ * zeros where src[s] is NULL.  src, dst, bytes: HOST arrays of n_segments entries (device
+ * addresses, read at call time and passed to the kernel by value).  Segments must not overlap.
+ * For a caller that refreshes the input buffers of a captured graph with a new batch (features,
+ * positions, lattices, sizes): one launch instead of one per tensor.  No counterpart in the
+ * reference, which hands every batch to its kernels in the loader's own tensors.
+ */
+int cf_copy_segments(int n_segments, const void *const *src, void *const *dst, const int64_t *bytes,
+                     void *stream);
 
 /*
  * Training loss of the regression module and its gradient in one launch: the per-sample

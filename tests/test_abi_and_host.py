@@ -97,6 +97,27 @@ def test_launch_share_is_validated_and_per_thread():
     assert L.cf_get_launch_share() == 1.0
 
 
+def test_size_header_is_validated_and_per_thread():
+    """cf_set_size_header stores a device address and two capacities for the calling thread;
+    nothing is launched and nothing at the address is touched."""
+    import threading
+    L = lib.load()
+    assert not L.cf_get_size_header()
+    fake = ctypes.c_void_p(4096)
+    for n_cap, e_cap in ((0, 10), (10, 0), (-2, 4), (10, 11)):       # non-positive, odd sum
+        assert L.cf_set_size_header(fake, n_cap, e_cap) == -1 and b"capacities" in L.cf_last_error()
+        assert not L.cf_get_size_header()
+    assert L.cf_set_size_header(fake, 10, 12) == 0 and L.cf_get_size_header() == 4096
+    seen = []
+    t = threading.Thread(target=lambda: seen.append(L.cf_get_size_header()))
+    t.start()
+    t.join()
+    assert seen == [None]
+    assert L.cf_set_size_header(None, 0, 0) == 0 and not L.cf_get_size_header()
+    with pytest.raises(lib.CrystalformerHipError, match="header"):
+        ops.live_sizes(torch.zeros(4, dtype=torch.int64), 10, 12)    # a CPU tensor
+
+
 def test_operators_refuse_cpu_tensors():
     a = torch.zeros(2, 8)
     with pytest.raises(lib.CrystalformerHipError, match="no CPU fallback"):

@@ -388,6 +388,53 @@ def test_graph_replay_matches_eager(dev):
     assert torch.equal(graphed(b), y_eager)
 
 
+@pytest.mark.parametrize("rule", ["A", "B"])
+def test_one_graph_serves_batches_of_any_size(dev, rule):
+    """One captured graph with capacity buffers replayed over batches whose crystal sizes, atom,
+    edge and crystal counts all differ (the counts are worked out on the device, nothing is read
+    back): every replay equals the eager forward over that batch bit for bit, including after a
+    larger batch has left its data behind in the buffers; an empty-handed overflow of the edge
+    capacity yields NaN and is reported."""
+    from crystalformer_amd.graphs import GraphedForward
+    from crystalformer_amd.synthetic import make_batch
+    over = dict(adaptive_cutoff_sigma=0.0) if rule == "A" else dict()
+    cfg, model = build_model("cfg2_default_b128", num_layers=2, **over)
+    model.to(dev).eval()
+    shapes = [(24, (1, 40), 11), (40, (1, 64), 12), (7, (1, 9), 13), (33, (2, 30), 14), (1, (17, 17), 15),
+              (40, (1, 64), 16), (12, (1, 5), 17)]
+    batches = [make_batch(n, sr, True, (3.0, 15.0), (60.0, 120.0), seed=s).to(dev) for n, sr, s in shapes]
+    assert len({(b.sizes.numel(), b.pos.shape[0], b.num_edges) for b in batches}) == len(batches)
+    eager = []
+    with torch.no_grad():
+        for b in batches:
+            eager.append(model(b).clone())
+    cap = (48, max(b.pos.shape[0] for b in batches) + 37, max(b.num_edges for b in batches) + 1001)
+    graphed = GraphedForward(model, batches[0], capacity=cap)
+    for rep in range(2):
+        for k in ([0, 1, 2, 3, 4, 5, 6] if rep == 0 else [5, 6, 1, 4, 2]):
+            y = graphed(batches[k]).clone()
+            torch.cuda.synchronize()
+            assert y.shape == eager[k].shape
+            assert torch.equal(y, eager[k]), (rule, rep, k, float((y - eager[k]).abs().max()))
+            with torch.no_grad():
+                assert torch.equal(model(batches[k]), eager[k])        # eager work between replays
+    assert not graphed.overflowed()
+    assert ops.current_live_sizes() is None and lib_header_is_clear()
+    # more edges than the capacity (one crystal of 150 atoms: 22 500 edges) cannot be seen on the host
+    small = GraphedForward(model, batches[2], capacity=(8, 200, 4000))
+    big = make_batch(1, (150, 150), False, (3.0, 15.0), (60.0, 120.0), seed=21).to(dev)
+    y = small(big)
+    assert small.overflowed() and bool(torch.isnan(y).all())
+    assert torch.equal(small(batches[2]), eager[2]) and not small.overflowed()
+    with pytest.raises(ValueError):
+        small(batches[1])                                                # atoms beyond the capacity: seen on the host
+
+
+def lib_header_is_clear():
+    from crystalformer_amd import lib
+    return not lib.load().cf_get_size_header()
+
+
 def test_graphs_in_flight_with_a_launch_share(dev):
     """Four graphs of the same model captured with a launch share below 1 and replayed round robin
     on four streams (the benchmark's throughput mode): every replay equals the eager result bit
