@@ -321,7 +321,8 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                 proj = proj.expand(proj.shape[0], H, proj.shape[2], proj.shape[3])
             attn = None
             if (P.value_pe_dist_real <= 0 and qs is not None and not need_weights and P.norm_func_mode == 0
-                    and config.REPRODUCIBLITY_STATE >= 2 and batch_q is batch_kv and not torch.is_grad_enabled()):
+                    and config.REPRODUCIBLITY_STATE >= 2 and batch_q is batch_kv and not torch.is_grad_enabled()
+                    and not (self.training and self.dropout > 0.0)):     # (dropout on the weights: the loop below)
                 # no value bins and nobody asks for the bias: lattice sums and attention in one launch
                 attn = hip_funcs.fused_encoding_attention(a, points, tvecs, batch_q, edges, qs, k, v, *adaptive)
             if attn is None:
@@ -329,12 +330,9 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                 # every positive map keeps rho >= gauss_lb, so no exponent of this block lies above this bound
                 # (it lets the encoding share its staged translations between the blocks of a model)
                 # (a few ulps of slack for the positive map's own rounding)
-                hip_funcs.KernelManager.WEAKEST_EXPONENT = -0.5 * P.gauss_lb_real * P.scale_real ** -2 * (1 - 1e-5)
-                try:
-                    out = hip_funcs.call(enc, a, points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real,
-                                         dist_max, P.value_pe_width_scale, proj, *adaptive)
-                finally:
-                    hip_funcs.KernelManager.WEAKEST_EXPONENT = None
+                weakest = -0.5 * P.gauss_lb_real * P.scale_real ** -2 * (1 - 1e-5)
+                out = hip_funcs.call(enc, a, points, dist2_min, tvecs, batch_q, edges, P.value_pe_dist_real,
+                                     dist_max, P.value_pe_width_scale, proj, *(adaptive or (None, None)), weakest)
                 bias = out[0]
                 values = out[1] if len(out) >= 2 else None
             else:

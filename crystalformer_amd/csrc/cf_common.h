@@ -7,16 +7,13 @@
 #include <stdio.h>
 
 #include "../../include/crystalformer_hip.h"
+#include "cf_index_rules.h"
 
 namespace cf {
 
 constexpr int WAVE = 64;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
-// The reference kernels divide by 2.0 * CUDART_PI_F (the float constant widened
-// to double); the translation half-widths are only bit-exact with that value.
-constexpr float PI_F = 3.141592654f;
-constexpr int MAX_RANGE = 64;
 
 // ---- error reporting -------------------------------------------------------
 void set_error(const char *fmt, ...);
@@ -231,40 +228,6 @@ __device__ __forceinline__ void wave_mem_sync()
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-}
-
-// Translation half-width along one axis: ceil((cutoff+0.01f)*rvl / (2*pi)),
-// float product, double quotient.  The double division only runs where it can
-// matter: a float quotient is within 1.3e-7 relative of the exact one, so its
-// ceiling is already the answer unless it lies that close to an integer.
-__device__ __forceinline__ int range_axis(float cutoff, float rvl, int minimum_range)
-{
-    const float num = (cutoff + 0.01f) * rvl;
-    const float qf = num * (float)(1.0 / (2.0 * (double)PI_F));
-    int r;
-    if (fabsf(qf - rintf(qf)) > 1.0e-6f * fabsf(qf) && fabsf(qf) < 1.0e6f) {
-        const float c = ceilf(qf);
-        r = c <= 0.f ? 0 : (c > (float)MAX_RANGE ? MAX_RANGE : (int)c);
-    } else {
-        const double q = ceil((double)num / (2.0 * (double)PI_F));
-        r = (q >= 0.0 && q <= (double)MAX_RANGE) ? (int)q : (q > (double)MAX_RANGE ? MAX_RANGE : 0);
-        if (q != q) r = MAX_RANGE;  // NaN exponent: bounded loop, result is NaN anyway
-    }
-    return max(r, minimum_range);
-}
-
-// Half-widths for one (atom, head).  cutoff == 0 selects the fixed cube.
-__device__ __forceinline__ void range_rule(float a, float cutoff, const float *rvl,
-                                           int lattice_range, int minimum_range,
-                                           int &R1, int &R2, int &R3)
-{
-    R1 = R2 = R3 = lattice_range;
-    if (cutoff != 0.0f) {
-        if (cutoff < 0.0f) cutoff = sqrtf(-0.5f / a) * (-cutoff);
-        R1 = range_axis(cutoff, rvl[0], minimum_range);
-        R2 = range_axis(cutoff, rvl[1], minimum_range);
-        R3 = range_axis(cutoff, rvl[2], minimum_range);
-    }
 }
 
 #endif  // __HIPCC__

@@ -50,16 +50,8 @@ __global__ void edge_index_kernel(const int64_t *atom_start, const int64_t *edge
 {
     int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= live_count(live_E, E)) return;
-    int64_t lo = 0, hi = B;   // invariant: edge_start[lo] <= e < edge_start[hi]
-    while (hi - lo > 1) {
-        int64_t mid = (lo + hi) >> 1;
-        if (edge_start[mid] <= e) lo = mid; else hi = mid;
-    }
-    const int64_t a0 = atom_start[lo];
-    const int64_t n = atom_start[lo + 1] - a0;
-    const int64_t local = e - edge_start[lo];
-    const int64_t il = local / n;
-    const int64_t i = a0 + il, j = a0 + (local - il * n);
+    const EdgeEnds r = edge_ends(atom_start, edge_start, B, e);
+    const int64_t i = r.i, j = r.j;
     if (edges) {
         edges[e] = i;
         edges[E + e] = j;
@@ -146,13 +138,8 @@ __global__ void layout_rows_kernel(const int64_t *atom_start, const int64_t *edg
         e_start[N] = edge_start[B];
         return;
     }
-    int64_t lo = 0, hi = B;   // invariant: atom_start[lo] <= i < atom_start[hi]
-    while (hi - lo > 1) {
-        const int64_t mid = (lo + hi) >> 1;
-        if (atom_start[mid] <= i) lo = mid; else hi = mid;
-    }
-    const int64_t a0 = atom_start[lo];
-    e_start[i] = edge_start[lo] + (i - a0) * (atom_start[lo + 1] - a0);
+    int64_t lo;
+    e_start[i] = row_start(atom_start, edge_start, B, i, &lo);
     if (batch) batch[i] = lo;
 }
 

@@ -244,6 +244,12 @@ __global__ __launch_bounds__(1024) void enc_dpa_row_kernel(EncArgs p, RowArgs r)
         for (int x = threadIdx.x; x < H * Dv; x += blockDim.x) r.out[i * H * Dv + x] = 0.f;
         return;
     }
+    if (n > r.max_row) {
+        // a row longer than the bound the caller gave (the LDS was sized with it): nothing of the
+        // row may be staged; the output row is NaN so that the broken promise cannot pass for a result
+        for (int x = threadIdx.x; x < H * Dv; x += blockDim.x) r.out[i * H * Dv + x] = __builtin_nanf("");
+        return;
+    }
     // ---- phase 1: lattice sums of the row
     {
         const int64_t nb = p.batch[i];

@@ -50,25 +50,15 @@ __global__ void edge_pairs_kernel(const int64_t *atom_start, const int64_t *edge
 {
     int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= live_count(live_E, E)) return;
-    int64_t lo = 0, hi = B;
-    while (hi - lo > 1) {
-        int64_t mid = (lo + hi) >> 1;
-        if (edge_start[mid] <= e) lo = mid; else hi = mid;
-    }
-    const int64_t a0 = atom_start[lo];
-    const int64_t n = atom_start[lo + 1] - a0;
-    const int64_t e0 = edge_start[lo];
-    const int64_t local = e - e0;
-    const int64_t il = local / n, jl = local - il * n;
-    if (il > jl) return;
-    // row il of the upper triangle starts after il*n - il*(il-1)/2 units
-    const int64_t u = unit_start[lo] + il * n - (il * (il - 1)) / 2 + (jl - il);
+    const EdgeEnds r = edge_ends(atom_start, edge_start, B, e);
+    const int64_t u = unit_of_edge(r, unit_start[r.crystal]);
+    if (u < 0) return;                    // (i > j: the reverse edge owns the unit)
     int64_t *d = pairs + PAIR_FIELDS * u;
     d[0] = e;
-    d[1] = e0 + jl * n + il;
-    d[2] = a0 + il;
-    d[3] = a0 + jl;
-    d[4] = lo;
+    d[1] = reverse_edge(r);
+    d[2] = r.i;
+    d[3] = r.j;
+    d[4] = r.crystal;
 }
 
 }  // namespace

@@ -80,9 +80,9 @@ class KernelManager:
     # Fixed cube: the geometry-only part of the encoding (which translations reach a bin, in which
     # order, their distances) is staged once per forward pass and shared by all blocks
     # (ops.staged_rings).  Needs an upper bound of the exponents the rings will meet, which the
-    # attention module sets around its call (-gauss_lb / (2 r0^2)); None: every launch stages for itself.
+    # attention module passes with its call (-gauss_lb / (2 r0^2), the encoding Function's last
+    # argument); without one every launch stages for itself.
     STAGED_RINGS: bool = True
-    WEAKEST_EXPONENT: Optional[float] = None
     # Adaptive boxes from the staged rings (forward): atom pairs whose half-widths all come out as
     # LATTICE_RANGE start from their rings, the others are staged by the pair kernel's body in the same
     # launch.  Off by default: it pays where nearly all pairs keep the cube (default model, inference, 128
@@ -142,9 +142,24 @@ def call(function, *args):
     return function.forward(_NoGradCtx(), *args)
 
 
-def _enc_backward_tail(ga_ik, gW_k, has_adaptive_args: bool):
-    base = (ga_ik, None, None, None, None, None, None, None, None, gW_k)
-    return base + (None, None) if has_adaptive_args else base
+class _Absent:
+    """Default of the optional trailing arguments of the encoding Functions: tells an argument that
+    was not passed from one passed as None (backward returns one gradient per argument passed)."""
+
+    def __repr__(self):
+        return "<not passed>"
+
+
+_ABSENT = _Absent()
+
+
+def _optional_args(*values):
+    """(values with the absent ones as None, number of them that were passed)."""
+    return tuple(None if v is _ABSENT else v for v in values), sum(v is not _ABSENT for v in values)
+
+
+def _enc_backward_tail(ga_ik, gW_k, optional_passed: int):
+    return (ga_ik, None, None, None, None, None, None, None, None, gW_k) + (None,) * optional_passed
 
 
 class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
@@ -157,7 +172,13 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale,
-                W_k, rvlen_n=None, cutoff_radius=None):
+                W_k, rvlen_n=_ABSENT, cutoff_radius=_ABSENT, weakest_exponent=_ABSENT):
+        """``weakest_exponent`` (an extension, after the reference's arguments): an upper bound
+        (<= 0) of every entry of ``a_ik``, e.g. -gauss_lb / (2 r0^2).  With it the geometry-only part
+        of the encoding is staged once per geometry and shared by the blocks of a model
+        (:func:`crystalformer_amd.ops.staged_rings`); without, every call stages for itself."""
+        (rvlen_n, cutoff_radius, weakest_exponent), ctx.optional_passed = _optional_args(
+            rvlen_n, cutoff_radius, weakest_exponent)
         a_ik = a_ik.contiguous().detach()
         rpos_ij_e = rpos_ij_e.contiguous()
         tvecs_n = tvecs_n.contiguous()
@@ -171,10 +192,10 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         # the cube and start from the rings, the others are staged by the pair kernel)
         # (adaptive boxes: on request only, see KernelManager.ADAPTIVE_RINGS)
         worth_it = fixed_cube or (KernelManager.ADAPTIVE_RINGS and ops.current_live_sizes() is None)
-        if (KernelManager.STAGED_RINGS and KernelManager.WEAKEST_EXPONENT is not None and pairs_u is not None
+        if (KernelManager.STAGED_RINGS and weakest_exponent is not None and pairs_u is not None
                 and worth_it and K > 0 and W_k is not None and _w_leading(W_k) == 1 and W_k.shape[-2] <= 32):
             rings = ops.staged_rings(rpos_ij_e, tvecs_n, pairs_u, K, dist_max, wscale, KernelManager.LATTICE_RANGE,
-                                     KernelManager.WEAKEST_EXPONENT)
+                                     float(weakest_exponent))
         if rings is not None:
             z_ek, v_ekd = ops.real_enc_fwd_rings(
                 a_ik, edge_ij_e, pairs_u, rings, K, dist_max, wscale, W_k, KernelManager.LATTICE_RANGE,
@@ -187,7 +208,6 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         ctx.save_for_backward(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n, W_k, z_ek)
         ctx.K, ctx.dist_max, ctx.wscale, ctx.cutoff_radius = K, dist_max, wscale, cutoff_radius
         ctx.ranges = (KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
-        ctx.adaptive_args = rvlen_n is not None
         # the backward's pair kernel (K <= 64, D <= 16) starts from the same staged translations
         ctx.rings = rings if (rings is not None and fixed_cube and K <= 64 and W_k.shape[-2] <= 16) else None
         if K <= 0:
@@ -205,7 +225,7 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
             ctx.wscale, W_k, rvlen_n, ctx.cutoff_radius, ctx.ranges[0], ctx.ranges[1],
             want_gW=W_k is not None and ctx.needs_input_grad[9],
             pairs_u=_pairs(batch_i, edge_ij_e, tvecs_n, ctx.K), rings=ctx.rings)
-        return _enc_backward_tail(ga_ik, gW_k, ctx.adaptive_args)
+        return _enc_backward_tail(ga_ik, gW_k, ctx.optional_passed)
 
 
 class RealPeriodicEncodingFuncCUDA(torch.autograd.Function):
@@ -215,7 +235,9 @@ class RealPeriodicEncodingFuncCUDA(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale,
-                W_k, rvlen_n=None, cutoff_radius=None):
+                W_k, rvlen_n=_ABSENT, cutoff_radius=_ABSENT, weakest_exponent=_ABSENT):
+        # (weakest_exponent: accepted for a common call signature; this path stages per call)
+        (rvlen_n, cutoff_radius, _), ctx.optional_passed = _optional_args(rvlen_n, cutoff_radius, weakest_exponent)
         a_ik = a_ik.contiguous().detach()
         rpos_ij_e = rpos_ij_e.contiguous()
         tvecs_n = tvecs_n.contiguous()
@@ -237,7 +259,6 @@ class RealPeriodicEncodingFuncCUDA(torch.autograd.Function):
                               s_ekk if W_k is not None else None)
         ctx.K, ctx.dist_max, ctx.wscale, ctx.cutoff_radius = K, dist_max, wscale, cutoff_radius
         ctx.ranges = (KernelManager.LATTICE_RANGE, KernelManager.MINIMUM_RANGE)
-        ctx.adaptive_args = rvlen_n is not None
         if K <= 0:
             return (z_ek,)
         return z_ek, v_out
@@ -256,7 +277,7 @@ class RealPeriodicEncodingFuncCUDA(torch.autograd.Function):
         ga_ik, _ = ops.real_enc_bwd(
             a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz, gv, ctx.K, ctx.dist_max,
             ctx.wscale, None, rvlen_n, ctx.cutoff_radius, ctx.ranges[0], ctx.ranges[1], want_gW=False)
-        return _enc_backward_tail(ga_ik, gW_k, ctx.adaptive_args)
+        return _enc_backward_tail(ga_ik, gW_k, ctx.optional_passed)
 
 
 def _dpa_forward(ctx, que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e):

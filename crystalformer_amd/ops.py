@@ -289,9 +289,11 @@ def staged_rings(rpos_ij_e: Tensor, tvecs_n: Tensor, pairs_u: Tensor, K: int, di
         return None
     # (a launch recorded into a graph and an eager one never share a buffer: a replay stages again)
     dev = require_device(rpos_ij_e, tvecs_n, pairs_u)
+    # (the stream is part of the key: rings staged on one stream are not handed to work on another,
+    # which nothing orders behind the staging)
     sig = tuple((t.data_ptr(), tuple(t.shape), t._version) for t in (rpos_ij_e, tvecs_n, pairs_u)) + \
-        (bool(torch.cuda.is_current_stream_capturing()), int(K), float(dist_max), float(wscale),
-         int(lattice_range), float(weakest_exponent))
+        (bool(torch.cuda.is_current_stream_capturing()), stream_handle(dev), int(K), float(dist_max),
+         float(wscale), int(lattice_range), float(weakest_exponent))
     for entry in _ring_cache:
         if entry[0] == sig:
             return entry[2]
@@ -319,7 +321,7 @@ def real_enc_fwd_rings(a_ik: Tensor, edge_ij_e: Tensor, pairs_u: Tensor, rings: 
     they were staged for).  Fixed cube: every atom pair starts from its ring.  Adaptive boxes
     (``rvlen_n`` and a non-zero ``cutoff_radius``; needs ``rpos_ij_e``, ``tvecs_n`` and ``batch_i`` too):
     the pairs whose half-widths all come out as ``lattice_range`` start from their rings, the others are
-    staged by the pair kernel in a second launch."""
+    staged by the pair kernel's body; a selection launch, then one launch with both roles."""
     dev = require_device(a_ik, edge_ij_e, pairs_u, rings, W_k, rpos_ij_e, tvecs_n, batch_i, rvlen_n)
     a_ik, W_k = _f32(a_ik, "a_ik"), _f32(W_k, "W_k")
     pairs_u, edge_ij_e = _i64(pairs_u, "pairs_u"), _i64(edge_ij_e, "edge_ij_e")

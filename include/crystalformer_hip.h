@@ -144,9 +144,13 @@ int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvec
  * Adaptive boxes (rvlen_n given and cutoff_radius != 0, the rule of
  * models/kernels/real_enc_fwd.cu:58-85): atom pairs whose (atom, head) half-widths all come out as
  * lattice_range have exactly the cube and are evaluated from the rings; the others are staged and
- * evaluated as cf_real_enc_fwd does.  Three launches (selection, rings, rest) that share `flags`,
- * cf_real_enc_flag_bytes(U, H) bytes of device scratch written and read by the call.  With the fixed
- * cube rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n and flags may be NULL.
+ * evaluated as cf_real_enc_fwd does.  Two launches: the selection (the range rule per atom pair and
+ * head group, into `flags`: cf_real_enc_flag_bytes(U, H) bytes of device scratch written and read by
+ * the call), then one launch whose work-groups take one of two roles, the rings' body over the
+ * rounds that hold a pair which keeps the cube and the staging body over the rounds that hold one
+ * which does not.  That launch needs up to 87 KB of dynamic LDS per work-group at K > 64 (53 KB at
+ * K <= 64).  With the fixed cube rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n and flags may be
+ * NULL, and there is one launch.
  */
 int64_t cf_real_enc_ring_bytes(int64_t U);
 int64_t cf_real_enc_flag_bytes(int64_t U, int64_t H);
@@ -248,9 +252,11 @@ int cf_real_enc_bwd_static(const float *a_ik, const float *rpos_ij_e, const floa
  *
  * Arguments as for cf_real_enc_fwd (K = 0) and cf_fused_dpa_fwd (no b_ij); que is pre-divided
  * by sqrt(Dk).  edge_ij_e must be sorted by source atom (e_start_i its CSR offsets); any
- * such list is accepted.  max_row is an upper bound on the edges of one source atom: a
+ * such list is accepted.  max_row is a HARD upper bound on the edges of one source atom: a
  * work-group keeps its row's max_row * H logits in LDS, 64 KB at most (rows of up to 1820
- * edges at H = 8), beyond that CF_ERR_UNSUPPORTED.
+ * edges at H = 8), beyond that CF_ERR_UNSUPPORTED.  The host cannot check the bound against
+ * e_start_i without reading it back; a row that exceeds it is not evaluated and its output row
+ * is NaN.
  * Output: out (N,H,Dv); rows of atoms without edges are zero.
  */
 int cf_fused_enc_dpa_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,

@@ -733,6 +733,20 @@ def test_other_normalisations_and_dropout_take_the_torch_loop(dev):
     attn.train()
     y_train = attn(*args, need_weights=False)[0]
     assert y_train.requires_grad and float((y_train.detach() - y_eval).abs().max()) > 1e-4
+    # train mode under no_grad on a block without value bins: the one-launch path (which has no
+    # dropout) must step aside, as the reference drops weights whenever `training` is set
+    # (models/indexed_lattice_multi_head_attention_cuda.py:757-759)
+    cfg0, model0 = build_model("cfg2_default_b128", num_layers=1, value_pe_dist_real=0, adaptive_cutoff_sigma=0.0,
+                               dropout=0.0)
+    attn0 = model0.encoder.layers[0].self_attn.to(dev)
+    attn0.eval()
+    with torch.no_grad():
+        y0_eval = attn0(*args, need_weights=False)[0]
+    attn0.train()
+    attn0.dropout = 0.4
+    with torch.no_grad():
+        y0_drop = attn0(*args, need_weights=False)[0]
+    assert float((y0_drop - y0_eval).abs().max()) > 1e-4
     attn.dropout = 0.0
     attn.params.norm_func_mode = -3
     y_scaled, w = attn(*args, need_weights=True)

@@ -199,3 +199,96 @@ def test_irregular_mean_and_minimum_distance():
     got2 = ks.minimum_distance(p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.rvlen, 9.0, 0, 0)
     d2big = tp.lattice_dist2(p.b.pos.double(), p.b.batch, p.b.trans_vec.double(), p.edges, 4)
     assert rel_err(got2, d2big.min(dim=1).values) < 1e-5
+
+
+# ---- the tolerance helpers (not restatements of reference code, but the element-wise parity bounds of
+# the GPU tests are built from them, so they are pinned like everything else)
+def _dense_translations(p, lattice_range):
+    """(E,T) squared distances of every edge over the fixed cube, float64, meshgrid-'ij' order."""
+    r = range(-lattice_range, lattice_range + 1)
+    n = torch.tensor(list(itertools.product(r, r, r)), dtype=torch.float64)          # (T,3)
+    shift = n @ p.b.trans_vec.double()[p.b.batch[p.edges[0]]]                         # (E,T,3)
+    return ((p.rpos.double()[:, None, :] + shift) ** 2).sum(-1)
+
+
+def test_conditioning_helper_is_the_sum_of_absolute_sensitivities():
+    """ref_real_enc_fwd_cond against central finite differences in float64: s_k = sum_n w_n g_k(d_n) / S
+    with every translation's distance (inside g) and squared distance (inside w) perturbed on its own;
+    cond is the sum over translations of |ds/d ln d_n| + |ds/d ln d2_n| (S held fixed).  A missing
+    factor, a wrong width or a signed instead of absolute sum fails this."""
+    p = Problem([2, 3], H=2, K=8, D=4, seed=31)
+    lr, K, dist_max, ws = 1, 8, 9.0, 0.8
+    cond = ks.real_enc_fwd_cond(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, K, dist_max, ws, None, 0.0, lr, 0)
+    d2 = _dense_translations(p, lr)                                                   # (E,T)
+    a = p.a.double()[p.edges[0]]                                                      # (E,H)
+    mu = dist_max / K
+    centres = torch.arange(1, K + 1, dtype=torch.float64) * mu
+
+    def parts(dd, dd2):
+        """unnormalised weights (E,H,T) from dd2 and Gaussians (E,T,K) from dd"""
+        w = torch.exp(a[:, :, None] * (dd2[:, None, :] - d2.min(dim=1).values[:, None, None]))
+        g = torch.exp(-((centres[None, None, :] - dd[:, :, None]) / (math.sqrt(2.0) * ws * mu)) ** 2)
+        return w, g
+    d = d2.sqrt()
+    w0, g0 = parts(d, d2)
+    S = w0.sum(-1)                                                                    # (E,H), held fixed
+    T = d2.shape[1]
+    expect = torch.zeros(p.E, 2, K, dtype=torch.float64)
+    h = 1e-6
+    for n in range(T):
+        bump = torch.zeros(T, dtype=torch.float64)
+        bump[n] = h
+        # relative perturbation of the distance inside the Gaussians
+        _, gp = parts(d * (1 + bump), d2)
+        _, gm = parts(d * (1 - bump), d2)
+        ds_dist = torch.einsum("eht,etk->ehk", w0, gp - gm) / (2 * h) / S[:, :, None]
+        # relative perturbation of the squared distance inside the weights
+        wp, _ = parts(d, d2 * (1 + bump))
+        wm, _ = parts(d, d2 * (1 - bump))
+        ds_w = torch.einsum("eht,etk->ehk", wp - wm, g0) / (2 * h) / S[:, :, None]
+        expect += ds_dist.abs() + ds_w.abs()
+    assert rel_err(cond, expect) < 1e-5
+    assert float((cond.double() - expect).abs().max()) <= 1e-5 * float(expect.abs().max())
+    # and it really bounds a float32 evaluation's error to first order: recompute s from distances
+    # rounded to float32 and compare with the float64 s
+    s64 = torch.einsum("eht,etk->ehk", w0, g0) / S[:, :, None]
+    w32, g32 = parts(d2.float().sqrt().double(), d2.float().double())
+    s32 = torch.einsum("eht,etk->ehk", w32, g32) / S[:, :, None]
+    assert bool(((s32 - s64).abs() <= 2.0 ** -23 * expect + 1e-15).all())
+
+
+def test_backward_magnitude_helper_is_the_sum_of_absolute_terms():
+    """ref_real_enc_bwd_magnitude against a brute-force expansion in float64: every individual product
+    that enters ga (gz p d2; p d2 g W gv; -(p d2)(p g W gv)) and gW (p g gv) is formed as its own
+    tensor entry and the absolute values are summed."""
+    p = Problem([2, 3], H=2, K=6, D=3, seed=32)
+    lr, K = 1, 6
+    z, _ = ks.real_enc_fwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, K, 9.0, 1.0, p.W, None, 0.0, lr, 0)
+    gz, gv = p.randn(p.E, 2), p.randn(p.E, 2, 3)
+    ga_mag, gW_mag = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z, gz, gv, K, 9.0,
+                                     1.0, p.W, None, 0.0, lr, 0, magnitude=True)
+    d2 = _dense_translations(p, lr)                                                   # (E,T)
+    a = p.a.double()[p.edges[0]]
+    logit = a[:, :, None] * d2[:, None, :]
+    prob = torch.softmax(logit, dim=-1)                                               # (E,H,T)
+    mu = 9.0 / K
+    centres = torch.arange(1, K + 1, dtype=torch.float64) * mu
+    g = torch.exp(-((centres[None, None, :] - d2.sqrt()[:, :, None]) / (math.sqrt(2.0) * mu)) ** 2)   # (E,T,K)
+    W = p.W.double()[0]                                                               # (H,D,K)
+    gv64, gz64 = gv.double(), gz.double()
+    t1 = gz64[:, :, None] * prob * d2[:, None, :]                                     # (E,H,T)
+    t2 = torch.einsum("eht,et,etk,hdk,ehd->ehtkd", prob, d2, g, W, gv64)
+    pd2 = prob * d2[:, None, :]
+    t3 = -torch.einsum("ehm,eht,etk,hdk,ehd->ehmtkd", pd2, prob, g, W, gv64)
+    per_edge = t1.abs().sum(-1) + t2.abs().sum((-1, -2, -3)) + t3.abs().sum((-1, -2, -3, -4))
+    ga_expect = torch.zeros(p.N, 2, dtype=torch.float64).index_add_(0, p.edges[0], per_edge)
+    gW_terms = torch.einsum("eht,etk,ehd->ehtdk", prob, g, gv64)
+    gW_expect = gW_terms.abs().sum((0, 2))[None]                                      # (1,H,D,K)
+    assert rel_err(ga_mag, ga_expect) < 1e-5 and rel_err(gW_mag, gW_expect) < 1e-5
+    # the signed sums are the gradients themselves, and never exceed the magnitudes
+    ga, gW = ks.real_enc_bwd(p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, z, gz, gv, K, 9.0, 1.0,
+                             p.W, None, 0.0, lr, 0)
+    signed = torch.zeros(p.N, 2, dtype=torch.float64).index_add_(
+        0, p.edges[0], t1.sum(-1) + t2.sum((-1, -2, -3)) + t3.sum((-1, -2, -3, -4)))
+    assert rel_err(ga, signed) < 1e-5 and rel_err(gW, gW_terms.sum((0, 2))[None]) < 1e-5
+    assert bool((ga.abs() <= ga_mag * (1 + 1e-6)).all()) and bool((gW.abs() <= gW_mag * (1 + 1e-6)).all())

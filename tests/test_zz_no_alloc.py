@@ -67,3 +67,50 @@ def test_static_scratch_backward_rejects_what_does_not_fit(dev):
     assert rc != 0
     msg = L.cf_last_error().decode()
     assert "built-in buffer holds 33554432" in msg and "cf_real_enc_bwd with a workspace" in msg
+
+
+def test_static_scratch_backward_allocates_nothing_and_runs_under_capture(dev):
+    """What the entry point is for.  (1) A warmed call with preallocated outputs leaves the device's
+    free memory and torch's allocator untouched.  (2) The same call recorded into a HIP graph (where
+    hipMalloc is not allowed) and replayed several times, with eager work and synchronisations in
+    between, gives the eager result bit for bit every time."""
+    L = lib.load()
+    p = Problem([20, 7, 33, 1, 12], H=8, K=64, D=16, seed=83)
+    a, rpos, tv, bt, ed, es, W = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.e_start, p.W)
+    pairs = ops.edge_pairs(p.b.sizes.to(dev))
+    z, _ = ops.real_enc_fwd(a, rpos, tv, bt, ed, 64, p.dist_max, p.wscale, W, pairs_u=pairs)
+    gz, gv = p.randn(p.E, 8).to(dev), p.randn(p.E, 8, 16).to(dev)
+    ga_ref, gW_ref = ops.real_enc_bwd(a, rpos, tv, bt, ed, es, z, gz, gv, 64, p.dist_max, p.wscale, W, pairs_u=pairs)
+    ga, gW = torch.empty_like(a), torch.empty_like(W)
+    N, H = a.shape
+    E, B = ed.shape[1], tv.shape[0]
+
+    def call(stream):
+        return L.cf_real_enc_bwd_static(ptr(a), ptr(rpos), ptr(tv), ptr(bt), ptr(ed), ptr(es), ptr(z), ptr(gz),
+                                        ptr(gv), N, H, E, B, 64, 16, float(p.dist_max), float(p.wscale), ptr(W), 1,
+                                        0, 0.0, 2, 0, ptr(pairs), pairs.shape[0], ptr(ga), ptr(gW), stream)
+    assert call(stream_handle(dev)) == 0, L.cf_last_error()           # warm: module loaded, symbol looked up
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    reserved_before, allocated_before = torch.cuda.memory_reserved(), torch.cuda.memory_allocated()
+    ga.fill_(float("nan"))
+    gW.fill_(float("nan"))
+    assert call(stream_handle(dev)) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert (torch.cuda.memory_reserved(), torch.cuda.memory_allocated()) == (reserved_before, allocated_before)
+    assert torch.equal(ga, ga_ref) and torch.equal(gW, gW_ref)
+    # under stream capture
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = call(stream_handle(dev))
+    assert rc == 0, L.cf_last_error()
+    for rep in range(3):
+        ga.fill_(float("nan"))
+        gW.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ga, ga_ref) and torch.equal(gW, gW_ref), rep
+        again, _ = ops.real_enc_bwd(a, rpos, tv, bt, ed, es, z, gz, gv, 64, p.dist_max, p.wscale, W, pairs_u=pairs)
+        assert torch.equal(again, ga_ref)                             # eager work between replays
+        torch.cuda.synchronize()
