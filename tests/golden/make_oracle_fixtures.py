@@ -3,7 +3,7 @@ evaluation takes minutes (7-block forward at 256 crystals, training step at 128 
 4-block forward on 200+-atom cells), so that the GPU parity tests compare against them
 without re-running the oracle every time:
 
-    python tests/golden/make_oracle_fixtures.py            # all three, about ten minutes on 8 cores
+    python tests/golden/make_oracle_fixtures.py            # all four, about fifteen minutes on 8 cores
 
 Nothing of the reference is imported or read: inputs come from the package's own seeded
 generator (crystalformer_amd/synthetic.py) and seeded parameter initialisation, results
@@ -165,7 +165,9 @@ def train_fixture(name, tag):
 
 
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["cfg3", "cfg4", "cfg5"]
+    which = sys.argv[1:] or ["cfg3", "cfg4", "cfg5", "cfg5full"]
+    if "cfg5full" in which:         # all 16 cells of 200..444 atoms, 1.77 M edges: about five minutes on 8 cores
+        forward_fixture("cfg5_stress_b16", make_config_batch("cfg5_stress_b16"), "cfg5_forward")
     if "cfg5" in which:
         forward_fixture("cfg5_stress_b16", cfg5_subset(make_config_batch("cfg5_stress_b16")), "cfg5_subset_forward")
     if "cfg4" in which:

@@ -246,6 +246,85 @@ def test_four_block_forward_on_large_cells(dev):
     check_forward_against_fixture(dev, "cfg5_stress_b16", b, "cfg5_subset_forward")
 
 
+def test_four_block_forward_on_all_sixteen_large_cells(dev):
+    """Config 5 at full size at model level: the 4-block default model over all 16 cells of 200..444
+    atoms (5,459 atoms, 1.77 M edges: the pair kernel staging for itself, its ticket scheduler, the
+    attention kernel's long-row variant), every 37th atom's block outputs and all 16 outputs against the
+    CPU oracle's stored results."""
+    b = make_config_batch("cfg5_stress_b16")
+    assert b.sizes.numel() == 16 and b.num_edges > 1_700_000
+    check_forward_against_fixture(dev, "cfg5_stress_b16", b, "cfg5_forward")
+
+
+def _stratified_edges(p, R, total, ring=192):
+    """Edges sampled per crystal and per number of staging passes of their atom pair (1, 2, 3 or more;
+    a pass stages ``ring`` translations of the union box of the pair's 16 (atom, head) columns).
+    ``R`` (N,H,3) are the half-widths.  Returns (edge ids sorted, passes of each)."""
+    i, j = p.edges
+    U = torch.maximum(R[i].amax(dim=1), R[j].amax(dim=1)).long()                   # (E,3) union half-widths
+    T = (2 * U + 1).prod(dim=1)
+    passes = (T + ring - 1) // ring
+    cls = passes.clamp(max=3)
+    strata = []
+    for c in range(int(p.b.sizes.numel())):
+        in_c = p.b.batch[i] == c
+        for k in (1, 2, 3):
+            ids = torch.nonzero(in_c & (cls == k)).flatten()
+            if ids.numel():
+                strata.append(ids[torch.randperm(ids.numel(), generator=p.g)])
+    quota = -(-total // len(strata))
+    picked = torch.cat([ids[:quota] for ids in strata])
+    if picked.numel() < total:          # small strata: the rest from the larger ones, in turn
+        spare = torch.cat([ids[quota:quota + total] for ids in strata])
+        picked = torch.cat([picked, spare[torch.randperm(spare.numel(), generator=p.g)[:total - picked.numel()]]])
+    sel = picked.sort().values
+    return sel, passes[sel]
+
+
+@pytest.mark.parametrize("name,r0,lattice_range", [("cfg5_stress_b16", 3.0, 2), ("cfg3_7block_b256", 2.0, 2),
+                                                   ("cfg3_7block_b256", 3.0, 2)])
+def test_pair_kernel_at_full_size_on_stratified_edges(dev, name, r0, lattice_range):
+    """The pair-evaluated forward at the benchmark's full sizes, where its multi-pass staging, ticket
+    scheduler and 32-bit row arithmetic are exercised: config 5 (1.77 M edges, r0 = 3 A) and config 3
+    with the wide blocks' r0 = 2 and 3 A, under both translation rules, on at least 2,000 edges
+    against the C oracle -- sampled from every crystal and, under the adaptive rule, from the atom
+    pairs whose union box takes one, two and three or more staging passes alike.  Exponents are those
+    a block can produce: a = -rho / (2 r0^2), rho in [0.5, 2.5]."""
+    b = make_config_batch(name)
+    p = Problem(b, H=8, K=64, D=16, seed=62)
+    p.dist_max = 10.0 * r0
+    rho = 0.5 + 2.0 * torch.rand(p.N, 8, generator=p.g)
+    p.a = -rho / (2.0 * r0 * r0)
+    sizes_d = b.sizes.to(dev)
+    pairs = ops.edge_pairs(sizes_d, p.N, p.E)
+    dv = to_dev(dev, p.a, p.rpos, p.b.trans_vec, p.b.batch, p.edges, p.W, p.rvlen)
+    crystals = int(b.sizes.numel())
+    for rule, cut, mr in (("A", 0.0, 0), ("B", -3.5, lattice_range)):
+        z, v = ops.real_enc_fwd(dv[0], dv[1], dv[2], dv[3], dv[4], 64, p.dist_max, 1.0, dv[5],
+                                dv[6] if rule == "B" else None, cut, lattice_range, mr, pairs_u=pairs)
+        assert bool(torch.isfinite(z).all()) and bool(torch.isfinite(v).all())
+        R = ks.translation_ranges(p.a, p.rvlen if rule == "B" else None, p.b.batch, cut, lattice_range, mr)
+        assert torch.equal(ops.translation_ranges(dv[0], dv[6] if rule == "B" else None, dv[3], cut, lattice_range,
+                                                  mr).cpu(), R)
+        sel, passes = _stratified_edges(p, R, 2100)
+        assert sel.numel() >= 2000 and len(set(p.b.batch[p.edges[0, sel]].tolist())) == crystals
+        if rule == "B":
+            counts = [int((passes.clamp(max=3) == k).sum()) for k in (1, 2, 3)]
+            # (which classes exist depends on the cells: config 5's long thin cells have all three)
+            assert sum(c > 0 for c in counts) >= (3 if name.startswith("cfg5") else 2), counts
+        z_ref, v_ref = ks.real_enc_fwd(p.a, p.rpos[sel], p.b.trans_vec, p.b.batch, p.edges[:, sel], 64, p.dist_max,
+                                       1.0, p.W, p.rvlen if rule == "B" else None, cut, lattice_range, mr)
+        cond = ks.real_enc_fwd_cond(p.a, p.rpos[sel], p.b.trans_vec, p.b.batch, p.edges[:, sel], 64, p.dist_max, 1.0,
+                                    p.rvlen if rule == "B" else None, cut, lattice_range, mr)
+        _, s_ref = ks.real_enc_fwd(p.a, p.rpos[sel], p.b.trans_vec, p.b.batch, p.edges[:, sel], 64, p.dist_max,
+                                   1.0, None, p.rvlen if rule == "B" else None, cut, lattice_range, mr)
+        T = (2 * R.long() + 1).prod(dim=-1).max().item()
+        from tests.helpers import atol_projected
+        assert_close(z[sel.to(dev)], z_ref, f"{name} rule {rule} z")
+        assert_close(v[sel.to(dev)], v_ref, f"{name} rule {rule} v",
+                     atol=atol_projected(s_ref, p.W, cond, translations=T))
+
+
 def test_training_step_at_128_crystals(dev):
     """Config 4: one training-mode forward + the reference's step loss + backward at 128 crystals
     (models/regression.py:117-121) on the HIP path (periodic-encoding and attention backward
