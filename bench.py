@@ -392,8 +392,8 @@ def main() -> int:
     ap.add_argument("--no-staged-rings", action="store_true",
                     help="every block stages its translations itself (pair kernel) instead of starting from the "
                          "rings staged once per forward")
-    ap.add_argument("--adaptive-rings", action="store_true",
-                    help="with --rule B: atom pairs that keep the cube start from the staged rings (off by default)")
+    ap.add_argument("--no-adaptive-rings", action="store_true",
+                    help="with --rule B: every atom pair staged by the pair kernel (none from the staged rings)")
     ap.add_argument("--no-fresh", action="store_true", help="skip the fresh-batch (another batch every step) figures")
     ap.add_argument("--fresh-capacity", choices=["bound", "pool"], default="bound",
                     help="capacity of the one graph that serves the fresh batches: the largest batch the "
@@ -442,8 +442,8 @@ def main() -> int:
         hip_funcs.KernelManager.FUSE_ENCODING_ATTENTION = False
     if args.no_staged_rings:
         hip_funcs.KernelManager.STAGED_RINGS = False
-    if args.adaptive_rings:
-        hip_funcs.KernelManager.ADAPTIVE_RINGS = True
+    if args.no_adaptive_rings:
+        hip_funcs.KernelManager.ADAPTIVE_RINGS = False
     dev = torch.device("cuda:0")
     if args.train and args.config == "cfg2_default_b128":
         args.config = "cfg4_train_b128"

@@ -31,12 +31,14 @@ const int64_t *live_units(int64_t U);
 int64_t *size_header_for_layout(int64_t N, int64_t E);
 
 // real_enc_mfma.hip
+// order / counts (nullable, adaptive boxes from staged rings): the launch takes the units
+// order[counts[0] .. counts[0] + counts[1]) (both counts on the device)
 int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,
                               const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
                               int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
                               int64_t W_num, const float *rvlen, float cutoff, int lattice_range,
-                              int min_range, unsigned int *sched, const unsigned char *unit_flags,
-                              const unsigned char *round_flags, float *z, float *v, hipStream_t st);
+                              int min_range, unsigned int *sched, const int *order, const int64_t *counts,
+                              float *z, float *v, hipStream_t st);
 
 // real_enc_mfma_bwd.hip
 int real_enc_bwd_pairs_blocks(int64_t U, int64_t H);
@@ -53,18 +55,12 @@ int launch_ring_stage(const float *rpos, const float *tvecs, const int64_t *pair
                       float bin_step, float s_scale, int lattice_range, float weak_a, float *cache, hipStream_t st);
 int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U, int64_t N, int64_t H, int64_t E,
                               int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
-                              const float *cache, const unsigned char *unit_flags, const unsigned char *round_flags,
+                              const float *cache, const int *order, const int64_t *n_units,
                               float *z, float *v, hipStream_t st);
-int64_t real_enc_round_count(int64_t U, int64_t H);
-int launch_real_enc_fwd_two_role(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,
-                                 const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
-                                 int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
-                                 const float *rvlen, float cutoff, int lattice_range, int min_range,
-                                 const float *cache, const unsigned char *unit_flags,
-                                 const unsigned char *round_flags, float *z, float *v, hipStream_t st);
-int launch_unit_floor(const float *a_ik, const float *rvlen, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
-                      float cutoff, int lattice_range, int min_range, unsigned char *unit_flags,
-                      unsigned char *round_flags, hipStream_t st);
+int64_t unit_partition_bytes(int64_t U);
+int launch_unit_partition(const float *a_ik, const float *rvlen, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
+                          float cutoff, int lattice_range, int min_range, void *scratch, int64_t **counts_out,
+                          int **order_out, hipStream_t st);
 
 #define CF_REQUIRE(cond, code, ...)            \
     do {                                       \

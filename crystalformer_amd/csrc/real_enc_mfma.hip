@@ -72,11 +72,10 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
                               const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
                               int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
                               int64_t W_num, const float *rvlen, float cutoff, int lattice_range,
-                              int min_range, unsigned int *sched, const unsigned char *unit_flags,
-                              const unsigned char *round_flags, float *z, float *v, hipStream_t st)
+                              int min_range, unsigned int *sched, const int *order, const int64_t *counts,
+                              float *z, float *v, hipStream_t st)
 {
     if (K < 0 || K > 128) return CF_ERR_UNSUPPORTED;
-    if (unit_flags && (cutoff == 0.0f || !round_flags)) return CF_ERR_UNSUPPORTED;   // selection: adaptive boxes only
     if (W && (D < 1 || D > 64)) return CF_ERR_UNSUPPORTED;
     PairArgs p{};
     p.a_ik = a_ik; p.rpos = rpos; p.tvecs = tvecs; p.batch = batch; p.edges = edges; p.pairs = pairs;
@@ -116,11 +115,15 @@ int launch_real_enc_fwd_pairs(const float *a_ik, const float *rpos, const float 
     // and the fixed stride, which costs nothing, does better (measured: 64.5 against 70 us at
     // 7 rounds per work-group; 1.66 against 1.81 ms at 217).
     if (rounds < 16 * blocks) p.sched = nullptr;
-    // unit selection: the units that do not keep the cube (the others run from the staged rings)
-    p.unit_flags = unit_flags; p.round_flags = round_flags; p.flag_want = 0;
-    if (unit_flags) p.sched = nullptr;
     p.live_U = live_units(U);
-    if (p.live_U && unit_flags) return CF_ERR_UNSUPPORTED;   // (the flags are laid out for a known U)
+    if (order) {
+        // the second of two lists of units (the first runs from the staged rings): counts[1] units
+        // from slot counts[0] on; how many rounds that makes is not known here, so no tickets
+        p.order = order;
+        p.order_first = counts;
+        p.live_U = counts + 1;
+        p.sched = nullptr;
+    }
 #define CF_PAIR(NTV, UNI, PRJ, DTV, SR) \
     real_enc_fwd_pair_kernel<NTV, UNI, PRJ, DTV, SR><<<(int)blocks, WPB * WAVE, lds, st>>>(p)
 #define CF_PAIR_MODE(NTV, UNI, SR)                                            \

@@ -38,14 +38,13 @@ struct PairArgs {
     float inv_bin_step;     // distance argument -> fractional bin coordinate
     float window;           // bins beyond which a Gaussian is below 2^-40 and is not evaluated
     const float *rings;     // staged translations of every unit (RIMG_WORDS each), nullable
-    // Unit selection (adaptive boxes run as two launches: units whose columns all keep the cube
-    // start from the staged rings, the others are staged by the pair kernel), nullable:
-    //   unit_flags[g U + u]  1: all active columns of unit u in head group g have the cube, else 0
-    //   round_flags[rd]      bit 0: some unit of round rd has the cube, bit 1: some existing unit has not
-    // A launch handles the units whose bit equals flag_want and walks only the rounds that hold one.
-    const unsigned char *unit_flags;
-    const unsigned char *round_flags;
-    int flag_want;
+    // Order of the units, nullable: slot -> unit (8 r + w is the slot of wavefront w in round r; without
+    // an order slot and unit are the same).  Adaptive boxes from staged rings split the units in two
+    // stably ordered sets this way -- those whose columns all keep the cube, then the others -- and
+    // give each set to its own launch: order_first (device, nullable) is the slot in `order` where
+    // this launch's units begin, live_U how many there are.
+    const int *order;
+    const int64_t *order_first;
     // Live unit count on the device, nullable (forward and staging kernels): U is then the capacity
     // of the unit list -- what the grid and the buffers are sized for -- and the kernel walks the
     // first *live_U units only.
@@ -58,6 +57,7 @@ __device__ __forceinline__ PairArgs with_live_units(const PairArgs &p)
 {
     PairArgs q = p;
     q.U = live_count(p.live_U, p.U);
+    if (p.order && p.order_first) q.order = p.order + live_count(p.order_first, p.U);
     return q;
 }
 #endif
@@ -241,91 +241,11 @@ __device__ __forceinline__ RoundPos round_pos(int rd, int rounds_per_hg, int hea
     return x;
 }
 
-// First round at or after rd_from, in steps of `stride`, that holds a unit for this launch (or
-// `rounds` when there is none): the 64 lanes look at 64 candidate rounds at a time.  Without round
-// flags every round counts.  Wave-uniform result; all wavefronts of a work-group agree.
-__device__ __forceinline__ int next_active_round(const PairArgs &p, int rd_from, int rounds, int stride, int lane)
+// order[slot] as a scalar load (slot is wave-uniform; the order was written by an earlier launch)
+__device__ __forceinline__ int ordered_unit(const int *order, int slot)
 {
-    if (!p.round_flags) return rd_from < rounds ? rd_from : rounds;
-    const unsigned char want = p.flag_want ? 1 : 2;
-    int64_t from = rd_from;
-    for (;;) {
-        const int64_t r = from + (int64_t)lane * stride;
-        const bool hit = r >= rounds || (p.round_flags[r] & want) != 0;
-        const unsigned long long m = __ballot(hit);
-        if (m != 0ull) {
-            const int l = __builtin_amdgcn_readfirstlane(__ffsll((long long)m) - 1);
-            const int64_t first = from + (int64_t)l * stride;
-            return first >= rounds ? rounds : (int)first;
-        }
-        from += (int64_t)WAVE * stride;
-    }
-}
-
-// The first three active rounds of a work-group (positions first, first + stride, ... without
-// flags): one look at 64 candidates, what that does not settle one search at a time.
-struct RoundSeq { int rd[3]; };
-__device__ __forceinline__ RoundSeq first_active_rounds(const PairArgs &p, int first, int rounds, int stride, int lane)
-{
-    RoundSeq s;
-    if (!p.round_flags) {
-#pragma unroll
-        for (int k = 0; k < 3; k++) {
-            const int64_t r = (int64_t)first + (int64_t)k * stride;
-            s.rd[k] = r < rounds ? (int)r : rounds;
-        }
-        return s;
-    }
-    const unsigned char want = p.flag_want ? 1 : 2;
-    const int64_t r0 = (int64_t)first + (int64_t)lane * stride;
-    bool hit0 = true;
-    if (r0 < rounds) hit0 = (p.round_flags[r0] & want) != 0;
-    unsigned long long m = __ballot(hit0);
-    int64_t beyond = (int64_t)first + (int64_t)WAVE * stride;       // first candidate the look did not cover
-#pragma unroll
-    for (int k = 0; k < 3; k++) {
-        if (m != 0ull) {
-            const int l = __builtin_amdgcn_readfirstlane(__ffsll((long long)m) - 1);
-            const int64_t r = (int64_t)first + (int64_t)l * stride;
-            s.rd[k] = r < rounds ? (int)r : rounds;
-            m &= m - 1ull;
-        } else {
-            s.rd[k] = beyond < rounds ? next_active_round(p, (int)beyond, rounds, stride, lane) : rounds;
-            beyond = (int64_t)s.rd[k] + stride;
-        }
-    }
-    return s;
-}
-
-// The active round after rd_last, from flags requested a round earlier: lane l holds whether
-// candidate rd_last + (l + 1) stride counts (request_round_candidates), the rest is a search.
-__device__ __forceinline__ bool request_round_candidate(const PairArgs &p, int rd_last, int rounds, int stride, int lane)
-{
-    const int64_t r = (int64_t)rd_last + (int64_t)(lane + 1) * stride;
-    if (r >= rounds) return true;
-    return (p.round_flags[r] & (p.flag_want ? 1 : 2)) != 0;
-}
-__device__ __forceinline__ int round_after(const PairArgs &p, bool candidate, int rd_last, int rounds, int stride, int lane)
-{
-    if (rd_last >= rounds) return rounds;
-    const unsigned long long m = __ballot(candidate);
-    if (m != 0ull) {
-        const int l = __builtin_amdgcn_readfirstlane(__ffsll((long long)m) - 1);
-        const int64_t r = (int64_t)rd_last + (int64_t)(l + 1) * stride;
-        return r < rounds ? (int)r : rounds;
-    }
-    const int64_t beyond = (int64_t)rd_last + (int64_t)(WAVE + 1) * stride;
-    return beyond < rounds ? next_active_round(p, (int)beyond, rounds, stride, lane) : rounds;
-}
-
-// flag of unit u in head group hg (request it a round ahead), and whether it selects the unit
-__device__ __forceinline__ int load_unit_flag(const PairArgs &p, int64_t u, int hg)
-{
-    return (int)p.unit_flags[(int64_t)hg * p.U + u];
-}
-__device__ __forceinline__ bool unit_selected(const PairArgs &p, int flag)
-{
-    return (__builtin_amdgcn_readfirstlane(flag) != 0) == (p.flag_want != 0);
+    typedef const int __attribute__((address_space(4))) *ConstInt;
+    return ((ConstInt)order)[slot];
 }
 
 // ---- unit descriptors --------------------------------------------------------

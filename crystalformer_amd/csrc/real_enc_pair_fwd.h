@@ -96,8 +96,9 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
     const int rounds = rounds_per_hg * p.head_groups;
     // unit of round rd_ for this wave (0 when the round or the unit does not exist: loads stay valid)
     auto unit_of = [&](int rd_, const RoundPos &rp) -> int64_t {
-        const int64_t u_ = (int64_t)rp.r * WPB + wave;
-        return (rd_ < rounds && u_ < p.U) ? u_ : 0;
+        const int64_t slot = (int64_t)rp.r * WPB + wave;
+        if (!(rd_ < rounds && slot < p.U)) return 0;
+        return p.order ? (int64_t)ordered_unit(p.order, (int)slot) : slot;
     };
     // exponent of column c of a unit in the head group of a round
     auto load_a = [&](const float *g_a, const UnitIds &d, const RoundPos &rp) -> float {
@@ -111,24 +112,11 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
     __shared__ int tick[2];
     unsigned int *__restrict__ sched = p.sched;
     const int stride = grid_size;
-    // Adaptive boxes with unit selection (p.unit_flags): this launch takes the units that do not keep
-    // the cube and walks only the rounds that hold one (no tickets then: the launcher passes none).
-    const bool select = !UNIFORM && p.unit_flags != nullptr;
     int rd_first = block_id, rd_next = block_id + stride, rd_next2 = block_id + 2 * stride;
-    if (select) {
-        const RoundSeq seq = first_active_rounds(p, block_id, rounds, stride, lane);
-        rd_first = seq.rd[0];
-        rd_next = seq.rd[1];
-        rd_next2 = seq.rd[2];
-    }
-    auto unit_flag = [&](int rd_, const RoundPos &rp) -> int {
-        return select ? load_unit_flag(p, unit_of(rd_, rp), rd_ < rounds ? rp.hg : 0) : 0;
-    };
     RoundPos pos = round_pos(rd_first, rounds_per_hg, p.head_groups);
     RoundPos pos_next = round_pos(rd_next, rounds_per_hg, p.head_groups);
     // fill the descriptor pipeline: current round complete, next round's ids known
     UnitIds ids = unit_ids(load_unit_ids(p.pairs, unit_of(rd_first, pos), lane));
-    int uflag = unit_flag(rd_first, pos);
     float a_cur;
     UnitGeom geo;
     UnitIds ids_next;
@@ -166,16 +154,12 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
     int it = 0;
     for (int rd = rd_first; rd < rounds; it++) {
         const int hg = pos.hg;
-        const int64_t u = (int64_t)pos.r * WPB + wave;
-        const bool unit_on = u < p.U && (!select || unit_selected(p, uflag));
+        const bool unit_on = (int64_t)pos.r * WPB + wave < p.U;
         const RoundPos pos_next2 = round_pos(rd_next2, rounds_per_hg, p.head_groups);
-        // (the round after rd_next2: its candidates' flags are requested here, looked at at the end)
         // (adaptive boxes: the addresses of the once-a-round loads are formed here, not kept in
         // registers across the rounds)
         int lane_r = lane;
         if (!UNIFORM) asm volatile("" : "+v"(lane_r));
-        bool candidate = false;
-        if (select) candidate = request_round_candidate(p, rd_next2, rounds, stride, lane_r);
         // ticket for the round after rd_next2 (once past the end, no more draws): requested here,
         // looked at only before the epilogue, like the loads below
         unsigned int ticket_old = 0;
@@ -186,7 +170,6 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
         const float *__restrict__ g_rvlen = UNIFORM ? nullptr : seg_pointer(&in->rvlen);
         const float gv_next = load_unit_geom(ids_next, lane_r, seg_pointer(&in->rpos), seg_pointer(&in->tvecs), g_rvlen);
         const float a_next = load_a(in->a_ik, ids_next, pos_next);
-        const int uflag_next = unit_flag(rd_next, pos_next);
         const int64_t dv_next2 = load_unit_ids(in->pairs, unit_of(rd_next2, pos_next2), lane_r);
         if (PROJ == PROJ_SHARED && hg != wa_hg) {
             const int hw = hg * 8 + wave;
@@ -654,11 +637,10 @@ __device__ __forceinline__ void real_enc_fwd_pair_body(const PairArgs &p, const 
         ids = ids_next;
         geo = geo_next;
         a_cur = a_next;
-        uflag = uflag_next;
         ids_next = ids_next2;
         pos = pos_next;
         pos_next = pos_next2;
-        int rd_next3 = select ? round_after(p, candidate, rd_next2, rounds, stride, lane) : rd_next2 + stride;
+        int rd_next3 = rd_next2 + stride;
         if (sched) {
             if (PROJ != PROJ_SHARED) __syncthreads();     // (the shared projection has its own barriers)
             rd_next3 = tick[it & 1];

@@ -155,45 +155,122 @@ __global__ __launch_bounds__(256) void ring_stage_kernel(PairArgs p_, float weak
     }
 }
 
-// ---------------------------------------------------------------- unit selection
-// Adaptive boxes: which units keep the fixed cube in all their active columns (the range rule of
-// every (atom, head) of the unit yields lattice_range on the three axes).  Those are evaluated from
-// the staged rings, on the bits the pair kernel's own shortcut for such units produces; the others
-// go to the pair kernel.  One wavefront per round (8 units) and head group: lane = (unit, head),
-// each lane applies the rule to its head of atoms i and j.
-__global__ __launch_bounds__(256) void unit_floor_kernel(PairArgs p, unsigned char *__restrict__ unit_flags,
-                                                         unsigned char *__restrict__ round_flags)
+// ---------------------------------------------------------------- adaptive boxes: two sets of units
+// Which units keep the fixed cube in all their active columns (the range rule of every (atom, head)
+// of the unit yields lattice_range on the three axes): those are evaluated from the staged rings, on
+// the bits the pair kernel's own shortcut for such units produces; the others go to the pair kernel.
+// Three small launches turn the rule into two stably ordered lists of units with their counts on the
+// device, so that each of the two kernels walks dense rounds of its own units, however many there
+// are of either kind:
+//   unit_keeps_kernel    a wavefront per 8 units, lane = (unit, head): the rule for its head of atoms i
+//                        and j; a byte per unit and the number of keepers per chunk of PART_CHUNK units;
+//   partition_kernel     every chunk places its keepers behind those of the chunks before it and its
+//                        others behind all keepers (ranks by ballots, chunks in order: the same lists on
+//                        every run); the first work-group leaves {keepers, others} in `counts`.
+constexpr int PART_CHUNK = 1024;                  // units per work-group of partition_kernel
+constexpr int KEEP_CHUNK = 128;                   // units per work-group of unit_keeps_kernel (8 per wavefront)
+
+__global__ __launch_bounds__(PART_CHUNK) void unit_keeps_kernel(PairArgs p_, unsigned char *__restrict__ keeps,
+                                                                int *__restrict__ chunk_keepers)
 {
-    const int lane = threadIdx.x & 63;
-    const int rounds_per_hg = (int)((p.U + WPB - 1) / WPB);
-    const int64_t rounds = (int64_t)rounds_per_hg * p.head_groups;
-    const int64_t rd = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (rd >= rounds) return;
-    const RoundPos rp = round_pos((int)rd, rounds_per_hg, p.head_groups);
+    __shared__ int keepers;
+    const PairArgs p = with_live_units(p_);
+    const int64_t first = (int64_t)blockIdx.x * KEEP_CHUNK;
+    if (first >= p.U) return;
+    if (threadIdx.x == 0) keepers = 0;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int w = lane >> 3, hh = lane & 7;
-    const int64_t u = (int64_t)rp.r * WPB + w;
+    const int64_t u = first + 8 * wave + w;
     const bool exists = u < p.U;
-    bool keeps = true;
+    bool keep = true;
     if (exists) {
         const int64_t *d = p.pairs + u * PAIR_FIELDS;
         const int64_t e_ij = d[0], e_ji = d[1], n = d[4];
-        const int h = rp.hg * 8 + hh;
-        if (h < p.H) {
+        if (hh < p.H) {
             const float rvl[3] = {p.rvlen[n * 3 + 0], p.rvlen[n * 3 + 1], p.rvlen[n * 3 + 2]};
 #pragma unroll
             for (int side = 0; side < 2; side++) {
                 if (side == 1 && e_ji == e_ij) continue;         // a self pair has one direction
                 int R1, R2, R3;
-                range_rule(p.a_ik[d[2 + side] * p.H + h], p.cutoff, rvl, p.lattice_range, p.min_range, R1, R2, R3);
-                keeps = keeps && R1 == p.lattice_range && R2 == p.lattice_range && R3 == p.lattice_range;
+                range_rule(p.a_ik[d[2 + side] * p.H + hh], p.cutoff, rvl, p.lattice_range, p.min_range, R1, R2, R3);
+                keep = keep && R1 == p.lattice_range && R2 == p.lattice_range && R3 == p.lattice_range;
             }
         }
     }
-    const unsigned long long km = __ballot(keeps);
+    const unsigned long long km = __ballot(keep);
     const bool unit_keeps = exists && ((km >> (8 * w)) & 0xFFull) == 0xFFull;
-    if (exists && hh == 0) unit_flags[(int64_t)rp.hg * p.U + u] = unit_keeps ? 1 : 0;
-    const unsigned long long any_keep = __ballot(unit_keeps), any_other = __ballot(exists && !unit_keeps);
-    if (lane == 0) round_flags[rd] = (unsigned char)((any_keep != 0ull ? 1 : 0) | (any_other != 0ull ? 2 : 0));
+    if (exists && hh == 0) keeps[u] = unit_keeps ? 1 : 0;
+    const int mine = __popcll(__ballot(unit_keeps && hh == 0));
+    if (lane == 0 && mine) atomicAdd(&keepers, mine);
+    __syncthreads();
+    if (threadIdx.x == 0) chunk_keepers[blockIdx.x] = keepers;
+}
+
+__global__ __launch_bounds__(PART_CHUNK) void partition_kernel(const unsigned char *__restrict__ keeps,
+                                                               const int *__restrict__ chunk_keepers, int64_t U_cap,
+                                                               const int64_t *live_U, int *__restrict__ order,
+                                                               int64_t *__restrict__ counts)
+{
+    __shared__ int part[PART_CHUNK / WAVE];
+    __shared__ int wave_keep[PART_CHUNK / WAVE];
+    __shared__ int before_total[2];
+    const int64_t U = live_count(live_U, U_cap);
+    const int64_t first = (int64_t)blockIdx.x * PART_CHUNK;
+    if (blockIdx.x == 0 && U == 0 && threadIdx.x == 0) counts[0] = counts[1] = counts[2] = 0;
+    if (first >= U) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // keepers in the chunks before this one, and in all chunks (counted per KEEP_CHUNK units)
+    constexpr int SUB = PART_CHUNK / KEEP_CHUNK;
+    const int subs = (int)((U + KEEP_CHUNK - 1) / KEEP_CHUNK);
+    int before = 0, total = 0;
+    for (int g = threadIdx.x; g < subs; g += PART_CHUNK) {
+        const int c = chunk_keepers[g];
+        total += c;
+        if (g < (int)blockIdx.x * SUB) before += c;
+    }
+    for (int off = 32; off >= 1; off >>= 1) {
+        before += __shfl_xor(before, off, WAVE);
+        total += __shfl_xor(total, off, WAVE);
+    }
+    if (lane == 0) {
+        part[wave] = before;
+        wave_keep[wave] = total;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int b = 0, t = 0;
+        for (int x = 0; x < PART_CHUNK / WAVE; x++) {
+            b += part[x];
+            t += wave_keep[x];
+        }
+        before_total[0] = b;
+        before_total[1] = t;
+        if (blockIdx.x == 0) {
+            counts[0] = t;
+            counts[1] = U - t;
+            counts[2] = 0;                   // scheduling words of the launch that follows
+        }
+    }
+    __syncthreads();
+    const int keep_before = before_total[0], keep_total = before_total[1];
+    const int64_t u = first + threadIdx.x;
+    const bool valid = u < U;
+    const bool keep = valid && keeps[u] != 0;
+    const unsigned long long km = __ballot(keep), vm = __ballot(valid);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    __syncthreads();
+    if (lane == 0) wave_keep[wave] = __popcll(km);
+    __syncthreads();
+    if (valid) {
+        int keep_in_chunk_before = 0;
+        for (int x = 0; x < wave; x++) keep_in_chunk_before += wave_keep[x];
+        const int rank_keep = keep_in_chunk_before + __popcll(km & below);
+        const int in_chunk = wave * WAVE + __popcll(vm & below);         // units before this one in the chunk
+        const int pos = keep ? keep_before + rank_keep
+                             : keep_total + (int)(first - keep_before) + (in_chunk - rank_keep);
+        order[pos] = (int)u;
+    }
 }
 
 // ---------------------------------------------------------------- consumer
@@ -201,9 +278,9 @@ __global__ __launch_bounds__(256) void unit_floor_kernel(PairArgs p, unsigned ch
 // of the next round's unit (its address follows from the round number alone) is requested a round
 // ahead into registers and copied to the wavefront's LDS ring at the top of its round.
 // LDS: per wave 3 x RS words, exchange buffer 4 NT x XPLANE, 8 x 2 edge ids, 8 x 16 reciprocals.
-// SELECT: only the units picked by p.unit_flags / p.flag_want are evaluated, and only the rounds
-// that hold one are walked (p.round_flags).
-template <int NT, int DT, bool SELECT>
+// With p.order the slots of the rounds hold the units the order lists (adaptive boxes: those that keep
+// the cube).
+template <int NT, int DT>
 __device__ __forceinline__ void real_enc_fwd_ring_body(const PairArgs &p, const float *__restrict__ cache,
                                                        const int block_id, const int grid_size)
 {
@@ -231,9 +308,11 @@ __device__ __forceinline__ void real_enc_fwd_ring_body(const PairArgs &p, const 
     const int rounds_per_hg = (int)((p.U + WPB - 1) / WPB);
     const int rounds = rounds_per_hg * p.head_groups;
     const int stride = grid_size;
+    // unit of this wavefront in round rd_ (0 when the round or the slot does not exist: loads stay valid)
     auto unit_of = [&](int rd_, const RoundPos &rp) -> int64_t {
-        const int64_t u_ = (int64_t)rp.r * WPB + wave;
-        return (rd_ < rounds && u_ < p.U) ? u_ : 0;
+        const int64_t slot = (int64_t)rp.r * WPB + wave;
+        if (!(rd_ < rounds && slot < p.U)) return 0;
+        return p.order ? (int64_t)ordered_unit(p.order, (int)slot) : slot;
     };
     auto load_a = [&](const UnitIds &d, const RoundPos &rp) -> float {
         const unsigned h_ = (unsigned)min(rp.hg * 8 + (c & 7), H - 1);
@@ -242,38 +321,21 @@ __device__ __forceinline__ void real_enc_fwd_ring_body(const PairArgs &p, const 
     using Image = RingImage;
     auto load_image = [&](int64_t u_) -> Image { return load_ring_image(cache, u_, lane); };
 
-    // rounds of this work-group: block_id, + grid, + 2 grid, ...; with SELECT those of them that
-    // hold a unit of this launch, known three rounds ahead
-    int rd, rd_next, rd_next2;
-    if (SELECT) {
-        const RoundSeq seq = first_active_rounds(p, block_id, rounds, stride, lane);
-        rd = seq.rd[0];
-        rd_next = seq.rd[1];
-        rd_next2 = seq.rd[2];
-    } else {
-        rd = block_id;
-        rd_next = rd + stride;
-        rd_next2 = rd + 2 * stride;
-    }
-    auto unit_flag = [&](int rd_, const RoundPos &rp) -> int {
-        return SELECT ? load_unit_flag(p, unit_of(rd_, rp), rd_ < rounds ? rp.hg : 0) : 0;
-    };
+    // rounds of this work-group: block_id, + grid, + 2 grid, ...
+    int rd = block_id, rd_next = rd + stride, rd_next2 = rd + 2 * stride;
     RoundPos pos = round_pos(rd, rounds_per_hg, p.head_groups);
     RoundPos pos_next = round_pos(rd_next, rounds_per_hg, p.head_groups);
-    UnitIds ids = unit_ids(load_unit_ids(g_pairs, unit_of(rd, pos), lane));
+    int64_t u = unit_of(rd, pos), u_next = unit_of(rd_next, pos_next);
+    UnitIds ids = unit_ids(load_unit_ids(g_pairs, u, lane));
     float a_cur = load_a(ids, pos);
-    Image img = load_image(unit_of(rd, pos));
-    int uflag = unit_flag(rd, pos);
-    UnitIds ids_next = unit_ids(load_unit_ids(g_pairs, unit_of(rd_next, pos_next), lane));
+    Image img = load_image(u);
+    UnitIds ids_next = unit_ids(load_unit_ids(g_pairs, u_next, lane));
 
     while (rd < rounds) {
         const int hg = pos.hg;
-        const int64_t u = (int64_t)pos.r * WPB + wave;
-        const bool unit_on = u < p.U && (!SELECT || unit_selected(p, uflag));
+        const bool unit_on = (int64_t)pos.r * WPB + wave < p.U;
         const RoundPos pos_next2 = round_pos(rd_next2, rounds_per_hg, p.head_groups);
-        // (the round after rd_next2: its candidates' flags are requested here, looked at at the end)
-        bool candidate = false;
-        if (SELECT) candidate = request_round_candidate(p, rd_next2, rounds, stride, lane);
+        const int64_t u_next2 = unit_of(rd_next2, pos_next2);
         // this round's image into the ring (the previous round's readers of the ring are done:
         // same wavefront, and the epilogue's barriers lie in between)
         const int near_cnt = unit_on ? __builtin_amdgcn_readlane(img.hdr, 0) : 0;
@@ -288,10 +350,9 @@ __device__ __forceinline__ void real_enc_fwd_ring_body(const PairArgs &p, const 
             ring_bits[lane] = 0;
         }
         // loads for the coming rounds
-        const Image img_next = load_image(unit_of(rd_next, pos_next));
+        const Image img_next = load_image(u_next);
         const float a_next = load_a(ids_next, pos_next);
-        const int uflag_next = unit_flag(rd_next, pos_next);
-        const int64_t dv_next2 = load_unit_ids(g_pairs, unit_of(rd_next2, pos_next2), lane);
+        const int64_t dv_next2 = load_unit_ids(g_pairs, u_next2, lane);
         if (hg != wa_hg) {
             const int hw = hg * 8 + wave;
             if (hw < H && K == 16 * NT && D == 16 * DT) {
@@ -436,44 +497,68 @@ __device__ __forceinline__ void real_enc_fwd_ring_body(const PairArgs &p, const 
         ids = ids_next;
         a_cur = a_next;
         img = img_next;
-        uflag = uflag_next;
         ids_next = ids_next2;
         pos = pos_next;
         pos_next = pos_next2;
-        const int rd_next3 = SELECT ? round_after(p, candidate, rd_next2, rounds, stride, lane)
-                                    : rd_next2 + stride;
+        u = u_next;
+        u_next = u_next2;
         rd = rd_next;
         rd_next = rd_next2;
-        rd_next2 = rd_next3;
+        rd_next2 += stride;
     }
 }
 
-template <int NT, int DT, bool SELECT>
+template <int NT, int DT>
 __global__ __launch_bounds__(512, 4) void real_enc_fwd_ring_kernel(PairArgs p_, const float *__restrict__ cache)
 {
     const PairArgs p = with_live_units(p_);
     if (p.U == 0) return;          // (an empty list: not even the descriptor of unit 0 may be read)
-    real_enc_fwd_ring_body<NT, DT, SELECT>(p, cache, (int)blockIdx.x, (int)gridDim.x);
+    real_enc_fwd_ring_body<NT, DT>(p, cache, (int)blockIdx.x, (int)gridDim.x);
 }
 
-// Adaptive boxes in one launch: the first pair_blocks work-groups run the pair kernel's body over the
-// rounds that hold an atom pair which does not keep the cube (few, long rounds; a work-group
-// without such a round leaves at once and frees its place), the others the ring body over the
-// rounds that hold one which does.  Two independent sets of work-groups, each with its own
-// numbering; they write different edges.
+// Adaptive boxes in one launch: the units that keep the cube (first list of the order) run the ring
+// body, the others (second list) the pair kernel's body, at the same time on disjoint sets of
+// work-groups.  How the work-groups are split follows the two counts, which only the device knows:
+// every work-group reads them and takes the same decision, places in proportion to the work of the two
+// lists (a unit of the second list priced at `pair_cost` units of the first), at most one work-group
+// per round, at least one per list that is not empty.
 template <int NT, int DT>
 __global__ __launch_bounds__(512, 4) void real_enc_fwd_two_role_kernel(PairArgs p_ring, PairArgs p_pair,
                                                                        const float *__restrict__ cache,
-                                                                       int pair_blocks)
+                                                                       float pair_cost)
 {
+    PairArgs pr = with_live_units(p_ring), pp = with_live_units(p_pair);
+    if (pr.U < pp.U) {
+        // Fewer than half of the units keep the cube: the split costs more than the rings save (measured
+        // on 256 crystals with r0 = 3 A, 36 % keepers: 515 against 487 us), so the pair body takes all of
+        // them -- the order lists every unit, the first list in front of the second.
+        pp.order = p_pair.order;
+        pp.U += pr.U;
+        pr.U = 0;
+    }
+    const int grid = (int)gridDim.x;
+    const int64_t rounds_ring = (pr.U + WPB - 1) / WPB, rounds_pair = (pp.U + WPB - 1) / WPB;
+    int pair_blocks = 0;
+    if (pp.U > 0) {
+        const float wp = (float)pp.U * pair_cost, wr = (float)pr.U;
+        pair_blocks = (int)((float)grid * (wp / (wp + wr)) + 0.5f);
+        pair_blocks = max(pair_blocks, 1);
+        if (pr.U > 0) pair_blocks = min(pair_blocks, grid - 1);
+        if ((int64_t)pair_blocks > rounds_pair) pair_blocks = (int)rounds_pair;
+    }
+    pair_blocks = __builtin_amdgcn_readfirstlane(pair_blocks);
+    // (tickets for the pair body's rounds only where a work-group has many of them, as in its own launch)
+    if (rounds_pair < 16 * (int64_t)pair_blocks) pp.sched = nullptr;
     if ((int)blockIdx.x < pair_blocks) {
         // (p_pair is the kernel's second argument, behind p_ring in the kernel-argument segment)
         static_assert(sizeof(PairArgs) % 8 == 0, "the second argument follows the first without padding");
         const PairArgsSeg seg = (PairArgsSeg)__builtin_amdgcn_kernarg_segment_ptr() + 1;
-        real_enc_fwd_pair_body<NT, false, PROJ_SHARED, DT, false>(p_pair, seg, (int)blockIdx.x, pair_blocks);
-    } else {
-        real_enc_fwd_ring_body<NT, DT, true>(p_ring, cache, (int)blockIdx.x - pair_blocks,
-                                             (int)gridDim.x - pair_blocks);
+        real_enc_fwd_pair_body<NT, false, PROJ_SHARED, DT, false>(pp, seg, (int)blockIdx.x, pair_blocks);
+    } else if (pr.U > 0) {
+        int ring_blocks = grid - pair_blocks;
+        if ((int64_t)ring_blocks > rounds_ring) ring_blocks = (int)rounds_ring;
+        const int b = (int)blockIdx.x - pair_blocks;
+        if (b < ring_blocks) real_enc_fwd_ring_body<NT, DT>(pr, cache, b, ring_blocks);
     }
 }
 
@@ -512,83 +597,46 @@ int launch_ring_stage(const float *rpos, const float *tvecs, const int64_t *pair
     return CF_OK;
 }
 
-// Flags for the two launches of the adaptive rule (see unit_floor_kernel): unit_flags holds
-// head_groups x U bytes, round_flags one byte per round.
-int64_t real_enc_round_count(int64_t U, int64_t H) { return ((U + WPB - 1) / WPB) * ((H + 7) / 8); }
-
-int launch_unit_floor(const float *a_ik, const float *rvlen, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
-                      float cutoff, int lattice_range, int min_range, unsigned char *unit_flags,
-                      unsigned char *round_flags, hipStream_t st)
+// Adaptive boxes from staged rings: the scratch holds {keepers, others, scheduling words} (4 int64), the order of the
+// units (U ints, rounded up to a multiple of 2), the keepers per chunk and a byte per unit.
+int64_t unit_partition_bytes(int64_t U)
 {
+    if (U <= 0) return 0;
+    const int64_t subs = (U + KEEP_CHUNK - 1) / KEEP_CHUNK;
+    return 32 + ((U + 1) / 2) * 8 + ((subs + 1) / 2) * 8 + ((U + 7) / 8) * 8;
+}
+
+// The two lists of units (see unit_keeps_kernel).  On return (device side) counts[0] / counts[1] hold
+// the numbers of units that keep the cube / do not, order[0 .. counts[0]) the first and
+// order[counts[0] .. U) the second kind.  One head group (H <= 8) only.
+int launch_unit_partition(const float *a_ik, const float *rvlen, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
+                          float cutoff, int lattice_range, int min_range, void *scratch, int64_t **counts_out,
+                          int **order_out, hipStream_t st)
+{
+    if (H > 8 || U < 1 || U >= (1ll << 31)) return CF_ERR_UNSUPPORTED;
+    int64_t *counts = (int64_t *)scratch;
+    int *order = (int *)(counts + 4);
+    int *chunk_keepers = order + ((U + 1) / 2) * 2;
+    const int64_t chunks = (U + PART_CHUNK - 1) / PART_CHUNK, subs = (U + KEEP_CHUNK - 1) / KEEP_CHUNK;
+    unsigned char *keeps = (unsigned char *)(chunk_keepers + ((subs + 1) / 2) * 2);
     PairArgs p{};
     p.a_ik = a_ik; p.rvlen = rvlen; p.pairs = pairs;
     p.N = N; p.U = U; p.H = (int)H;
-    p.head_groups = (int)((H + 7) / 8);
+    p.head_groups = 1;
     p.cutoff = cutoff; p.lattice_range = lattice_range; p.min_range = min_range;
-    const int64_t rounds = real_enc_round_count(U, H);
-    if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;
-    if (rounds < 1) return CF_OK;
-    unit_floor_kernel<<<(int)((rounds + 3) / 4), 256, 0, st>>>(p, unit_flags, round_flags);
-    return CF_OK;
-}
-
-// Adaptive boxes, one launch for both kinds of atom pairs (real_enc_fwd_two_role_kernel).
-int launch_real_enc_fwd_two_role(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,
-                                 const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
-                                 int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
-                                 const float *rvlen, float cutoff, int lattice_range, int min_range,
-                                 const float *cache, const unsigned char *unit_flags,
-                                 const unsigned char *round_flags, float *z, float *v, hipStream_t st)
-{
-    if (K < 1 || K > 128 || !W || D < 1 || D > 32 || cutoff == 0.0f || !unit_flags || !round_flags)
-        return CF_ERR_UNSUPPORTED;
-    if (E * H >= (1ll << 32) || N * H >= (1ll << 32)) return CF_ERR_UNSUPPORTED;      // 32-bit rows in the ring body
-    PairArgs pp{};
-    pp.a_ik = a_ik; pp.rpos = rpos; pp.tvecs = tvecs; pp.batch = batch; pp.edges = edges; pp.pairs = pairs;
-    pp.W = W; pp.rvlen = rvlen; pp.z = z; pp.v = v; pp.sched = nullptr;
-    pp.N = N; pp.E = E; pp.U = U; pp.W_num = 1;
-    pp.H = (int)H; pp.K = (int)K; pp.D = (int)D;
-    pp.head_groups = (int)((H + 7) / 8);
-    pp.cutoff = cutoff; pp.lattice_range = lattice_range; pp.min_range = min_range;
-    pp.bin_step = bin_step; pp.s_scale = s_scale; pp.inv_bin_step = 1.0f / bin_step;
-    pp.window = sqrtf(40.0f) / bin_step;
-    pp.unit_flags = unit_flags; pp.round_flags = round_flags; pp.flag_want = 0;       // pairs that leave the cube
-    PairArgs pr = pp;                                                                   // pairs that keep it
-    pr.rpos = nullptr; pr.tvecs = nullptr; pr.batch = nullptr; pr.edges = nullptr; pr.rvlen = nullptr;
-    pr.cutoff = 0.f; pr.flag_want = 1;
-    const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
-    const int DT = D > 16 ? 2 : 1;
-    const size_t shared_proj = sizeof(float) * ((size_t)4 * NT * XPLANE + WPB * 16) + sizeof(int64_t) * WPB * 2 + 8;
-    const size_t lds_ring = sizeof(float) * (size_t)WPB * 3 * RS + shared_proj;
-    const size_t lds_pair = sizeof(float) * (size_t)WPB * 3 * (RING_CAP + 16) + shared_proj;
-    const size_t lds = lds_ring > lds_pair ? lds_ring : lds_pair;
-    const int64_t rounds = ((U + WPB - 1) / WPB) * pp.head_groups;
-    if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;
-    if (rounds < 1) return CF_OK;
-    const int64_t cap = persistent_grid_cap(2);
-    const int64_t ring_blocks = rounds < cap ? rounds : cap;
-    int64_t pair_blocks = cap / 8 < 1 ? 1 : cap / 8;       // few long rounds: an eighth of the places, freed at once where idle
-    if (pair_blocks > rounds) pair_blocks = rounds;
-    const int grid = (int)(ring_blocks + pair_blocks);
-#define CF_TWO(NTV, DTV) \
-    real_enc_fwd_two_role_kernel<NTV, DTV><<<grid, WPB * WAVE, lds, st>>>(pr, pp, cache, (int)pair_blocks)
-#define CF_TWO_NT(NTV) do { if (DT == 1) CF_TWO(NTV, 1); else CF_TWO(NTV, 2); } while (0)
-    switch (NT) {
-        case 1: CF_TWO_NT(1); break;
-        case 2: CF_TWO_NT(2); break;
-        case 4: CF_TWO_NT(4); break;
-        default: CF_TWO_NT(8); break;
-    }
-#undef CF_TWO_NT
-#undef CF_TWO
+    p.live_U = live_units(U);
+    unit_keeps_kernel<<<(int)subs, PART_CHUNK, 0, st>>>(p, keeps, chunk_keepers);
+    partition_kernel<<<(int)chunks, PART_CHUNK, 0, st>>>(keeps, chunk_keepers, U, p.live_U, order, counts);
+    *counts_out = counts;
+    *order_out = order;
     return CF_OK;
 }
 
 // Forward from staged rings (shared projection, D <= 32).  CF_ERR_UNSUPPORTED otherwise.
-// With unit flags only the units that keep the cube are evaluated.
+// With an order only the first *n_units units it lists are evaluated (n_units on the device).
 int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U, int64_t N, int64_t H, int64_t E,
                               int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
-                              const float *cache, const unsigned char *unit_flags, const unsigned char *round_flags,
+                              const float *cache, const int *order, const int64_t *n_units,
                               float *z, float *v, hipStream_t st)
 {
     if (K < 1 || K > 128 || !W || D < 1 || D > 32) return CF_ERR_UNSUPPORTED;
@@ -600,10 +648,8 @@ int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U
     p.head_groups = (int)((H + 7) / 8);
     p.bin_step = bin_step; p.s_scale = s_scale; p.inv_bin_step = 1.0f / bin_step;
     p.window = sqrtf(40.0f) / bin_step;
-    p.unit_flags = unit_flags; p.round_flags = round_flags; p.flag_want = 1;      // units that keep the cube
-    const bool select = unit_flags != nullptr;
-    p.live_U = live_units(U);
-    if (p.live_U && select) return CF_ERR_UNSUPPORTED;       // (the flags are laid out for a known U)
+    p.live_U = order ? n_units : live_units(U);
+    p.order = order;
     const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
     const int DT = D > 16 ? 2 : 1;
     size_t lds = sizeof(float) * ((size_t)WPB * 3 * RS + (size_t)4 * NT * XPLANE + WPB * 16) +
@@ -614,11 +660,7 @@ int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U
     const int64_t cap = persistent_grid_cap(2);
     if (blocks > cap) blocks = cap;
     if (blocks < 1) return CF_OK;
-#define CF_RING(NTV, DTV)                                                                               \
-    do {                                                                                                \
-        if (select) real_enc_fwd_ring_kernel<NTV, DTV, true><<<(int)blocks, WPB * WAVE, lds, st>>>(p, cache);   \
-        else real_enc_fwd_ring_kernel<NTV, DTV, false><<<(int)blocks, WPB * WAVE, lds, st>>>(p, cache);         \
-    } while (0)
+#define CF_RING(NTV, DTV) real_enc_fwd_ring_kernel<NTV, DTV><<<(int)blocks, WPB * WAVE, lds, st>>>(p, cache)
 #define CF_RING_NT(NTV) do { if (DT == 1) CF_RING(NTV, 1); else CF_RING(NTV, 2); } while (0)
     switch (NT) {
         case 1: CF_RING_NT(1); break;
@@ -628,6 +670,61 @@ int launch_real_enc_fwd_rings(const float *a_ik, const int64_t *pairs, int64_t U
     }
 #undef CF_RING_NT
 #undef CF_RING
+    return CF_OK;
+}
+
+// Adaptive boxes: both lists of launch_unit_partition in one launch (real_enc_fwd_two_role_kernel).
+int launch_real_enc_fwd_two_role(const float *a_ik, const float *rpos, const float *tvecs, const int64_t *batch,
+                                 const int64_t *edges, const int64_t *pairs, int64_t U, int64_t N, int64_t H,
+                                 int64_t E, int64_t K, int64_t D, float bin_step, float s_scale, const float *W,
+                                 const float *rvlen, float cutoff, int lattice_range, int min_range,
+                                 const float *cache, const int *order, const int64_t *counts, float *z, float *v,
+                                 hipStream_t st)
+{
+    if (K < 1 || K > 128 || !W || D < 1 || D > 32 || cutoff == 0.0f || !order || !counts || H > 8)
+        return CF_ERR_UNSUPPORTED;
+    if (E * H >= (1ll << 32) || N * H >= (1ll << 32)) return CF_ERR_UNSUPPORTED;      // 32-bit rows in the ring body
+    PairArgs pp{};
+    pp.a_ik = a_ik; pp.rpos = rpos; pp.tvecs = tvecs; pp.batch = batch; pp.edges = edges; pp.pairs = pairs;
+    pp.W = W; pp.rvlen = rvlen; pp.z = z; pp.v = v; pp.sched = nullptr;
+    pp.N = N; pp.E = E; pp.U = U; pp.W_num = 1;
+    pp.H = (int)H; pp.K = (int)K; pp.D = (int)D;
+    pp.head_groups = 1;
+    pp.cutoff = cutoff; pp.lattice_range = lattice_range; pp.min_range = min_range;
+    pp.bin_step = bin_step; pp.s_scale = s_scale; pp.inv_bin_step = 1.0f / bin_step;
+    pp.window = sqrtf(40.0f) / bin_step;
+    pp.order = order; pp.order_first = counts; pp.live_U = counts + 1;              // the units that leave the cube
+    pp.sched = reinterpret_cast<unsigned int *>(const_cast<int64_t *>(counts) + 2); // (zeroed with the counts)
+    PairArgs pr = pp;                                                               // the units that keep it
+    pr.rpos = nullptr; pr.tvecs = nullptr; pr.batch = nullptr; pr.edges = nullptr; pr.rvlen = nullptr;
+    pr.cutoff = 0.f; pr.order_first = nullptr; pr.live_U = counts; pr.sched = nullptr;
+    const int NT = K <= 16 ? 1 : K <= 32 ? 2 : K <= 64 ? 4 : 8;
+    const int DT = D > 16 ? 2 : 1;
+    const size_t shared_proj = sizeof(float) * ((size_t)4 * NT * XPLANE + WPB * 16) + sizeof(int64_t) * WPB * 2 + 8;
+    const size_t lds_ring = sizeof(float) * (size_t)WPB * 3 * RS + shared_proj;
+    const size_t lds_pair = sizeof(float) * (size_t)WPB * 3 * (RING_CAP + 16) + shared_proj;
+    const size_t lds = lds_ring > lds_pair ? lds_ring : lds_pair;
+    const int64_t rounds = (U + WPB - 1) / WPB;
+    if (rounds >= (1ll << 30)) return CF_ERR_UNSUPPORTED;
+    if (rounds < 1) return CF_OK;
+    const int64_t cap = persistent_grid_cap(2);
+    const int grid = (int)(rounds < cap ? rounds : cap);
+    // a unit that leaves the cube costs about this many units that keep it (its box holds more
+    // translations, and they are staged in the launch)
+    // (swept on 128 and 256 crystals: 1.5 / 2 / 2.5 / 3 / 4 give 0.506 / 0.461 / 0.431 / 0.420 / 0.414 ms per
+    // forward of the default model and 3.45 / 3.17 / 3.20 / 3.19 / 3.45 ms of the seven-block one)
+    const float pair_cost = 3.0f;
+#define CF_TWO(NTV, DTV) \
+    real_enc_fwd_two_role_kernel<NTV, DTV><<<grid, WPB * WAVE, lds, st>>>(pr, pp, cache, pair_cost)
+#define CF_TWO_NT(NTV) do { if (DT == 1) CF_TWO(NTV, 1); else CF_TWO(NTV, 2); } while (0)
+    switch (NT) {
+        case 1: CF_TWO_NT(1); break;
+        case 2: CF_TWO_NT(2); break;
+        case 4: CF_TWO_NT(4); break;
+        default: CF_TWO_NT(8); break;
+    }
+#undef CF_TWO_NT
+#undef CF_TWO
     return CF_OK;
 }
 
@@ -644,7 +741,10 @@ void bin_scales(int64_t K, double dist_max, double wscale, float &bin_step, floa
 }
 }  // namespace
 
-extern "C" int64_t cf_real_enc_ring_bytes(int64_t U) { return (U < 0 ? 0 : U) * RIMG_WORDS * (int64_t)sizeof(float); }
+extern "C" int64_t cf_real_enc_ring_bytes(int64_t U)
+{
+    return U <= 0 ? 0 : U * RIMG_WORDS * (int64_t)sizeof(float);
+}
 
 extern "C" int cf_real_enc_ring_stage(const float *rpos_ij_e, const float *tvecs_n, const int64_t *pairs_u, int64_t U,
                                       int64_t K, double dist_max, double wscale, int lattice_range,
@@ -671,7 +771,7 @@ extern "C" int cf_real_enc_ring_stage(const float *rpos_ij_e, const float *tvecs
 extern "C" int64_t cf_real_enc_flag_bytes(int64_t U, int64_t H)
 {
     if (U < 0 || H < 1) return 0;
-    return ((H + 7) / 8) * U + cf::real_enc_round_count(U, H);
+    return cf::unit_partition_bytes(U);
 }
 
 extern "C" int cf_real_enc_fwd_rings(const float *a_ik, const float *rpos_ij_e, const float *tvecs_n,
@@ -709,29 +809,33 @@ extern "C" int cf_real_enc_fwd_rings(const float *a_ik, const float *rpos_ij_e, 
     }
     // Adaptive boxes: the units whose columns all keep the cube from the rings, the rest by the
     // pair kernel; both write their own edges of z and v.
-    CF_REQUIRE(!cf::live_units(U), CF_ERR_UNSUPPORTED,
-               "cf_real_enc_fwd_rings: adaptive boxes from the rings need sizes known on the host "
-               "(a size header is set): use cf_real_enc_fwd");
     CF_REQUIRE(minimum_range >= 0 && minimum_range <= MAX_RANGE, CF_ERR_INVALID_ARGUMENT,
                "cf_real_enc_fwd_rings: minimum_range %d outside 0..%d", minimum_range, MAX_RANGE);
     CF_REQUIRE(rpos_ij_e && tvecs_n && batch_i && edge_ij_e, CF_ERR_INVALID_ARGUMENT,
                "cf_real_enc_fwd_rings: adaptive boxes need rpos_ij_e, tvecs_n, batch_i and edge_ij_e");
+    if (H > 8) {
+        // (the two lists are per head group; with more than one, every unit goes to the pair kernel)
+        int rc = cf::launch_real_enc_fwd_pairs(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, N, H, E, K, D,
+                                               bin_step, s_scale, W_k, 1, rvlen_n, cutoff, lattice_range, minimum_range,
+                                               nullptr, nullptr, nullptr, z_ek, v_ekd, st);
+        CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported shape");
+        CF_CHECK_LAUNCH("cf_real_enc_fwd_rings (adaptive boxes)");
+        return CF_OK;
+    }
     CF_REQUIRE(flags && flag_bytes >= cf_real_enc_flag_bytes(U, H), CF_ERR_INVALID_ARGUMENT,
                "cf_real_enc_fwd_rings: adaptive boxes need %lld bytes of flags, %lld given",
                (long long)cf_real_enc_flag_bytes(U, H), (long long)flag_bytes);
-    unsigned char *unit_flags = (unsigned char *)flags;
-    unsigned char *round_flags = unit_flags + ((H + 7) / 8) * U;
-    int rc = cf::launch_unit_floor(a_ik, rvlen_n, pairs_u, U, N, H, cutoff, lattice_range, minimum_range, unit_flags,
-                                   round_flags, st);
+    // Two lists of units, then one launch with a role for each: from the rings the units that keep the
+    // cube, the pair kernel's body for the others.  Either list may be empty or hold everything; the
+    // counts stay on the device.
+    int64_t *counts = nullptr;
+    int *order = nullptr;
+    int rc = cf::launch_unit_partition(a_ik, rvlen_n, pairs_u, U, N, H, cutoff, lattice_range, minimum_range, flags,
+                                       &counts, &order, st);
     CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported size");
-    // One launch for both kinds of atom pairs.  (Tried before: the two kernels one after the other,
-    // 60.4 us per block at 128 crystals, the pair kernel's part being one long round of a few
-    // work-groups; and that launch on a second stream between two events beside the ring launch, where
-    // fork and join cost more than the overlap won, 62.5 us and 0.31 against 0.26 ms per step with
-    // four forwards in flight.)
     rc = cf::launch_real_enc_fwd_two_role(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, pairs_u, U, N, H, E, K, D,
                                           bin_step, s_scale, W_k, rvlen_n, cutoff, lattice_range, minimum_range,
-                                          (const float *)rings, unit_flags, round_flags, z_ek, v_ekd, st);
+                                          (const float *)rings, order, counts, z_ek, v_ekd, st);
     CF_REQUIRE(rc == CF_OK, rc, "cf_real_enc_fwd_rings: unsupported shape");
     CF_CHECK_LAUNCH("cf_real_enc_fwd_rings (adaptive boxes)");
     return CF_OK;

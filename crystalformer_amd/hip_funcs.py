@@ -83,12 +83,11 @@ class KernelManager:
     # attention module passes with its call (-gauss_lb / (2 r0^2), the encoding Function's last
     # argument); without one every launch stages for itself.
     STAGED_RINGS: bool = True
-    # Adaptive boxes from the staged rings (forward): atom pairs whose half-widths all come out as
-    # LATTICE_RANGE start from their rings, the others are staged by the pair kernel's body in the same
-    # launch.  Off by default: it pays where nearly all pairs keep the cube (default model, inference, 128
-    # crystals: 0.426 against 0.471 ms per forward) and costs where many do not (the split of the
-    # work-groups between the two kinds is fixed, and a round that holds both kinds is walked twice).
-    ADAPTIVE_RINGS = False
+    # Adaptive boxes from the staged rings (forward, up to 8 heads): the atom pairs whose half-widths all
+    # come out as LATTICE_RANGE have exactly the cube and start from their rings, the others are staged by
+    # the pair kernel; two stably ordered lists of units and their counts are worked out on the device,
+    # and each kernel walks dense rounds of its own list, whatever the split is.
+    ADAPTIVE_RINGS = True
     compiled: bool = False
 
 
@@ -190,8 +189,7 @@ class RealPeriodicEncodingWithProjFuncCUDA(torch.autograd.Function):
         fixed_cube = rvlen_n is None or cutoff_radius is None or float(cutoff_radius) == 0.0
         # (adaptive boxes too: atom pairs whose half-widths all come out as LATTICE_RANGE have exactly
         # the cube and start from the rings, the others are staged by the pair kernel)
-        # (adaptive boxes: on request only, see KernelManager.ADAPTIVE_RINGS)
-        worth_it = fixed_cube or (KernelManager.ADAPTIVE_RINGS and ops.current_live_sizes() is None)
+        worth_it = fixed_cube or (KernelManager.ADAPTIVE_RINGS and a_ik.shape[1] <= 8)
         if (KernelManager.STAGED_RINGS and weakest_exponent is not None and pairs_u is not None
                 and worth_it and K > 0 and W_k is not None and _w_leading(W_k) == 1 and W_k.shape[-2] <= 32):
             rings = ops.staged_rings(rpos_ij_e, tvecs_n, pairs_u, K, dist_max, wscale, KernelManager.LATTICE_RANGE,

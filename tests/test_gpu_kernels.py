@@ -1367,9 +1367,10 @@ def test_staged_rings_limits(dev):
 @pytest.mark.parametrize("cutoff,lr,mr", [(-3.5, 2, 2), (-3.5, 1, 1), (-2.0, 2, 2), (5.0, 1, 1), (-3.5, 2, 0)])
 @pytest.mark.parametrize("H,K,D", [(8, 64, 16), (4, 16, 8), (16, 32, 8), (2, 100, 4), (8, 64, 32)])
 def test_real_enc_fwd_from_staged_rings_with_adaptive_boxes(dev, H, K, D, cutoff, lr, mr):
-    """Adaptive boxes in two launches: atom pairs whose half-widths all come out as lattice_range start from
-    the staged rings, the others are staged by the pair kernel.  Against the oracle and against the pair
-    kernel alone; the problems hold pairs of both kinds."""
+    """Adaptive boxes from staged rings: atom pairs whose half-widths all come out as lattice_range start from
+    the rings, the others are staged by the pair kernel, each kind in a launch over its own list of units (16
+    heads: all by the pair kernel).  Against the oracle and against the pair kernel alone; the problems hold
+    pairs of both kinds."""
     p = Problem([1, 3, 9, 2, 17, 1, 6], H=H, K=K, D=D, seed=41)
     z_ref, v_ref = enc_fwd_ref(p, K, p.W, cutoff, lr, mr)
     rpos, tv, pairs, rings = _staged(dev, p, K, lr)

@@ -890,14 +890,15 @@ def test_blocks_share_one_staging_of_the_translations(dev):
         torch.cuda.synchronize()
 
 
-def test_adaptive_boxes_take_the_staged_rings_on_request(dev):
-    """The reference kernels' default rule (adaptive boxes, floor at lattice_range): with ADAPTIVE_RINGS the
-    forward runs as selection + one launch in which the pairs that keep the cube start from the staged rings and
-    the others are staged; outputs and gradients equal those of the pair kernel alone.  Off by default."""
+def test_adaptive_boxes_take_the_staged_rings(dev):
+    """The reference kernels' default rule (adaptive boxes, floor at lattice_range): the forward splits the
+    atom pairs on the device into those that keep the cube, which start from the staged rings, and the
+    others, which the pair kernel stages; outputs and gradients equal those of the pair kernel alone
+    (KernelManager.ADAPTIVE_RINGS off)."""
     name = "cfg2_default_b128"
     b = select_crystals(make_config_batch(name), range(40)).to(dev)
     cfg, model = build_model(name)                     # adaptive_cutoff_sigma = -3.5, minimum_range on
-    assert cfg.adaptive_cutoff_sigma < 0 and not hip_funcs.KernelManager.ADAPTIVE_RINGS
+    assert cfg.adaptive_cutoff_sigma < 0 and hip_funcs.KernelManager.ADAPTIVE_RINGS
     model.to(dev).train()
     model(b)                                           # first training pass: stores the batch statistics
 
@@ -912,7 +913,7 @@ def test_adaptive_boxes_take_the_staged_rings_on_request(dev):
             return y.detach().clone(), {k: p.grad.clone() for k, p in model.named_parameters()
                                         if p.grad is not None}, [entry[0] for entry in log]
         finally:
-            hip_funcs.KernelManager.ADAPTIVE_RINGS = False
+            hip_funcs.KernelManager.ADAPTIVE_RINGS = True
             ops.set_event_log(None)
     y1, g1, names1 = step(True)
     y0, g0, names0 = step(False)
