@@ -32,8 +32,9 @@ PEAK_FP32_TFLOPS = 157.3          # fp32 on the matrix cores (and packed vector 
 PEAK_FP32_VALU_TFLOPS = 78.6      # one fp32 FMA per lane and cycle: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz x 2
 PEAK_HBM_GBS = 8000.0
 PROFILE_FILE = os.path.join(ROOT, "profiles", "traffic.json")
-KERNEL_SOURCES = {"fwd": ("real_enc_ring.hip", "real_enc_mfma.hip", "real_enc_pair_fwd.h", "real_enc_pair.h", "cf_common.h"),
-                  "bwd": ("real_enc_mfma_bwd.hip", "real_enc_pair.h", "cf_common.h")}
+KERNEL_SOURCES = {"fwd": ("real_enc_ring.hip", "real_enc_mfma.hip", "real_enc_pair_fwd.h", "real_enc_pair.h", "cf_common.h",
+                          "cf_index_rules.h"),
+                  "bwd": ("real_enc_mfma_bwd.hip", "real_enc_pair.h", "cf_common.h", "cf_index_rules.h")}
 
 
 def kernel_fingerprint(direction: str) -> str:
@@ -69,9 +70,14 @@ def stored_counters(key: str, required: bool):
     now = kernel_fingerprint(key.rsplit(":", 1)[1])
     entry["current"] = entry.get("kernel_sha16") == now
     if not entry["current"]:
-        print(f"bench.py: WARNING: counters for '{key}' were taken with other kernel sources "
-              f"({entry.get('kernel_sha16')} at {entry.get('commit')}, now {now}); "
-              f"the executed-work figures in the line are stale", file=sys.stderr)
+        msg = (f"counters for '{key}' were taken with other kernel sources ({entry.get('kernel_sha16')} at "
+               f"{entry.get('commit')}, now {now})")
+        if required:
+            raise SystemExit(f"bench.py: {msg}: collect them again (bench.py --profile-kernel under rocprofv3 --pmc, "
+                             f"then --ingest-counters), or pass --no-counters to report the roofline without "
+                             f"executed work")
+        print(f"bench.py: WARNING: {msg}; they are not used", file=sys.stderr)
+        return None
     return entry
 
 
@@ -417,9 +423,11 @@ def main() -> int:
     if args.ingest_counters:
         cfg_name = "cfg4_train_b128" if (args.train and args.config == "cfg2_default_b128") else args.config
         key = args.ingest_key or f"{cfg_name}:{args.rule}:{'bwd' if args.train else 'fwd'}"
-        staged = args.rule == "A" and not args.no_staged_rings     # forward: from the staged rings (fixed cube)
+        # forward: from the staged rings (fixed cube), both roles in one launch (adaptive boxes), or the pair kernel
+        staged = not args.no_staged_rings and (args.rule == "A" or not args.no_adaptive_rings)
         kernel = args.ingest_kernel or ("real_enc_bwd_pair_kernel" if args.train else
-                                        "real_enc_fwd_ring_kernel" if staged else "real_enc_fwd_pair_kernel")
+                                        ("real_enc_fwd_ring_kernel" if args.rule == "A" else
+                                         "real_enc_fwd_two_role_kernel") if staged else "real_enc_fwd_pair_kernel")
         return ingest_counters(args.ingest_counters, key, kernel)
 
     if args.gpus != 1:
@@ -601,8 +609,11 @@ def main() -> int:
                                                                   required=not args.no_counters)
     work = executed_work(counters, enc_avg_ms) if (counters and enc_avg_ms > 0) else None
     roofline = {
-        "kernel": ("real_enc_fwd_ring_kernel (periodic encoding forward from the staged translations, projection "
-                   "fused)" if calls["real_enc_fwd_rings"] else
+        "kernel": (("real_enc_fwd_ring_kernel (periodic encoding forward from the staged translations, projection "
+                    "fused)" if args.rule == "A" else
+                    "real_enc_fwd_two_role_kernel (periodic encoding forward, adaptive boxes: atom pairs that keep the "
+                    "cube from the staged translations, the others staged in the same launch; with its two list-building "
+                    "launches)") if calls["real_enc_fwd_rings"] else
                    "real_enc_fwd_pair_kernel (periodic encoding forward, projection fused)"),
         "bound": "mfma",
         # executed fp32 work (instruction counters of a stored rocprofv3 --pmc run of this kernel
