@@ -70,7 +70,8 @@ double cf_get_launch_share(void);
  * the first live N (E, U) items only; results for those are bit-identical to a call with the
  * live sizes as arguments.  Entry points: cf_batch_layout, cf_edge_index, cf_edge_pairs,
  * cf_gauss_exponents, cf_linear_rows (rows = atoms), cf_real_enc_ring_stage,
- * cf_real_enc_fwd_rings (fixed cube), cf_real_enc_fwd (pair list), cf_fused_dpa_fwd.  The other
+ * cf_real_enc_fwd_rings (either rule), cf_real_enc_fwd (pair list; without one it refuses),
+ * cf_fused_dpa_fwd.  The other
  * entry points ignore the header (per-crystal ones run over all B lattices handed in; crystals
  * beyond the live ones must have size 0).  Read at launch: a captured graph keeps the header
  * address it was captured with.
@@ -144,13 +145,18 @@ int cf_real_enc_fwd(const float *a_ik, const float *rpos_ij_e, const float *tvec
  * Adaptive boxes (rvlen_n given and cutoff_radius != 0, the rule of
  * models/kernels/real_enc_fwd.cu:58-85): atom pairs whose (atom, head) half-widths all come out as
  * lattice_range have exactly the cube and are evaluated from the rings; the others are staged and
- * evaluated as cf_real_enc_fwd does.  Two launches: the selection (the range rule per atom pair and
- * head group, into `flags`: cf_real_enc_flag_bytes(U, H) bytes of device scratch written and read by
- * the call), then one launch whose work-groups take one of two roles, the rings' body over the
- * rounds that hold a pair which keeps the cube and the staging body over the rounds that hold one
- * which does not.  That launch needs up to 87 KB of dynamic LDS per work-group at K > 64 (53 KB at
- * K <= 64).  With the fixed cube rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n and flags may be
- * NULL, and there is one launch.
+ * evaluated as cf_real_enc_fwd does.  Three launches: the range rule per atom pair (a byte per
+ * pair, a count per chunk of 128); a stable partition of the pair indices into two lists, the
+ * pairs that keep the cube first, with both lengths beside them; then one launch whose
+ * work-groups take one of two roles, the rings' body over the first list and the staging body
+ * over the second, the split worked out on the device from the two lengths (where fewer than
+ * half the pairs keep the cube the staging body takes all of them).  All of it lives in `flags`:
+ * cf_real_enc_flag_bytes(U, H) = 32 + 8 (ceil(U/2) + ceil(ceil(U/128)/2) + ceil(U/8)) bytes of
+ * device scratch, 8-byte aligned, written and read by the call; nothing in it needs clearing.
+ * The last launch needs up to 87 KB of dynamic LDS per work-group at K > 64 (53 KB at K <= 64).
+ * More than 8 heads: the staging body alone, over all pairs.  Works under a size header (U is
+ * then the capacity).  With the fixed cube rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n and
+ * flags may be NULL, and there is one launch.
  */
 int64_t cf_real_enc_ring_bytes(int64_t U);
 int64_t cf_real_enc_flag_bytes(int64_t U, int64_t H);
