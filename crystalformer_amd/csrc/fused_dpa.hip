@@ -151,6 +151,12 @@ __device__ __forceinline__ float4_v ld4(const void *base, uint32_t byte_off)
 {
     return *reinterpret_cast<const float4_v *>(static_cast<const char *>(base) + byte_off);
 }
+// The same for data that is read once (the b_ij stream): marked as streaming so that it does not
+// push the key / value rows, which every query row of a crystal reads again, out of the caches.
+__device__ __forceinline__ float4_v ld4_stream(const void *base, uint32_t byte_off)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const float4_v *>(static_cast<const char *>(base) + byte_off));
+}
 __device__ __forceinline__ float ld1(const void *base, uint32_t byte_off)
 {
     return *reinterpret_cast<const float *>(static_cast<const char *>(base) + byte_off);
@@ -198,7 +204,7 @@ __global__ __launch_bounds__(256, (PREFETCH ? 6 : 7)) void fused_dpa_fwd_stream_
     float4_v k4[4], v4[4], b4[4];
     float av[4];
     auto fetch = [&](int u, uint32_t e, uint32_t j) {
-        if (HAS_B) b4[u] = ld4(p.bij, (e * HD4 + piece) * 16u);      // independent of the key index: first
+        if (HAS_B) b4[u] = ld4_stream(p.bij, (e * HD4 + piece) * 16u);   // independent of the key index: first
         if (HAS_A) av[u] = ld1(p.aij, (e * H + h) * 4u);
         k4[u] = ld4(p.key, (j * HD4 + piece) * 16u);
         v4[u] = ld4(p.val, (j * HD4 + piece) * 16u);
@@ -322,6 +328,11 @@ __device__ __forceinline__ void st4(void *base, uint32_t byte_off, float4_v v)
 {
     *reinterpret_cast<float4_v *>(static_cast<char *>(base) + byte_off) = v;
 }
+// (for data written once and not read again by this launch: the gb_ij stream)
+__device__ __forceinline__ void st4_stream(void *base, uint32_t byte_off, float4_v v)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<float4_v *>(static_cast<char *>(base) + byte_off));
+}
 
 template <int DV4, bool HAS_B, bool WANT_GB>
 __global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs p, int LPE)
@@ -361,7 +372,7 @@ __global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             pr[u] = ld1(p.prob_in, (ec[u] * H + h) * 4u);
-            if (HAS_B) b4[u] = ld4(p.bij, (ec[u] * HD4 + piece) * 16u);
+            if (HAS_B) b4[u] = ld4_stream(p.bij, (ec[u] * HD4 + piece) * 16u);
             m4[u] = ld4(p.val, (j[u] * HD4 + piece) * 16u);
         }
 #pragma unroll
@@ -374,7 +385,7 @@ __global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs
             float gs = d4.x * t4.x + d4.y * t4.y + d4.z * t4.z + d4.w * t4.w;
             gs = head_sum<DV4>(gs);
             if (valid) {
-                if (WANT_GB) st4(p.gbij, (ec[u] * HD4 + piece) * 16u, t4);
+                if (WANT_GB) st4_stream(p.gbij, (ec[u] * HD4 + piece) * 16u, t4);
                 if (lead) st1(p.gaij, (ec[u] * H + h) * 4u, gs);
             }
             gsv[u] = valid ? gs : 0.f;

@@ -483,6 +483,42 @@ def test_fused_dpa_fwd_on_an_arbitrary_edge_list(dev, H, D):
     assert float(out.cpu()[~has].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("H,D,sizes", [(8, 16, [70, 90, 3, 130, 1, 101]), (4, 16, [150, 5, 160, 137]),
+                                       (16, 16, [33, 70, 2, 45]), (8, 8, [150, 131, 7, 160]),
+                                       (2, 32, [130, 171, 1])])
+@pytest.mark.parametrize("bias,vals", [(True, True), (False, True), (True, False), (False, False)])
+def test_fused_dpa_fwd_long_rows(dev, H, D, sizes, bias, vals):
+    """Rows longer than two steps of a work-group on average take the variant that keeps the key
+    indices a step ahead and every load of a step in flight: lane layouts of 16, 32 and 64 lanes per
+    edge, crystals whose sizes are no multiple of a step (single-atom crystals between long ones),
+    with and without a_ij / b_ij."""
+    p, q, k, v, a, b = dpa_problem(sizes, H, D, D, 36, bias, vals)
+    assert p.E > 2 * (16 * 64 // (H * D // 4)) * p.N            # the launch rule for long rows
+    out, prob = ops.fused_dpa_fwd(*to_dev(dev, q, k, v, a, b, p.edges, p.e_start))
+    out_ref, prob_ref = ks.fused_dpa_fwd(q, k, v, a, b, p.edges, p.e_start)
+    out_atol, _ = dpa_atols(p, q, k, v, b, prob_ref, out_ref)
+    assert_close(out, out_ref, "out", atol=out_atol)
+    assert_close(prob, prob_ref, "prob", atol=ATOL_PROB)
+
+
+def test_fused_dpa_fwd_long_rows_on_an_arbitrary_edge_list(dev):
+    """The same variant on an edge list that is no dense block (a random fifth of the edges removed,
+    one atom without edges)."""
+    p, q, k, v, a, b = dpa_problem([120, 150, 90], 8, 16, 16, 37)
+    gen = torch.Generator().manual_seed(6)
+    keep = torch.rand(p.E, generator=gen) > 0.2
+    keep &= p.edges[0] != 133
+    edges = p.edges[:, keep].contiguous()
+    e_start = tp.edge_row_offsets(edges, p.N)
+    a, b = a[keep].contiguous(), b[keep].contiguous()
+    assert edges.shape[1] > 2 * 32 * p.N
+    out, prob = ops.fused_dpa_fwd(*to_dev(dev, q, k, v, a, b, edges, e_start))
+    out_ref, prob_ref = ks.fused_dpa_fwd(q, k, v, a, b, edges, e_start)
+    assert_close(out, out_ref, "out")
+    assert_close(prob, prob_ref, "prob", atol=ATOL_PROB)
+    assert float(out[133].abs().max()) == 0.0
+
+
 def test_fused_dpa_beyond_the_reference_size_limit(dev):
     """The reference's kernels stop at 320 atoms per crystal; these do not."""
     p, q, k, v, a, b = dpa_problem([444, 3], 8, 16, 16, 32)
