@@ -197,7 +197,11 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             self.lattice_pos_weights = None
         elif params.gauss_state.startswith("q") or params.gauss_state == "1":
             self.lattice_pos_weights = Parameter(torch.empty((self.kdim), **kw))
-        elif params.gauss_state.startswith("x") and params.gauss_state != "x-xn":
+        elif params.gauss_state == "x-xn":
+            # two factors, multiplied in forward (models/indexed_lattice_multi_head_attention_cuda.py:859-861, 993-997)
+            self.lattice_pos_weights = Parameter(torch.empty((self.kdim, embed_dim), **kw))
+            self.lattice_pos_weights2 = Parameter(torch.empty((self.kdim), **kw))
+        elif params.gauss_state.startswith("x"):
             self.lattice_pos_weights = Parameter(torch.empty((num_heads, embed_dim), **kw))
         else:
             raise NotImplementedError(f"gauss_state={params.gauss_state!r}")
@@ -217,6 +221,16 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             raise NotImplementedError("value_pe_wave_* > 0 has no HIP kernel")
         self._reset_parameters()
 
+    def position_weights(self) -> Optional[Tensor]:
+        """The weights that turn a query (or the block input) into the Gaussian exponents' raw value:
+        the parameter itself, or for ``gauss_state="x-xn"`` the product of its two factors, (H, embed_dim)
+        (models/indexed_lattice_multi_head_attention_cuda.py:992-997)."""
+        W = self.lattice_pos_weights
+        if W is not None and self.params.gauss_state == "x-xn":
+            H, K, D = self.num_heads, self.kdim, self.embed_dim
+            W = (self.lattice_pos_weights2.view(H, 1, K // H) @ W.reshape(H, K // H, D)).reshape(H, D)
+        return W
+
     def _reset_parameters(self):
         xavier_uniform_(self.q_proj_weight)
         xavier_uniform_(self.k_proj_weight)
@@ -235,6 +249,20 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                 normal_(self.lattice_pos_weights, 0., self.embed_dim ** -0.5)
             elif gs == "x-xavier":
                 xavier_uniform_(self.lattice_pos_weights)
+            elif gs == "x-xn":
+                xavier_uniform_(self.lattice_pos_weights)
+                normal_(self.lattice_pos_weights2, 0., (self.kdim // self.num_heads) ** -0.5)
+            elif gs == "x-xn2":
+                # the product of the two factors of "x-xn", drawn once
+                # (models/indexed_lattice_multi_head_attention_cuda.py:905-915)
+                H, K, D = self.num_heads, self.kdim, self.embed_dim
+                W = self.lattice_pos_weights
+                W1 = torch.empty((K, D), device=W.device, dtype=W.dtype)
+                W2 = torch.empty((H, 1, K // H), device=W.device, dtype=W.dtype)
+                xavier_uniform_(W1)
+                normal_(W2, 0., (K // H) ** -0.5)
+                with torch.no_grad():
+                    W.copy_((W2 @ W1.reshape(H, K // H, D)).reshape_as(W))
             else:
                 raise NotImplementedError(gs)
         if self.pe_dist_proj is not None:
@@ -306,7 +334,7 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                     self.training, spec[0], spec[1], P.gauss_lb_real, -0.5 * P.scale_real ** -2,
                     1.0 / math.sqrt(q.shape[-1]))
             else:
-                a = gaussian_exponents(q, query, self.lattice_pos_weights, self.gauss_scale, P, self.training)
+                a = gaussian_exponents(q, query, self.position_weights(), self.gauss_scale, P, self.training)
             dist_max = P.value_pe_dist_max
             if dist_max < 0:
                 dist_max = (-dist_max) * P.scale_real
@@ -439,7 +467,7 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             a1, a2 = rho[:, :H // 2] * coef_real, rho[:, H // 2:] * coef_reci
         else:
             func = make_positive_func(P.positive_func)
-            alpha = normalised_alpha(q, query, self.lattice_pos_weights, self.gauss_scale, P, self.training)
+            alpha = normalised_alpha(q, query, self.position_weights(), self.gauss_scale, P, self.training)
             if P.domain == "reci":
                 a = func(alpha, P.gauss_lb_reci) * coef_reci
                 return ReciPeriodicEncodingFuncCUDA.apply(a, kr_base, rvecs, vcell, batch_q, edges), None, qs

@@ -837,6 +837,54 @@ def test_other_normalisations_and_dropout_take_the_torch_loop(dev):
     attn.params.norm_func_mode = 0
 
 
+@pytest.mark.parametrize("state", ["x", "x-xavier", "x-xn", "x-xn2"])
+def test_exponents_from_the_block_input(dev, state):
+    """gauss_state "x*": the exponents' raw value is a linear map of the block's input instead of the
+    query (models/indexed_lattice_multi_head_attention_cuda.py:855-864, 992-997).  For "x-xn" the map is
+    the product of two parameters, formed in forward.  Output against the oracle's pieces with
+    alpha = x W^T, and gradients reach every parameter."""
+    cfg, model = build_model("cfg2_default_b128", num_layers=1, value_pe_dist_real=16, adaptive_cutoff_sigma=0.0,
+                             gauss_state=state)
+    model.to(dev).train()
+    attn = model.encoder.layers[0].self_attn
+    names = dict(attn.named_parameters())
+    if state == "x-xn":
+        assert names["lattice_pos_weights"].shape == (128, 128) and names["lattice_pos_weights2"].shape == (128,)
+    else:
+        assert names["lattice_pos_weights"].shape == (8, 128) and "lattice_pos_weights2" not in names
+    W = attn.position_weights()
+    assert W.shape == (8, 128)
+    if state == "x-xn":
+        ref = torch.einsum("hk,hkd->hd", names["lattice_pos_weights2"].view(8, 16),
+                           names["lattice_pos_weights"].view(8, 16, 128))
+        assert_close(W, ref.detach().cpu(), "product of the two factors")
+    p = Problem([3, 1, 6], H=8, K=0, seed=96)
+    x = p.randn(p.N, 128).to(dev).requires_grad_(True)
+    bt, ed = p.b.batch.to(dev), p.edges.to(dev)
+    rpos, tv = p.rpos.to(dev), p.b.trans_vec.to(dev)
+    attn.eval()
+    out, _ = attn(x, x, x, bt, bt, ed, rpos, None, tv, need_weights=False)
+    P = {k: v.detach().cpu() for k, v in attn.state_dict().items()}
+    xq = x.detach().cpu()
+    q = (xq @ P["q_proj_weight"].T + P["in_proj_bias"][:128]).view(p.N, 8, 16)
+    k = (xq @ P["k_proj_weight"].T + P["in_proj_bias"][128:256]).view(p.N, 8, 16)
+    v = (xq @ P["v_proj_weight"].T + P["in_proj_bias"][256:]).view(p.N, 8, 16)
+    alpha = xq @ W.detach().cpu().T                                     # (N, H)
+    assert cfg.normalize_gauss and float(P["gauss_scale"][0]) == 0.0     # no stored statistics: those of the batch
+    an = (alpha - alpha.mean()) / alpha.std()
+    a = tp.positive_elu(an, cfg.gauss_lb_real, 0.1) * (-0.5 / 1.4 ** 2)
+    z, vpe = tp.periodic_encoding(a, p.b.pos, p.b.batch, p.b.trans_vec, p.edges, 2, 16, 14.0, 1.0, P["pe_dist_proj"])
+    o, _ = tp.indexed_attention(q, k, v, p.b.sizes, p.edges, z, vpe)
+    ref_out = o.reshape(p.N, 128) @ P["out_proj.weight"].T + P["out_proj.bias"]
+    assert_close(out, ref_out, f"attention output, gauss_state {state}", rtol=2e-5)
+    attn.train()
+    out, _ = attn(x, x, x, bt, bt, ed, rpos, None, tv, need_weights=False)
+    out.square().sum().backward()
+    for name, prm in attn.named_parameters():
+        if "scale" not in name:
+            assert prm.grad is not None and float(prm.grad.abs().max()) > 0, name
+
+
 def test_blocks_share_one_staging_of_the_translations(dev):
     """Fixed cube, value bins, shared projection: the translations of every atom pair are staged once per
     forward pass and all blocks (and their backward passes) start from them.  Same outputs and gradients as
