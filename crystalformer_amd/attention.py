@@ -11,6 +11,7 @@ torch / rocBLAS.
 from __future__ import annotations
 
 import math
+import warnings
 from typing import Optional, Tuple
 
 import torch
@@ -216,9 +217,16 @@ class CrystalformerMultiheadAttentionCUDA(Module):
             (params.value_pe_dist_reci if params.domain in ("reci", "RECI") else 0)
         if bins > 0:
             self.pe_dist_proj = Parameter(torch.empty(cond, heads, self.head_dim, bins, **kw))
-        if (params.domain in ("real", "multihead") and params.value_pe_wave_real > 0) or \
-                (params.domain in ("reci", "RECI") and params.value_pe_wave_reci > 0):
-            raise NotImplementedError("value_pe_wave_* > 0 has no HIP kernel")
+        waves = params.value_pe_wave_real if params.domain in ("real", "multihead") else \
+            (params.value_pe_wave_reci if params.domain in ("reci", "RECI") else 0)
+        if waves > 0:
+            # As on the reference's kernel path (models/indexed_lattice_multi_head_attention_cuda.py:872-878,
+            # 600-614, 938-947): the parameter exists, is initialised in the same order and travels in the
+            # state_dict, and nothing computes a value encoding from it (only the reference's PyTorch path
+            # evaluates the plane-wave encodings).
+            self.pe_wave_proj = Parameter(torch.empty(cond, heads, self.head_dim, waves ** 3, **kw))
+            warnings.warn("value_pe_wave_* > 0: pe_wave_proj is kept for state_dict compatibility and has no effect "
+                          "on the output, as on the reference's kernel path", stacklevel=2)
         self._reset_parameters()
 
     def position_weights(self) -> Optional[Tensor]:
@@ -270,6 +278,14 @@ class CrystalformerMultiheadAttentionCUDA(Module):
                 for idx, W in enumerate(self.pe_dist_proj):
                     if idx != 0 and self.params.value_pe_condproj in ("I", "J", "IJ"):
                         W.set_(self.pe_dist_proj[0])
+                    else:
+                        flat = W.view(-1, W.shape[-1])
+                        xavier_uniform_(flat, flat.shape[1] ** -0.5)
+        if self.pe_wave_proj is not None:
+            with torch.no_grad():
+                for idx, W in enumerate(self.pe_wave_proj):
+                    if idx != 0 and self.params.value_pe_condproj in ("I", "J", "IJ"):
+                        W.set_(self.pe_wave_proj[0])
                     else:
                         flat = W.view(-1, W.shape[-1])
                         xavier_uniform_(flat, flat.shape[1] ** -0.5)

@@ -91,6 +91,43 @@ def test_default_model_initialisation_digests():
         assert hashlib.sha256(v.detach().contiguous().numpy().tobytes()).hexdigest() == ref[k]["sha256"], k
 
 
+def test_optional_parameters_of_the_attention_module():
+    """Options off the default path that add parameters, as the reference's kernel-path module lays them
+    out (models/indexed_lattice_multi_head_attention_cuda.py:855-878, 894-947): the plane-wave projection
+    is created and initialised after the distance projection (it has no effect on that module's output,
+    and none here), gauss_state "x-xn" has two factors.  Parameters drawn before the new ones keep the
+    values of the default model (same random stream up to there), and the golden initialisation of
+    the default configuration is untouched."""
+    import warnings
+    from crystalformer_amd.latticeformer import Latticeformer
+    torch.manual_seed(7)
+    base = Latticeformer(small_cfg()).state_dict()
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        torch.manual_seed(7)
+        waves = Latticeformer(small_cfg(value_pe_wave_real=2)).state_dict()
+    assert any("pe_wave_proj" in str(w.message) for w in caught)
+    key = "encoder.layers.0.self_attn.pe_wave_proj"
+    dist = "encoder.layers.0.self_attn.pe_dist_proj"
+    assert waves[key].shape == (1, base[dist].shape[1], base[dist].shape[2], 8)
+    assert float(waves[key].abs().max()) > 0
+    keys = list(waves.keys())
+    assert keys.index(key) == keys.index(dist) + 1
+    for k in ("input_embeddings.weight", "encoder.layers.0.self_attn.q_proj_weight", dist,
+              "encoder.layers.0.self_attn.lattice_pos_weights"):
+        assert torch.equal(waves[k], base[k]), k
+    torch.manual_seed(7)
+    two = Latticeformer(small_cfg(gauss_state="x-xn"))
+    attn = two.encoder.layers[0].self_attn
+    H, D = attn.num_heads, attn.embed_dim
+    assert attn.lattice_pos_weights.shape == (attn.kdim, D) and attn.lattice_pos_weights2.shape == (attn.kdim,)
+    assert attn.position_weights().shape == (H, D)
+    torch.manual_seed(7)
+    one = Latticeformer(small_cfg(gauss_state="x-xn2")).encoder.layers[0].self_attn
+    # "x-xn2" is the product of the same two factors, drawn once at initialisation
+    assert torch.equal(one.lattice_pos_weights, attn.position_weights())
+
+
 # ------------------------------------------------- reciprocal-space blocks
 RECI_CASES = [("real_reci_k16_r1", dict(domain="real-reci"), 13),
               ("multihead_k0_r2", dict(domain="multihead", value_pe_dist_real=0, lattice_range=2), 14),
