@@ -204,7 +204,8 @@ __global__ __launch_bounds__(256, (PREFETCH ? 6 : 7)) void fused_dpa_fwd_stream_
     float4_v k4[4], v4[4], b4[4];
     float av[4];
     auto fetch = [&](int u, uint32_t e, uint32_t j) {
-        if (HAS_B) b4[u] = ld4_stream(p.bij, (e * HD4 + piece) * 16u);   // independent of the key index: first
+        // (independent of the key index: first; long rows: a stream that is read once)
+        if (HAS_B) b4[u] = PREFETCH ? ld4_stream(p.bij, (e * HD4 + piece) * 16u) : ld4(p.bij, (e * HD4 + piece) * 16u);
         if (HAS_A) av[u] = ld1(p.aij, (e * H + h) * 4u);
         k4[u] = ld4(p.key, (j * HD4 + piece) * 16u);
         v4[u] = ld4(p.val, (j * HD4 + piece) * 16u);
@@ -334,7 +335,8 @@ __device__ __forceinline__ void st4_stream(void *base, uint32_t byte_off, float4
     __builtin_nontemporal_store(v, reinterpret_cast<float4_v *>(static_cast<char *>(base) + byte_off));
 }
 
-template <int DV4, bool HAS_B, bool WANT_GB>
+// STREAM (long rows): b_ij is read and gb_ij written with the streaming hint.
+template <int DV4, bool HAS_B, bool WANT_GB, bool STREAM>
 __global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs p, int LPE)
 {
     __shared__ float part[DPA_WPQ][WAVE][4];
@@ -372,7 +374,7 @@ __global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             pr[u] = ld1(p.prob_in, (ec[u] * H + h) * 4u);
-            if (HAS_B) b4[u] = ld4_stream(p.bij, (ec[u] * HD4 + piece) * 16u);
+            if (HAS_B) b4[u] = STREAM ? ld4_stream(p.bij, (ec[u] * HD4 + piece) * 16u) : ld4(p.bij, (ec[u] * HD4 + piece) * 16u);
             m4[u] = ld4(p.val, (j[u] * HD4 + piece) * 16u);
         }
 #pragma unroll
@@ -385,7 +387,10 @@ __global__ __launch_bounds__(256) void fused_dpa_bwd_query_stream_kernel(DpaArgs
             float gs = d4.x * t4.x + d4.y * t4.y + d4.z * t4.z + d4.w * t4.w;
             gs = head_sum<DV4>(gs);
             if (valid) {
-                if (WANT_GB) st4_stream(p.gbij, (ec[u] * HD4 + piece) * 16u, t4);
+                if (WANT_GB) {
+                    if (STREAM) st4_stream(p.gbij, (ec[u] * HD4 + piece) * 16u, t4);
+                    else st4(p.gbij, (ec[u] * HD4 + piece) * 16u, t4);
+                }
                 if (lead) st1(p.gaij, (ec[u] * H + h) * 4u, gs);
             }
             gsv[u] = valid ? gs : 0.f;
@@ -616,14 +621,24 @@ void launch_fwd_stream(const DpaArgs &p, int dv4, int lpe, hipStream_t st)
 #undef CF_DPA_FWD
 }
 
+template <int DV4, bool STREAM>
+void launch_bwd_query_dv(const DpaArgs &p, int lpe, hipStream_t st)
+{
+    const dim3 grid((unsigned)p.N), block(DPA_WPQ * WAVE);
+    if (p.bij && p.gbij) fused_dpa_bwd_query_stream_kernel<DV4, true, true, STREAM><<<grid, block, 0, st>>>(p, lpe);
+    else if (p.bij) fused_dpa_bwd_query_stream_kernel<DV4, true, false, STREAM><<<grid, block, 0, st>>>(p, lpe);
+    else if (p.gbij) fused_dpa_bwd_query_stream_kernel<DV4, false, true, STREAM><<<grid, block, 0, st>>>(p, lpe);
+    else fused_dpa_bwd_query_stream_kernel<DV4, false, false, STREAM><<<grid, block, 0, st>>>(p, lpe);
+}
+
 template <int DV4>
 void launch_bwd_stream_dv(const DpaArgs &p, int lpe, hipStream_t st)
 {
     const dim3 grid((unsigned)p.N), block(DPA_WPQ * WAVE);
-    if (p.bij && p.gbij) fused_dpa_bwd_query_stream_kernel<DV4, true, true><<<grid, block, 0, st>>>(p, lpe);
-    else if (p.bij) fused_dpa_bwd_query_stream_kernel<DV4, true, false><<<grid, block, 0, st>>>(p, lpe);
-    else if (p.gbij) fused_dpa_bwd_query_stream_kernel<DV4, false, true><<<grid, block, 0, st>>>(p, lpe);
-    else fused_dpa_bwd_query_stream_kernel<DV4, false, false><<<grid, block, 0, st>>>(p, lpe);
+    // (the forward's rule for long rows: more than two steps of a work-group on average)
+    const int64_t step_edges = 4 * DPA_WPQ * (WAVE / lpe);
+    if (p.E > 2 * step_edges * p.N) launch_bwd_query_dv<DV4, true>(p, lpe, st);
+    else launch_bwd_query_dv<DV4, false>(p, lpe, st);
     fused_dpa_bwd_key_stream_kernel<DV4><<<grid, block, 0, st>>>(p, lpe);
 }
 
