@@ -58,10 +58,16 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 #pragma unroll
     for (int m = 0; m < NT; m++) ck[m] = p.bin_step * (float)(16 * m + c + 1);
 
-    // this wave's head: the running block of gW lives in LDS between rounds (one 16-byte slot per
-    // lane and tile, touched by its own lane only), the projection operands are fetched per round
-    // just before they are used: 32 registers less across the accumulation
+    // this wave's head: the projection operands are fetched per round just before they are used.
+    // The running block of gW: staging for itself, the kernel has no registers to spare and keeps it
+    // in LDS between rounds (one 16-byte slot per lane and tile, touched by its own lane only); from
+    // staged rings it stays in registers, and the LDS it would take holds a second exchange buffer
+    // (S next to Q': one exchange and two barriers per round instead of two and four).
     float4_t *gw_slot = reinterpret_cast<float4_t *>(PXbuf + WPB * 16) + (wave * NT) * WAVE + lane;
+    float *Sbuf2 = PXbuf + WPB * 16;                                    // (RINGS only; same place)
+    float4_t gWreg[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) gWreg[t] = float4_t{0.f, 0.f, 0.f, 0.f};
     int wa_hg = -1;
 
     const int rounds_per_hg = (int)((p.U + WPB - 1) / WPB);
@@ -104,7 +110,7 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int d = 4 * qq + r, k = 16 * t + cc;
-                    if (d < D && k < K) dst[(unsigned)(d * K + k)] = gw_slot[t * WAVE][r];
+                    if (d < D && k < K) dst[(unsigned)(d * K + k)] = RINGS ? gWreg[t][r] : gw_slot[t * WAVE][r];
                 }
         }
     };
@@ -182,7 +188,10 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         if (hg != wa_hg) {
             if (wa_hg >= 0) flush_gW(wa_hg);
 #pragma unroll
-            for (int t = 0; t < NT; t++) gw_slot[t * WAVE] = float4_t{0.f, 0.f, 0.f, 0.f};
+            for (int t = 0; t < NT; t++) {
+                if (RINGS) gWreg[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+                else gw_slot[t * WAVE] = float4_t{0.f, 0.f, 0.f, 0.f};
+            }
             wa_hg = hg;
         }
         const int64_t e_ij = ids.e_ij, e_ji = ids.e_ji;
@@ -447,22 +456,22 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
         for (int m = 0; m < NT; m++)
 #pragma unroll
             for (int r = 0; r < 4; r++) accQ[m][r] = fmaf(-px, accS[m][r], accQ[m][r]);
-        const int passes = p.gW_part ? 2 : 1;
-        for (int pass = 0; pass < passes; pass++) {
-            // pass 0 exchanges Q' (projection, dot with gv, ga), pass 1 exchanges S (gW update):
-            // Q' first, so that its accumulators are dead before the gW block comes in from LDS
+        if constexpr (RINGS) {
+            // ---- one exchange: Q' and (for the weight gradient) S parked side by side
+            const bool want_gW = p.gW_part != nullptr && g_gv != nullptr;
             {
-                float *col = Sbuf + xch_base(q, c & 7, wave, c >> 3);
+                const int at = xch_base(q, c & 7, wave, c >> 3);
 #pragma unroll
                 for (int m = 0; m < NT; m++)
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
                         // (inactive columns hold zeros: their weights are masked in the loop)
-                        col[(4 * m + r) * XPLANE] = pass == 0 ? accQ[m][r] : accS[m][r];
+                        Sbuf[at + (4 * m + r) * XPLANE] = accQ[m][r];
+                        if (want_gW) Sbuf2[at + (4 * m + r) * XPLANE] = accS[m][r];
                     }
             }
             __syncthreads();
-            if (pass == 0) {
+            {
                 float4_t out = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int t4 = 0; t4 < NT; t4++) {
@@ -480,36 +489,94 @@ __global__ __launch_bounds__(512, 4) void real_enc_bwd_pair_kernel(PairArgs p)
                     const float PX = PXbuf[(c_r & 7) * 16 + (c_r >> 3) * 8 + wave];      // (unit_j, dir_j)
                     p.ga_edge[row_out] = fmaf(PX, gz_out, dot);
                 }
-                // operands of the gW update of the next pass, requested now so that they arrive
-                // while S is being exchanged
-                if (hw < H && p.gW_part && g_gv) {
+            }
+            if (want_gW) {
+                // This head's gradient rows once more, transposed: lane (q, j) holds gv[column j][4q .. 4q + 3],
+                // the update wants gv[column 4 s4 + q][c].  Through the wavefront's own ring, whose records
+                // have been used (16 rows of 17 floats): no second fetch from memory.
+                float *T = ring_d2;
 #pragma unroll
-                    for (int s4 = 0; s4 < 4; s4++) {
-                        const int e_k = __builtin_amdgcn_ds_bpermute((4 * s4 + q) << 2, col_edge);   // column 4*s4 + q
-                        const unsigned row_k = (unsigned)e_k * (unsigned)H + (unsigned)hw;
-                        if (e_k >= 0 && c < D) gvk[s4] = g_gv[(uint64_t)row_k * (unsigned)D + (unsigned)c_r];
-                    }
-                }
-            } else {
+                for (int r = 0; r < 4; r++) T[c * 17 + 4 * q + r] = gv4[r];
+                wave_mem_sync();
                 // gW_h[d][bin] += sum over the 16 columns of gv[col][d] * S[bin][col]
                 // A[i = d][k = col], B[k = col][j = bin]; column 4*s4 + kk
-                float4_t gWacc[NT];
-#pragma unroll
-                for (int t = 0; t < NT; t++) gWacc[t] = gw_slot[t * WAVE];
 #pragma unroll
                 for (int s4 = 0; s4 < 4; s4++) {
                     const int colk = 4 * s4 + q;                    // this lane's reduction index
-                    const float av = gvk[s4];
+                    const float av = T[colk * 17 + c];
                     // bin 16 t + c of column colk: plane 4 t + c % 4, q index c / 4
-                    const float *srck = Sbuf + (c & 3) * XPLANE + xch_base(c >> 2, wave, colk & 7, colk >> 3);
+                    const float *srck = Sbuf2 + (c & 3) * XPLANE + xch_base(c >> 2, wave, colk & 7, colk >> 3);
 #pragma unroll
                     for (int t = 0; t < NT; t++)
-                        gWacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, srck[4 * t * XPLANE], gWacc[t], 0, 0, 0);
+                        gWreg[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, srck[4 * t * XPLANE], gWreg[t], 0, 0, 0);
                 }
-#pragma unroll
-                for (int t = 0; t < NT; t++) gw_slot[t * WAVE] = gWacc[t];
             }
             __syncthreads();
+        } else {
+        const int passes = p.gW_part ? 2 : 1;
+            for (int pass = 0; pass < passes; pass++) {
+                // pass 0 exchanges Q' (projection, dot with gv, ga), pass 1 exchanges S (gW update):
+                // Q' first, so that its accumulators are dead before the gW block comes in from LDS
+                {
+                    float *col = Sbuf + xch_base(q, c & 7, wave, c >> 3);
+    #pragma unroll
+                    for (int m = 0; m < NT; m++)
+    #pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            // (inactive columns hold zeros: their weights are masked in the loop)
+                            col[(4 * m + r) * XPLANE] = pass == 0 ? accQ[m][r] : accS[m][r];
+                        }
+                }
+                __syncthreads();
+                if (pass == 0) {
+                    float4_t out = {0.f, 0.f, 0.f, 0.f};
+    #pragma unroll
+                    for (int t4 = 0; t4 < NT; t4++) {
+                        float sb[4];
+    #pragma unroll
+                        for (int r = 0; r < 4; r++) sb[r] = src[(4 * t4 + r) * XPLANE];
+    #pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            out = __builtin_amdgcn_mfma_f32_16x16x4f32(Wa[4 * t4 + r], sb[r], out, 0, 0, 0);
+                    }
+                    // lane (q, j): components d = 4q + r of W Q' for column j; dot with gv
+                    float dot = out[0] * gv4[0] + out[1] * gv4[1] + out[2] * gv4[2] + out[3] * gv4[3];
+                    dot = rows_sum(dot);
+                    if (q == 0 && e_out >= 0 && hw < H) {
+                        const float PX = PXbuf[(c_r & 7) * 16 + (c_r >> 3) * 8 + wave];      // (unit_j, dir_j)
+                        p.ga_edge[row_out] = fmaf(PX, gz_out, dot);
+                    }
+                    // operands of the gW update of the next pass, requested now so that they arrive
+                    // while S is being exchanged
+                    if (hw < H && p.gW_part && g_gv) {
+    #pragma unroll
+                        for (int s4 = 0; s4 < 4; s4++) {
+                            const int e_k = __builtin_amdgcn_ds_bpermute((4 * s4 + q) << 2, col_edge);   // column 4*s4 + q
+                            const unsigned row_k = (unsigned)e_k * (unsigned)H + (unsigned)hw;
+                            if (e_k >= 0 && c < D) gvk[s4] = g_gv[(uint64_t)row_k * (unsigned)D + (unsigned)c_r];
+                        }
+                    }
+                } else {
+                    // gW_h[d][bin] += sum over the 16 columns of gv[col][d] * S[bin][col]
+                    // A[i = d][k = col], B[k = col][j = bin]; column 4*s4 + kk
+                    float4_t gWacc[NT];
+    #pragma unroll
+                    for (int t = 0; t < NT; t++) gWacc[t] = gw_slot[t * WAVE];
+    #pragma unroll
+                    for (int s4 = 0; s4 < 4; s4++) {
+                        const int colk = 4 * s4 + q;                    // this lane's reduction index
+                        const float av = gvk[s4];
+                        // bin 16 t + c of column colk: plane 4 t + c % 4, q index c / 4
+                        const float *srck = Sbuf + (c & 3) * XPLANE + xch_base(c >> 2, wave, colk & 7, colk >> 3);
+    #pragma unroll
+                        for (int t = 0; t < NT; t++)
+                            gWacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, srck[4 * t * XPLANE], gWacc[t], 0, 0, 0);
+                    }
+    #pragma unroll
+                    for (int t = 0; t < NT; t++) gw_slot[t * WAVE] = gWacc[t];
+                }
+                __syncthreads();
+            }
         }
         ids = ids_next;
         geo = geo_next;
@@ -623,8 +690,10 @@ int launch_real_enc_bwd_pairs(const float *a_ik, const float *rpos, const float 
     const int side = 2 * lattice_range + 1;
     if (rings && (!uniform || side * side * side > RIMG_CAP)) rings = nullptr;     // not what rings are staged for
     p.rings = rings;
-    const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + (size_t)4 * NT * XPLANE + WPB * 16 +
-                                        (size_t)WPB * NT * WAVE * 4) + 16;
+    // rings, exchange buffer, PX, and either the gW slots or (from staged rings) a second exchange buffer
+    const size_t gw_words = (size_t)WPB * NT * WAVE * 4, xch_words = (size_t)4 * NT * XPLANE;
+    const size_t lds = sizeof(float) * ((size_t)WPB * 3 * BRING_SLOTS + xch_words + WPB * 16 +
+                                        (rings ? xch_words : gw_words)) + 16;
     if (((U + WPB - 1) / WPB) * ((H + 7) / 8) >= (1ll << 30)) return CF_ERR_UNSUPPORTED;   // 32-bit round positions
     if (E >= (1ll << 31) || E * H >= (1ll << 32) || N * H >= (1ll << 32)) return CF_ERR_UNSUPPORTED;   // 32-bit ids, rows
     const int blocks = real_enc_bwd_pairs_blocks(U, H);
