@@ -10,12 +10,13 @@
 // Gaussians are evaluated once per translation for 2 x 16 weight columns
 // (8 heads of i and of j, each with p and p*d2), S and Q accumulate on
 // v_mfma_f32_16x16x4_f32.  A work-group is 8 wavefronts; per round every
-// wavefront owns one unit, then the 8 wavefronts exchange S and Q through LDS
-// and wavefront w does head w for all 8 units: W S and W Q (the forward's
-// projection, twice), the two dot products with gv, and the rank-16 update of
-// that head's D x K block of gW, which stays in registers for the whole kernel
-// and is written once per work-group; a second kernel adds the per-work-group
-// blocks in a fixed order.  No atomics.
+// wavefront owns one unit, then the 8 wavefronts exchange Q' = Q - PX S (and S,
+// when the weight gradient is wanted) through LDS and wavefront w does head w
+// for all 8 units: W Q' (the forward's projection), its dot product with gv,
+// and the rank-16 update of that head's D x K block of gW, which is kept for the
+// whole kernel (in registers from staged rings, otherwise in LDS slots of its
+// own) and written once per work-group; a second kernel adds the
+// per-work-group blocks in a fixed order.  No atomics.
 #include <type_traits>
 #include "real_enc_pair.h"
 
