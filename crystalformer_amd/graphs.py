@@ -76,6 +76,25 @@ class GraphedForward:
             B, N, E = (int(c) for c in capacity)
             if B < 1 or N < B or E < N:
                 raise ValueError("capacity is (crystals, atoms, edges) with crystals <= atoms <= edges")
+            # Inside the graph the tail of every per-atom / per-edge tensor is unwritten memory: only
+            # operators that read the live counts may see them.  The real-space blocks with one
+            # projection do; reciprocal-space blocks, species-conditioned projections and the
+            # per-crystal torch loop index with whole edge lists, and exponents worked out by torch
+            # expressions take their statistics over whole tensors: refused here.
+            for m in model.modules():
+                P = getattr(m, "params", None)
+                if P is None or not hasattr(m, "pe_dist_proj"):
+                    continue
+                from .attention import fused_exponents_spec
+                if (P.domain != "real" or P.value_pe_condproj != "no" or P.norm_func_mode != 0
+                        or fused_exponents_spec(P) is None):
+                    raise ValueError("GraphedForward(capacity=...) serves real-space attention blocks with one "
+                                     "projection, the plain softmax and exponents from the query through the "
+                                     "exponent kernel (domain 'real', value_pe_condproj 'no', norm_func_mode 0, "
+                                     f"gauss_state 'q*', positive_func elu/abs/exp); got domain {P.domain!r}, "
+                                     f"value_pe_condproj {P.value_pe_condproj!r}, norm_func_mode "
+                                     f"{P.norm_func_mode}, gauss_state {P.gauss_state!r}, positive_func "
+                                     f"{P.positive_func!r}")
             E += (N + E) % 2                    # (atoms + edges is even for any batch)
             self.capacity = (B, N, E)
             dev = batch.pos.device

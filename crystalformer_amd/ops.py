@@ -921,6 +921,9 @@ def gauss_exponents(q_ihd: Tensor, w_hd: Tensor, gauss_scale: Optional[Tensor], 
 def kr_base(rpos_ij_e: Tensor, rvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor) -> Tensor:
     """(E,3) phases <b_d, p_j - p_i> of the reciprocal-space encoding
     (models/indexed_latticeformer_encoder.py:245-251)."""
+    if current_live_sizes() is not None:
+        raise _lib.CrystalformerHipError("reciprocal-space operators do not run under a size header "
+                                         "(they walk whole edge lists)")
     dev = require_device(rpos_ij_e, rvecs_n, batch_i, edge_ij_e)
     rpos_ij_e, rvecs_n = _f32(rpos_ij_e, "rpos_ij_e"), _f32(rvecs_n, "rvecs_n")
     batch_i, edge_ij_e = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e")
@@ -948,6 +951,9 @@ def _reci_operands(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i):
 def reci_enc_fwd(a_ik: Tensor, kr_base_e: Tensor, rvecs_n: Tensor, vcell_n: Tensor, batch_i: Tensor,
                  e_start_i: Tensor, lattice_range: int) -> Tuple[Tensor, Tensor]:
     """``(z_ek, sumexp_ek)`` of the reciprocal-space lattice sum."""
+    if current_live_sizes() is not None:
+        raise _lib.CrystalformerHipError("reciprocal-space operators do not run under a size header "
+                                         "(they walk whole edge lists)")
     dev = require_device(a_ik, kr_base_e, rvecs_n, vcell_n, batch_i, e_start_i)
     a_ik, kr_base_e, rvecs_n, batch_i, e_start_i = _reci_operands(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i)
     vcell_n = _f32(vcell_n, "vcell_n")

@@ -509,6 +509,31 @@ def test_one_graph_serves_batches_of_any_size(dev, rule):
         small(batches[1])                                                # atoms beyond the capacity: seen on the host
 
 
+def test_capacity_graph_refuses_models_it_cannot_serve(dev):
+    """With capacity buffers the tails of the per-atom and per-edge tensors are unwritten memory, so
+    only configurations whose operators all read the live counts are accepted: reciprocal-space
+    blocks, species-conditioned projections, other normalisations and exponents from torch
+    expressions are refused when the graph is built, and the reciprocal-space operators refuse a
+    size header themselves."""
+    from crystalformer_amd import lib
+    from crystalformer_amd.graphs import GraphedForward
+    from crystalformer_amd.synthetic import make_batch
+    b = make_batch(4, (2, 9), True, (3.0, 15.0), (60.0, 120.0), seed=31).to(dev)
+    for over in (dict(domain="real-reci"), dict(value_pe_condproj="i"), dict(norm_func_mode=3),
+                 dict(gauss_state="x")):
+        cfg, model = build_model("cfg2_default_b128", num_layers=2, adaptive_cutoff_sigma=0.0, **over)
+        model.to(dev).eval()
+        with pytest.raises(ValueError, match="capacity"):
+            GraphedForward(model, b, capacity=(8, 64, 2048))
+    header = torch.zeros(4, dtype=torch.int64, device=dev)
+    E = 100
+    with ops.live_sizes(header, 20, E):
+        with pytest.raises(lib.CrystalformerHipError, match="size header"):
+            ops.kr_base(torch.zeros(E, 3, device=dev), torch.zeros(2, 3, 3, device=dev),
+                        torch.zeros(20, dtype=torch.int64, device=dev), torch.zeros(2, E, dtype=torch.int64, device=dev))
+    assert ops.current_live_sizes() is None and lib_header_is_clear()
+
+
 def lib_header_is_clear():
     from crystalformer_amd import lib
     return not lib.load().cf_get_size_header()
