@@ -107,6 +107,14 @@ def current_live_sizes() -> Optional[live_sizes]:
     return getattr(_live, "current", None)
 
 
+def _refuse_live_sizes(what: str) -> None:
+    """Operators whose kernels take their counts from the arguments walk whole tensors: under a size
+    header the tails of those tensors are unwritten memory, so they refuse to run there."""
+    if current_live_sizes() is not None:
+        raise _lib.CrystalformerHipError(f"{what} does not run under a size header (it walks whole tensors); "
+                                         f"leave the live_sizes context first")
+
+
 class _timed:
     def __init__(self, name: str, **info):
         self.name, self.info = name, info
@@ -373,6 +381,7 @@ def real_enc_bwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tens
                  rings: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
     """``rings`` from :func:`staged_rings` (same geometry, pair list, bin grid and cube): the pair
     kernel starts from the staged translations instead of working them out again."""
+    _refuse_live_sizes("real_enc_bwd")
     dev = require_device(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, e_start_i, z_ek, gz_ek, gv_ekd,
                          W_k, rvlen_n, pairs_u, rings)
     pairs_u = _i64(pairs_u, "pairs_u")
@@ -473,6 +482,7 @@ def fused_enc_dpa_fwd(a_ik: Tensor, rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i:
 
 def translation_ranges(a_ik: Tensor, rvlen_n: Optional[Tensor], batch_i: Tensor,
                        cutoff_radius: float, lattice_range: int, minimum_range: int) -> Tensor:
+    _refuse_live_sizes("translation_ranges")
     dev = require_device(a_ik, rvlen_n, batch_i)
     a_ik, rvlen_n, batch_i = _f32(a_ik, "a_ik"), _f32(rvlen_n, "rvlen_n"), _i64(batch_i, "batch_i")
     N, H = a_ik.shape
@@ -518,6 +528,7 @@ def fused_dpa_fwd(que: Tensor, key: Tensor, val: Tensor, aij_eh: Optional[Tensor
 def fused_dpa_bwd(que: Tensor, key: Tensor, val: Tensor, bij_ehd: Optional[Tensor], batch_i: Tensor,
                   edge_ij_e: Tensor, e_start_i: Tensor, prob_eh: Tensor, out: Tensor, gout: Tensor,
                   atom_start_n: Optional[Tensor] = None, edge_start_n: Optional[Tensor] = None):
+    _refuse_live_sizes("fused_dpa_bwd")
     dev = require_device(que, key, val, bij_ehd, batch_i, edge_ij_e, e_start_i, prob_eh, out, gout)
     que, key, val, bij_ehd = _f32(que, "que"), _f32(key, "key"), _f32(val, "val"), _f32(bij_ehd, "bij_ehd")
     prob_eh, out, gout = _f32(prob_eh, "prob_eh"), _f32(out, "out"), _f32(gout, "gout")
@@ -561,6 +572,7 @@ def irregular_mean_fwd(x_ik: Tensor, start_n: Tensor) -> Tensor:
 
 
 def irregular_mean_bwd(go_nk: Tensor, batch_i: Tensor, start_n: Tensor) -> Tensor:
+    _refuse_live_sizes("irregular_mean_bwd")
     dev = require_device(go_nk, batch_i, start_n)
     go_nk, batch_i, start_n = _f32(go_nk, "go_nk"), _i64(batch_i, "batch_i"), _i64(start_n, "start_n")
     N = batch_i.numel()
@@ -576,6 +588,7 @@ def irregular_mean_bwd(go_nk: Tensor, batch_i: Tensor, start_n: Tensor) -> Tenso
 def minimum_distance(rpos_ij_e: Tensor, tvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor,
                      rvlen_n: Optional[Tensor], cutoff_radius: float, lattice_range: int = 2,
                      minimum_range: int = 0) -> Tensor:
+    _refuse_live_sizes("minimum_distance")
     dev = require_device(rpos_ij_e, tvecs_n, batch_i, edge_ij_e, rvlen_n)
     rpos_ij_e, tvecs_n, rvlen_n = _f32(rpos_ij_e, "rpos_ij_e"), _f32(tvecs_n, "tvecs_n"), \
         _f32(rvlen_n, "rvlen_n")
@@ -921,9 +934,7 @@ def gauss_exponents(q_ihd: Tensor, w_hd: Tensor, gauss_scale: Optional[Tensor], 
 def kr_base(rpos_ij_e: Tensor, rvecs_n: Tensor, batch_i: Tensor, edge_ij_e: Tensor) -> Tensor:
     """(E,3) phases <b_d, p_j - p_i> of the reciprocal-space encoding
     (models/indexed_latticeformer_encoder.py:245-251)."""
-    if current_live_sizes() is not None:
-        raise _lib.CrystalformerHipError("reciprocal-space operators do not run under a size header "
-                                         "(they walk whole edge lists)")
+    _refuse_live_sizes("the reciprocal-space encoding")
     dev = require_device(rpos_ij_e, rvecs_n, batch_i, edge_ij_e)
     rpos_ij_e, rvecs_n = _f32(rpos_ij_e, "rpos_ij_e"), _f32(rvecs_n, "rvecs_n")
     batch_i, edge_ij_e = _i64(batch_i, "batch_i"), _i64(edge_ij_e, "edge_ij_e")
@@ -951,9 +962,7 @@ def _reci_operands(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i):
 def reci_enc_fwd(a_ik: Tensor, kr_base_e: Tensor, rvecs_n: Tensor, vcell_n: Tensor, batch_i: Tensor,
                  e_start_i: Tensor, lattice_range: int) -> Tuple[Tensor, Tensor]:
     """``(z_ek, sumexp_ek)`` of the reciprocal-space lattice sum."""
-    if current_live_sizes() is not None:
-        raise _lib.CrystalformerHipError("reciprocal-space operators do not run under a size header "
-                                         "(they walk whole edge lists)")
+    _refuse_live_sizes("the reciprocal-space encoding")
     dev = require_device(a_ik, kr_base_e, rvecs_n, vcell_n, batch_i, e_start_i)
     a_ik, kr_base_e, rvecs_n, batch_i, e_start_i = _reci_operands(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i)
     vcell_n = _f32(vcell_n, "vcell_n")
@@ -976,6 +985,7 @@ def reci_enc_bwd(a_ik: Tensor, kr_base_e: Tensor, rvecs_n: Tensor, batch_i: Tens
     """``ga_ik`` of the reciprocal-space lattice sum: by default the reference kernel's
     definition, which leaves the normalisation term's derivative out; with
     ``normalisation_grad`` the full derivative of z."""
+    _refuse_live_sizes("reci_enc_bwd")
     dev = require_device(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i, gz_ek, sumexp_ek)
     a_ik, kr_base_e, rvecs_n, batch_i, e_start_i = _reci_operands(a_ik, kr_base_e, rvecs_n, batch_i, e_start_i)
     gz_ek, sumexp_ek = _f32(gz_ek, "gz_ek"), _f32(sumexp_ek, "sumexp_ek")
