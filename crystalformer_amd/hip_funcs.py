@@ -29,7 +29,7 @@ from . import lib as _lib
 from . import ops
 
 __all__ = [
-    "KernelManager", "compile_kernels", "CUPY_AVAILABLE", "HIP_AVAILABLE",
+    "KernelManager", "Kernel", "compile_kernels", "CUPY_AVAILABLE", "HIP_AVAILABLE",
     "RealPeriodicEncodingFuncCUDA", "RealPeriodicEncodingWithProjFuncCUDA",
     "FusedDotProductAttentionCUDA", "IrregularMeanCUDA", "compute_minimum_distance",
     "ReciPeriodicEncodingFuncCUDA", "fused_encoding_attention",
@@ -43,6 +43,26 @@ def _hip_available() -> bool:
 HIP_AVAILABLE = _hip_available()
 # The reference gates its kernel path on this flag (models/latticeformer.py:139-143).
 CUPY_AVAILABLE = HIP_AVAILABLE
+
+
+class Kernel:
+    """A named entry point of the HIP library: the counterpart of the reference's holder of one
+    compiled CuPy kernel (models/cuda_funcs/kernel_manager.py:15-22).  ``Kernel(name)(grid, block,
+    args)`` keeps the reference's call shape; the launch geometry is the library's own business, so
+    ``grid`` and ``block`` are ignored and ``args`` (raw pointers, sizes, stream handle) go to the C
+    function, whose status code is returned.  ``Kernel(name)(*args)`` does the same."""
+
+    def __init__(self, name: str):
+        self.name = name
+        self.code = None            # (no source text: the library is built ahead of time)
+        self.raw_kernel = None
+
+    def __call__(self, *call_args, **_ignored):
+        if self.raw_kernel is None:
+            self.raw_kernel = getattr(_lib.load(), self.name)
+        if len(call_args) == 3 and isinstance(call_args[2], (tuple, list)):
+            call_args = tuple(call_args[2])
+        return self.raw_kernel(*call_args)
 
 
 class KernelManager:

@@ -296,3 +296,15 @@ def test_graph_replay_refuses_other_crystal_sizes():
     with pytest.raises(ValueError, match="layout differs"):
         _same_layout(owner, CrystalBatch(torch.zeros(5, 98), torch.zeros(5, 3), torch.zeros(5, dtype=torch.long),
                                          torch.zeros(2, 3, 3), torch.tensor([2, 3])))
+
+
+def test_kernel_holder_resolves_library_entry_points():
+    """``Kernel`` (exported like the reference's, models/cuda_funcs/__init__.py:12-27) names an entry
+    point of the C library; both call shapes reach it, unknown names fail at the first call."""
+    from crystalformer_amd import hip_funcs
+    assert "Kernel" in hip_funcs.__all__
+    k = hip_funcs.Kernel("cf_version")
+    assert k.name == "cf_version" and k.code is None
+    assert k() == k((1,), (64,), ()) == lib.load().cf_version()
+    with pytest.raises(AttributeError):
+        hip_funcs.Kernel("cf_no_such_entry_point")()
