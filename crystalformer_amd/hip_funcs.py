@@ -110,6 +110,37 @@ class KernelManager:
     ADAPTIVE_RINGS = True
     compiled: bool = False
 
+    # The reference's kernel slots (models/cuda_funcs/kernel_manager.py:27-53), each naming the entry
+    # point of the library that does that kernel's work (the *_v2 dynamic-parallelism variants and the
+    # transposes, which nothing here needs, have none).
+    real_enc_fwd: Kernel = Kernel("cf_real_enc_fwd")
+    real_enc_bwd: Kernel = Kernel("cf_real_enc_bwd")
+    real_enc_proj_fwd: Kernel = Kernel("cf_real_enc_fwd")
+    real_enc_proj_bwd: Kernel = Kernel("cf_real_enc_bwd")
+    reci_enc_fwd: Kernel = Kernel("cf_reci_enc_fwd")
+    reci_enc_bwd: Kernel = Kernel("cf_reci_enc_bwd")
+    fused_dpa_fwd: Kernel = Kernel("cf_fused_dpa_fwd")
+    fused_dpa_fwd_v3: Kernel = Kernel("cf_fused_dpa_fwd")
+    fused_dpa_bwd: Kernel = Kernel("cf_fused_dpa_bwd")
+    fused_dpa_bwd_v3: Kernel = Kernel("cf_fused_dpa_bwd")
+    fused_dpa_bwd_q: Kernel = Kernel("cf_fused_dpa_bwd")
+    fused_dpa_bwd_q_v3: Kernel = Kernel("cf_fused_dpa_bwd")
+    irregular_mean_fwd: Kernel = Kernel("cf_irregular_mean_fwd")
+    minimum_distance: Kernel = Kernel("cf_minimum_distance")
+
+    @staticmethod
+    def get_kernel_names():
+        """Names of the kernel slots (models/cuda_funcs/kernel_manager.py:60-66)."""
+        return sorted(name for name, value in KernelManager.__dict__.items() if isinstance(value, Kernel))
+
+    @staticmethod
+    def get_kernel(name: str) -> "Kernel":
+        return KernelManager.__dict__[name]
+
+    @staticmethod
+    def set_kernel(name: str, kernel: "Kernel") -> None:
+        setattr(KernelManager, name, kernel)
+
 
 def compile_kernels(lattice_range: int, head_num: int, key_head_dim: int, value_pe_dim: int,
                     value_head_dim: int, set_minimum_range: bool) -> None:

@@ -308,3 +308,24 @@ def test_kernel_holder_resolves_library_entry_points():
     assert k() == k((1,), (64,), ()) == lib.load().cf_version()
     with pytest.raises(AttributeError):
         hip_funcs.Kernel("cf_no_such_entry_point")()
+
+
+def test_kernel_manager_slots_name_exported_entry_points():
+    """The reference's kernel slots and their accessors (models/cuda_funcs/kernel_manager.py:27-76):
+    every slot names a symbol that the header declares and the library exports."""
+    KM = hip_funcs.KernelManager
+    names = KM.get_kernel_names()
+    for wanted in ("real_enc_fwd", "real_enc_bwd", "real_enc_proj_fwd", "real_enc_proj_bwd", "reci_enc_fwd",
+                   "reci_enc_bwd", "fused_dpa_fwd", "fused_dpa_bwd", "fused_dpa_bwd_q", "irregular_mean_fwd",
+                   "minimum_distance"):
+        assert wanted in names
+    L = lib.load()
+    for name in names:
+        k = KM.get_kernel(name)
+        assert isinstance(k, hip_funcs.Kernel) and k.name in lib.SIGNATURES and hasattr(L, k.name), name
+    mine = hip_funcs.Kernel("cf_version")
+    KM.set_kernel("minimum_distance", mine)
+    try:
+        assert KM.get_kernel("minimum_distance") is mine
+    finally:
+        KM.set_kernel("minimum_distance", hip_funcs.Kernel("cf_minimum_distance"))
