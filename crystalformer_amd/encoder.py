@@ -26,6 +26,18 @@ from .hip_funcs import linear as linear_hip
 from .params import LatticeformerParams
 
 
+def get_edge_index(sizes, device) -> Tensor:
+    """(2,E) int64 edge list of all atom pairs inside each crystal, rows (i, j) of a crystal's
+    dense block in i-major order (models/indexed_latticeformer_encoder.py:15-32), built by the
+    device kernel instead of a host loop over crystals."""
+    if not torch.is_tensor(sizes):
+        sizes = torch.tensor(list(sizes), dtype=torch.int64)
+    sizes = sizes.to(device=device, dtype=torch.int64)
+    if sizes.numel() == 0 or int(sizes.sum()) == 0:
+        return torch.zeros((2, 0), dtype=torch.int64, device=device)
+    return ops.edge_index(sizes)[0]
+
+
 def det_3x3(m: Tensor) -> Tensor:
     """Cofactor expansion, term order of models/indexed_latticeformer_encoder.py:34-44."""
     return (m[:, 0, 0] * m[:, 1, 1] * m[:, 2, 2] + m[:, 0, 1] * m[:, 1, 2] * m[:, 2, 0]

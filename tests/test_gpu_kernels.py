@@ -563,6 +563,18 @@ def test_irregular_mean(dev, sizes, D):
     assert_close(gx, ref, "mean bwd")
 
 
+def test_get_edge_index_by_the_reference_name(dev):
+    """encoder.get_edge_index(sizes, device): the reference's host function
+    (models/indexed_latticeformer_encoder.py:15-32) served by the device kernel, from a list or a
+    tensor of sizes, crystals without atoms included."""
+    from crystalformer_amd.encoder import get_edge_index
+    for sizes in ([3, 1, 4], [2, 0, 5, 0], [7]):
+        ref = tp.get_edge_index(sizes)
+        assert torch.equal(get_edge_index(sizes, dev).cpu(), ref)
+        assert torch.equal(get_edge_index(torch.tensor(sizes), dev).cpu(), ref)
+    assert get_edge_index([], dev).shape == (2, 0) and get_edge_index([0, 0], dev).shape == (2, 0)
+
+
 @pytest.mark.parametrize("sizes", [[1], [3, 1, 4, 1, 5], [64, 1, 33], [200]])
 def test_edge_index_bit_exact(dev, sizes):
     b = make_sized_batch(sizes, seed=42)
