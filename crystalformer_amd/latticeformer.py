@@ -52,10 +52,14 @@ class Latticeformer(nn.Module):
         dropout = getattr(params, "dropout", 0.1)
         head_num = getattr(params, "head_num", 8)
         norm_type = getattr(params, "norm_type", "bn")
+        # Two options that cannot run in the reference either: its forward multiplies by an `atom_feat`
+        # table that no code creates (models/latticeformer.py:219-223), and its gradient scaler calls
+        # avr_pool with two arguments where the function takes three (models/latticeformer.py:23,
+        # models/pooling.py:19).  There is no behaviour to reproduce, so they are refused by name.
         if getattr(params, "use_cgcnn_feat", False):
-            raise NotImplementedError("use_cgcnn_feat")
+            raise NotImplementedError("use_cgcnn_feat: the reference defines no atom_feat table for it")
         if getattr(params, "scale_grad", 0.0) > 0:
-            raise NotImplementedError("scale_grad")
+            raise NotImplementedError("scale_grad: the reference's GradientScaler cannot run (avr_pool arity)")
 
         lattice_params = LatticeformerParams()
         lattice_params.parseFromArgs(params)
